@@ -1,0 +1,13 @@
+"""MI355X-native target-verify hot path of DFlash speculative decoding.
+
+Host-side mirror of the dflash-mlx operators on this path (same names, argument
+meaning and fallback behaviour), backed by hand-written gfx950 kernels in
+``libdflash_mi355.so`` (C ABI: include/dflash_mi355.h):
+
+* ``verify_matmul`` / ``verify_qmm`` - M=16 int4 affine quantized matmul;
+  ``VerifyQuantizedLinear`` / ``install_verify_linears`` - the module swap.
+* ``RecurrentRollbackCache`` / ``tape_replay_kernel`` - GatedDeltaNet tape-replay
+  rollback; ``RollbackArena`` - the same for all layers in one launch;
+  ``KVCache.trim`` - attention-cache trim.
+"""
+__version__ = "0.1.0"

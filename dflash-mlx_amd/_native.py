@@ -1,0 +1,89 @@
+"""ctypes binding of libdflash_mi355.so (the C ABI declared in include/dflash_mi355.h).
+
+There is no software fallback: if the library has not been built, or an entry
+point reports an error, the caller gets an exception.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
+
+ABI_VERSION = 1
+
+BF16, FP16, FP32 = 0, 1, 2
+QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
+
+# every symbol include/dflash_mi355.h declares
+EXPORTED_SYMBOLS = (
+    "dflash_abi_version",
+    "dflash_last_error",
+    "dflash_qmm_m16_workspace_bytes",
+    "dflash_qmm_m16",
+    "dflash_tape_replay",
+    "dflash_conv_state_rebuild",
+)
+
+
+class NativeLibraryError(RuntimeError):
+    """The HIP library is missing, mismatched, or one of its calls failed."""
+
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    c = ctypes
+    lib.dflash_abi_version.restype = c.c_int
+    lib.dflash_abi_version.argtypes = []
+    lib.dflash_last_error.restype = c.c_char_p
+    lib.dflash_last_error.argtypes = []
+    lib.dflash_qmm_m16_workspace_bytes.restype = c.c_size_t
+    lib.dflash_qmm_m16_workspace_bytes.argtypes = [c.c_int] * 5
+    lib.dflash_qmm_m16.restype = c.c_int
+    lib.dflash_qmm_m16.argtypes = (
+        [c.c_void_p] * 6 + [c.c_size_t] + [c.c_int] * 7 + [c.c_void_p]
+    )
+    lib.dflash_tape_replay.restype = c.c_int
+    lib.dflash_tape_replay.argtypes = (
+        [c.c_void_p] * 6 + [c.c_int] + [c.c_void_p] + [c.c_int] * 12 + [c.c_void_p]
+    )
+
+
+    lib.dflash_conv_state_rebuild.restype = c.c_int
+    lib.dflash_conv_state_rebuild.argtypes = [c.c_void_p] * 4 + [c.c_int] * 6 + [c.c_void_p]
+
+
+def lib() -> ctypes.CDLL:
+    """Load (once) and return the native library; raise if it is not there."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise NativeLibraryError(
+            f"{LIB_PATH} not found: build it with `python dflash-mlx_amd/build_ext.py` "
+            "(hipcc --offload-arch=gfx950); there is no fallback for the HIP path"
+        )
+    loaded = ctypes.CDLL(LIB_PATH)
+    for name in EXPORTED_SYMBOLS:
+        if not hasattr(loaded, name):
+            raise NativeLibraryError(f"{LIB_PATH} does not export {name}")
+    _declare(loaded)
+    got = loaded.dflash_abi_version()
+    if got != ABI_VERSION:
+        raise NativeLibraryError(f"ABI version {got} != expected {ABI_VERSION}; rebuild the library")
+    _lib = loaded
+    return loaded
+
+
+def is_built() -> bool:
+    return os.path.exists(LIB_PATH)
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = lib().dflash_last_error().decode("utf-8", "replace")
+        raise NativeLibraryError(f"{what} failed (code {rc}): {msg}")

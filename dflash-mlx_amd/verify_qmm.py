@@ -1,0 +1,136 @@
+"""M=16 int4 affine quantized matmul for the target-verify step (host side).
+
+Mirror of dflash_mlx/verify_qmm.py: the same call surface, env switches, gate
+and shape dispatch, with the device work done by the gfx950 kernel behind
+``dflash_qmm_m16`` (include/dflash_mi355.h) instead of a Metal kernel.
+
+    verify_matmul(x, w, scales, biases, *, transpose=True, group_size=64, bits=4)
+
+* ``DFLASH_VERIFY_QMM=1`` enables the kernel (verify_qmm.py:11-12); otherwise, and
+  for every call the gate rejects (verify_qmm.py:246-263) or whose shape fails a
+  divisibility guard (:300, :317), the stock ``quantized_matmul`` runs instead -
+  silently, as in the reference.
+* ``DFLASH_VERIFY_VARIANT`` in {auto, mma2big, mma2big_pipe} and
+  ``DFLASH_VERIFY_QMM_KPARTS`` select the variant (:15-22, 292-297).
+* An eligible call needs device tensors and the built HIP library; there is no
+  software fallback for it.
+"""
+from __future__ import annotations
+
+import os
+from typing import Dict, Tuple
+
+import torch
+
+from . import _native
+from .quantized import quantized_matmul
+
+_DTYPE_CODE = {torch.bfloat16: _native.BF16, torch.float16: _native.FP16}
+_VARIANT_CODE = {"mma2big": _native.QMM_MMA2BIG, "mma2big_pipe": _native.QMM_MMA2BIG_PIPE}
+
+
+def is_enabled() -> bool:
+    return os.environ.get("DFLASH_VERIFY_QMM", "") == "1"
+
+
+def _variant() -> str:
+    return os.environ.get("DFLASH_VERIFY_VARIANT", "auto")
+
+
+def _auto_variant(K: int, N: int) -> Tuple[str, int]:
+    if K >= 8192 or N <= 8192:
+        return ("mma2big_pipe", 8)
+    return ("mma2big", 1)
+
+
+def _should_use_verify(x: torch.Tensor, group_size: int, bits: int, transpose: bool) -> bool:
+    if not is_enabled():
+        return False
+    if bits != 4 or group_size not in (32, 64, 128):
+        return False
+    if x.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    if not transpose:
+        return False
+    m = 1
+    for d in x.shape[:-1]:
+        m *= d
+    return m == 16
+
+
+# One zero-initialised scratch buffer per (device, stream): calls on a stream are
+# ordered, so they can share it; the kernel hands it back zeroed where it has to be.
+_WORKSPACES: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    ws = _WORKSPACES.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 22), dtype=torch.uint8, device=device)
+        _WORKSPACES[key] = ws
+    return ws
+
+
+def _launch(x2: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
+            K: int, N: int, group_size: int, variant: str, k_parts: int) -> torch.Tensor:
+    if not x2.is_cuda:
+        raise _native.NativeLibraryError(
+            "verify_matmul: the M=16 kernel runs on the GPU only; got tensors on "
+            f"{x2.device} (unset DFLASH_VERIFY_QMM to use the stock operator)")
+    lib = _native.lib()
+    if scales.dtype not in _DTYPE_CODE or biases.dtype != scales.dtype:
+        raise TypeError(f"scales/biases must both be bf16 or fp16, got {scales.dtype}/{biases.dtype}")
+    y = torch.empty((16, N), dtype=x2.dtype, device=x2.device)
+    stream = torch.cuda.current_stream(x2.device).cuda_stream
+    vcode = _VARIANT_CODE[variant]
+    need = lib.dflash_qmm_m16_workspace_bytes(K, N, group_size, vcode, k_parts)
+    ws_ptr, ws_bytes = None, 0
+    if need:
+        ws = _workspace(x2.device, stream, need)
+        ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
+    rc = lib.dflash_qmm_m16(x2.data_ptr(), w.data_ptr(), scales.data_ptr(), biases.data_ptr(),
+                            y.data_ptr(), ws_ptr, ws_bytes, K, N, group_size,
+                            _DTYPE_CODE[x2.dtype], _DTYPE_CODE[scales.dtype], vcode, k_parts, stream)
+    _native.check(rc, "dflash_qmm_m16")
+    return y
+
+
+def verify_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
+                  *, transpose: bool = True, group_size: int = 64, bits: int = 4) -> torch.Tensor:
+    if not _should_use_verify(x, group_size, bits, transpose):
+        return quantized_matmul(x, w, scales, biases, transpose=transpose,
+                                group_size=group_size, bits=bits)
+
+    orig_shape = x.shape
+    x2 = x.reshape(16, orig_shape[-1]).contiguous()
+    w_q = w.contiguous()
+    scales = scales.contiguous()
+    biases = biases.contiguous()
+
+    K = int(x2.shape[-1])
+    N = int(w_q.shape[0])
+
+    variant = _variant()
+    auto_kp = None
+    if variant == "auto":
+        variant, auto_kp = _auto_variant(K, N)
+
+    K_PARTS = auto_kp if auto_kp is not None else int(os.environ.get("DFLASH_VERIFY_QMM_KPARTS", "4"))
+
+    if variant == "mma2big_pipe":
+        if N % 32 != 0 or K % (32 * K_PARTS) != 0:
+            return quantized_matmul(x, w, scales, biases, transpose=transpose,
+                                    group_size=group_size, bits=bits)
+        y = _launch(x2, w_q, scales, biases, K, N, group_size, "mma2big_pipe", K_PARTS)
+        return y.reshape(*orig_shape[:-1], N)
+
+    if N % 32 != 0 or K % 32 != 0:
+        return quantized_matmul(x, w, scales, biases, transpose=transpose,
+                                group_size=group_size, bits=bits)
+    y = _launch(x2, w_q, scales, biases, K, N, group_size, "mma2big", 1)
+    return y.reshape(*orig_shape[:-1], N)
+
+
+# the name the hot path is known by
+verify_qmm = verify_matmul

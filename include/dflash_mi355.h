@@ -1,0 +1,122 @@
+/*
+ * dflash_mi355.h - C ABI of libdflash_mi355.so, the MI355X (gfx950) device side of
+ * the dflash-mlx target-verify hot path.
+ *
+ * The reference reaches its device kernels through
+ *   mx.fast.metal_kernel(name, input_names, output_names, source)(inputs=..., grid=...,
+ *   threadgroup=..., output_shapes=..., output_dtypes=...)
+ * (dflash_mlx/verify_qmm.py:120-125, 306-313, 323-330; dflash_mlx/kernels.py:393-406).
+ * Each entry point below replaces one such launch site.  Conventions:
+ *   - every pointer is caller-owned DEVICE memory unless named *_host;
+ *   - kernels are enqueued on `stream` (a hipStream_t passed as void*; NULL = the
+ *     default stream) and the call returns without waiting;
+ *   - inputs are never written, outputs never alias inputs;
+ *   - no entry point allocates device memory: scratch comes in as `workspace`;
+ *   - return value 0 on success, a negative DFLASH_ERR_* otherwise (nothing is
+ *     thrown across the boundary); dflash_last_error() describes the last failure
+ *     on the calling thread.
+ */
+#ifndef DFLASH_MI355_H
+#define DFLASH_MI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DFLASH_ABI_VERSION 1
+
+enum {
+  DFLASH_OK = 0,
+  DFLASH_ERR_ARG = -1,       /* null pointer / unknown enum value            */
+  DFLASH_ERR_SHAPE = -2,     /* shape the kernels do not cover               */
+  DFLASH_ERR_WORKSPACE = -3, /* workspace missing or too small               */
+  DFLASH_ERR_HIP = -4        /* a HIP runtime call failed                    */
+};
+
+enum { DFLASH_BF16 = 0, DFLASH_FP16 = 1, DFLASH_FP32 = 2 };
+
+/* Shape dispatch of dflash_mlx/verify_qmm.py:19-22, 299-331. */
+enum { DFLASH_QMM_MMA2BIG = 0, DFLASH_QMM_MMA2BIG_PIPE = 1 };
+
+int dflash_abi_version(void);
+const char* dflash_last_error(void);
+
+/*
+ * M=16 int4 affine quantized matmul, y[16,N] = x[16,K] . (scale*q + bias)^T.
+ * Replaces the `verify_mma2big_*` launch (verify_qmm.py:323-330, variant
+ * DFLASH_QMM_MMA2BIG, k_parts ignored) and the `verify_mma2big_pipe_*` launch plus
+ * the host-side `partials.sum(axis=0).astype(T)` (verify_qmm.py:306-314, variant
+ * DFLASH_QMM_MMA2BIG_PIPE: K is cut into k_parts contiguous slices whose fp32
+ * partial products are summed in slice order and rounded once).
+ *
+ *   x        [16, K]            act_dtype (bf16 / fp16), row-major
+ *   w_q      [N, K/8]           uint32, element k of row n = (w_q[n][k>>3] >> 4*(k&7)) & 15
+ *   scales   [N, K/group_size]  sb_dtype (bf16 / fp16)
+ *   biases   [N, K/group_size]  sb_dtype
+ *   y        [16, N]            act_dtype
+ *   workspace                   >= dflash_qmm_m16_workspace_bytes(...) bytes, 256-byte
+ *                               aligned, ZERO-FILLED ONCE by the caller before its first
+ *                               use; the kernel leaves it zero-filled where it must be,
+ *                               so it can be reused by later calls on the same stream.
+ *                               Calls that share a workspace must not overlap in time.
+ * Requirements: group_size in {32,64,128}; N % 16 == 0; K % group_size == 0;
+ * for the pipe variant K % (32*k_parts) == 0.  Results are deterministic
+ * (bit-identical from run to run for identical inputs).
+ */
+size_t dflash_qmm_m16_workspace_bytes(int K, int N, int group_size, int variant, int k_parts);
+
+int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* scales, const void* biases,
+                   void* y, void* workspace, size_t workspace_bytes, int K, int N, int group_size,
+                   int act_dtype, int sb_dtype, int variant, int k_parts, void* stream);
+
+/*
+ * GatedDeltaNet tape replay: for every slot s and value head hv apply the first
+ * steps[s] recorded steps to the recurrent state,
+ *     S[dv][dk] <- g_t * S[dv][dk] + k_t[dk] * delta_t[dv],   t = 0 .. steps[s]-1,
+ * skipping steps whose mask byte is zero.  Replaces the `tape_replay{,_vec}{,_mask}`
+ * launch of dflash_mlx/kernels.py:393-406 (kernel body :244-293).  The reference
+ * slices the tape to the accepted length on the host (recurrent_rollback_cache.py:
+ * 160-167); here the full tape is passed and the accepted length is an argument, read
+ * from device memory when steps_dev is given so that it never has to visit the host.
+ *
+ *   tape      [slots, T, Hv, Dv]   tape_dtype (bf16 / fp16 / fp32)
+ *   k         [slots, T, Hk, Dk]   k_dtype    (bf16 / fp16 / fp32), Hv % Hk == 0
+ *   g         [slots, T, Hv] (g_per_dk = 0) or [slots, T, Hv, Dk] (g_per_dk = 1), g_dtype
+ *   state_in  [slots, Hv, Dv, Dk]  state_dtype (fp32 / bf16 / fp16), Dk contiguous
+ *   state_out same shape and dtype, must not alias state_in
+ *   steps_dev [slots] int32 device array, or NULL to use steps_host for every slot;
+ *             values are clamped to [0, T]
+ *   mask      [slots, T] uint8 or NULL
+ * exact_order != 0 forces the step-by-step evaluation order of the reference kernel
+ * (always used for bf16/fp16 states, which are rounded after every step,
+ * kernels.py:281-283); otherwise an fp32 state is updated through the algebraically
+ * equal form  S = (prod g) S0 + sum_t (prod_{u>t} g_u) delta_t (x) k_t.
+ * Requirements: Dk % 4 == 0, Dk <= 1024, T*(Dv + 2*Dk + 1)*4 bytes <= 64 KiB.
+ */
+int dflash_tape_replay(const void* tape, const void* k, const void* g, const void* state_in,
+                       void* state_out, const int32_t* steps_dev, int steps_host,
+                       const uint8_t* mask, int slots, int T, int Hk, int Hv, int Dk, int Dv,
+                       int state_dtype, int tape_dtype, int k_dtype, int g_dtype, int g_per_dk,
+                       int exact_order, void* stream);
+
+/*
+ * Conv-window rebuild of a GatedDeltaNet layer after a partial acceptance: output
+ * row j of a slot is row steps+j of concat([conv_prev, qkv], axis=rows).  Replaces the
+ * array ops of dflash_mlx/recurrent_rollback_cache.py:129-146 (zeros stand in for a
+ * missing conv_prev, :136-140).
+ *
+ *   conv_prev [slots, keep, C] or NULL    qkv [slots, T, C]    conv_out [slots, keep, C]
+ *   elements of elem_bytes bytes, copied verbatim; steps as in dflash_tape_replay,
+ *   clamped to [0, T]; keep = conv_kernel_size - 1.
+ */
+int dflash_conv_state_rebuild(const void* conv_prev, const void* qkv, void* conv_out,
+                              const int32_t* steps_dev, int steps_host, int slots, int T, int keep,
+                              int C, int elem_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DFLASH_MI355_H */

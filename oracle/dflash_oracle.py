@@ -1,0 +1,538 @@
+"""CPU restatement of the dflash-mlx target-verify hot path (TEST INFRASTRUCTURE).
+
+This module is a checker, not a product: only the test-suite, the smoke entry
+and the benchmark's ``cpu_baseline`` leg may import it.  The shipped package
+never routes a computation through it.
+
+Everything here is plain NumPy (pure-Python loops only in the ``*_bruteforce``
+helpers meant for tiny inputs).  Each function names the reference lines it
+restates (paths relative to the dflash-mlx tree).
+
+bf16 has no NumPy dtype; bf16 tensors travel as ``uint16`` bit patterns and the
+helpers ``bf16_to_f32`` / ``f32_to_bf16`` convert (round-to-nearest-even).
+
+Pinning status (what the test-suite checks each function against, none of it
+a re-typed formula):
+
+* qmm            - brute-force Python loop on tiny shapes, closed-form known
+                   answers (all-8 codes with bias=-8*scale -> 0, one-hot x,
+                   nibble-order probe), linearity / N-slice / K-split
+                   invariants, and ``torch`` dequant+matmul as an independent
+                   library route.
+* tape replay    - forward/replay consistency against the independent
+                   ``gated_delta_ops_with_tape`` restatement, closed forms
+                   (0 steps, delta==0, g==1 rank-1), unrolled fp64 sum.
+* conv rebuild,
+  KV trim,
+  acceptance     - exhaustive brute force over all small index patterns.
+* parity unpinned: bit-level rounding/accumulation order of MLX's own
+  ``mx.quantized_matmul`` on ``mx.cpu`` (third-party mlx >= 0.25, not present
+  in this build environment) - absorbed by the stated tolerance band; and the
+  gathered per-expert qmm, which has no counterpart in the reference.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+
+# ----------------------------------------------------------------------------
+# bf16 / fp16 helpers
+# ----------------------------------------------------------------------------
+
+
+def f32_to_bf16(a: np.ndarray) -> np.ndarray:
+    """float32 -> bf16 bit pattern (uint16), round-to-nearest-even, NaN kept."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    u = a.view(np.uint32).astype(np.uint64)
+    rounding = ((u >> 16) & 1) + 0x7FFF
+    r = ((u + rounding) >> 16).astype(np.uint16)
+    nan = np.isnan(a)
+    if nan.any():
+        r = np.where(nan, np.uint16(0x7FC0), r)
+    return r
+
+
+def bf16_to_f32(b: np.ndarray) -> np.ndarray:
+    """bf16 bit pattern (uint16) -> float32 (exact)."""
+    b = np.ascontiguousarray(b, dtype=np.uint16)
+    return (b.astype(np.uint32) << 16).view(np.float32)
+
+
+def round_bf16(a: np.ndarray) -> np.ndarray:
+    """Round float32 values to the nearest bf16, returned as float32."""
+    return bf16_to_f32(f32_to_bf16(a))
+
+
+def round_to(a: np.ndarray, dtype: str) -> np.ndarray:
+    """Round fp32 values through ``dtype`` in {'bf16','fp16','fp32'}; returns fp32."""
+    if dtype == "bf16":
+        return round_bf16(a)
+    if dtype == "fp16":
+        return np.asarray(a, dtype=np.float32).astype(np.float16).astype(np.float32)
+    if dtype == "fp32":
+        return np.asarray(a, dtype=np.float32)
+    raise ValueError(f"unknown dtype {dtype}")
+
+
+# ----------------------------------------------------------------------------
+# int4 affine format (MLX): 8 codes per uint32, low nibble first
+# ----------------------------------------------------------------------------
+
+
+def unpack_int4(w_packed: np.ndarray) -> np.ndarray:
+    """[N, K/8] uint32 -> [N, K] uint8 codes.
+
+    Element k of a row sits in word k>>3 at bit 4*(k&7) (verify_qmm.py:70-75:
+    ``nib = (packed >> (ki*4)) & 0xF`` written to k = k_base + ki).
+    """
+    w = np.ascontiguousarray(w_packed).view(np.uint32)
+    shifts = (4 * np.arange(8, dtype=np.uint32))[None, None, :]
+    codes = (w[:, :, None] >> shifts) & np.uint32(0xF)
+    return codes.reshape(w.shape[0], w.shape[1] * 8).astype(np.uint8)
+
+
+def pack_int4(codes: np.ndarray) -> np.ndarray:
+    """[N, K] codes in 0..15 -> [N, K/8] uint32, low nibble first (inverse of unpack)."""
+    codes = np.asarray(codes).astype(np.uint32)
+    n, k = codes.shape
+    assert k % 8 == 0
+    c = codes.reshape(n, k // 8, 8)
+    shifts = (4 * np.arange(8, dtype=np.uint32))[None, None, :]
+    return (c << shifts).sum(axis=2, dtype=np.uint64).astype(np.uint32)
+
+
+def dequant_affine(
+    w_packed: np.ndarray,
+    scales_f32: np.ndarray,
+    biases_f32: np.ndarray,
+    group_size: int,
+    *,
+    round_dtype: Optional[str] = None,
+    out_dtype=np.float64,
+) -> np.ndarray:
+    """w~[n,k] = q[n,k]*s[n,k//gs] + b[n,k//gs].
+
+    ``round_dtype`` in {'bf16','fp16'} reproduces the reference kernel's
+    per-weight rounding ``T(float(nib) * s + b)`` (verify_qmm.py:75); ``None``
+    keeps the exact affine value.
+    """
+    q = unpack_int4(w_packed)
+    n, k = q.shape
+    g = k // group_size
+    assert scales_f32.shape == (n, g) and biases_f32.shape == (n, g)
+    if round_dtype is None:
+        s = np.repeat(scales_f32.astype(np.float64), group_size, axis=1)
+        b = np.repeat(biases_f32.astype(np.float64), group_size, axis=1)
+        return (q.astype(np.float64) * s + b).astype(out_dtype)
+    s = np.repeat(scales_f32.astype(np.float32), group_size, axis=1)
+    b = np.repeat(biases_f32.astype(np.float32), group_size, axis=1)
+    w = q.astype(np.float32) * s + b  # fp32 multiply then add
+    return round_to(w, round_dtype).astype(out_dtype)
+
+
+def qmm_exact(
+    x_f32: np.ndarray,
+    w_packed: np.ndarray,
+    scales_f32: np.ndarray,
+    biases_f32: np.ndarray,
+    group_size: int = 64,
+    *,
+    n_chunk: int = 2048,
+) -> np.ndarray:
+    """y = x . (s*q + b)^T in float64 with no intermediate rounding.
+
+    The closed form the north-star states; ``x_f32`` holds the already
+    bf16/fp16-rounded activations as fp32.  Returns float64 [M, N].
+    """
+    x = np.asarray(x_f32, dtype=np.float64)
+    n = w_packed.shape[0]
+    out = np.empty((x.shape[0], n), dtype=np.float64)
+    for n0 in range(0, n, n_chunk):
+        n1 = min(n, n0 + n_chunk)
+        w = dequant_affine(w_packed[n0:n1], scales_f32[n0:n1], biases_f32[n0:n1], group_size)
+        out[:, n0:n1] = x @ w.T
+    return out
+
+
+def qmm_kernel_semantics(
+    x_f32: np.ndarray,
+    w_packed: np.ndarray,
+    scales_f32: np.ndarray,
+    biases_f32: np.ndarray,
+    group_size: int = 64,
+    *,
+    dtype: str = "bf16",
+    k_parts: int = 1,
+    n_chunk: int = 2048,
+) -> np.ndarray:
+    """The reference Metal kernels' arithmetic (verify_qmm.py:66-116, 154-156, 226-230, 314).
+
+    Weights are dequantised with per-weight rounding to T, products are
+    accumulated in fp32 (K split into ``k_parts`` contiguous slices whose fp32
+    partials are summed, then one rounding to T).  Accumulation order inside a
+    slice is not reproduced (fp32 matmul), which is below tolerance.
+    Returns fp32 values already rounded to ``dtype``.
+    """
+    x = np.asarray(x_f32, dtype=np.float32)
+    m, k = x.shape
+    n = w_packed.shape[0]
+    assert k % k_parts == 0
+    ks = k // k_parts
+    acc = np.zeros((m, n), dtype=np.float32)
+    for n0 in range(0, n, n_chunk):
+        n1 = min(n, n0 + n_chunk)
+        w = dequant_affine(
+            w_packed[n0:n1], scales_f32[n0:n1], biases_f32[n0:n1], group_size,
+            round_dtype=dtype, out_dtype=np.float32,
+        )
+        part = np.zeros((m, n1 - n0), dtype=np.float32)
+        for p in range(k_parts):
+            part += x[:, p * ks:(p + 1) * ks] @ w[:, p * ks:(p + 1) * ks].T
+        acc[:, n0:n1] = part
+    return round_to(acc, dtype)
+
+
+def qmm_bruteforce(x_f32, w_packed, scales_f32, biases_f32, group_size):
+    """Pure-Python triple loop over the closed form (tiny shapes only)."""
+    m, k = x_f32.shape
+    n = w_packed.shape[0]
+    out = [[0.0] * n for _ in range(m)]
+    wp = np.ascontiguousarray(w_packed).view(np.uint32)
+    for mi in range(m):
+        for ni in range(n):
+            acc = 0.0
+            for ki in range(k):
+                word = int(wp[ni, ki >> 3])
+                q = (word >> (4 * (ki & 7))) & 0xF
+                g = ki // group_size
+                acc += float(x_f32[mi, ki]) * (float(scales_f32[ni, g]) * q + float(biases_f32[ni, g]))
+            out[mi][ni] = acc
+    return np.array(out, dtype=np.float64)
+
+
+def qmm_gather_exact(x_f32, expert_ids, w_packed_e, scales_e, biases_e, group_size=64):
+    """Per-row expert selection: y[p] = x[p] . deq(W[expert_ids[p]])^T (float64).
+
+    No counterpart in the reference (its MoE experts go through mlx_lm's
+    third-party gather op); closed form only - parity unpinned.
+    """
+    p = x_f32.shape[0]
+    n = w_packed_e.shape[1]
+    out = np.empty((p, n), dtype=np.float64)
+    for i in range(p):
+        e = int(expert_ids[i])
+        out[i] = qmm_exact(x_f32[i:i + 1], w_packed_e[e], scales_e[e], biases_e[e], group_size)[0]
+    return out
+
+
+# ----------------------------------------------------------------------------
+# verify_qmm host logic
+# ----------------------------------------------------------------------------
+
+
+def should_use_verify(flag_value: str, x_shape: Sequence[int], x_dtype: str,
+                      group_size: int, bits: int, transpose: bool) -> bool:
+    """verify_qmm.py:246-263 with the env flag passed in explicitly."""
+    if flag_value != "1":
+        return False
+    if bits != 4 or group_size not in (32, 64, 128):
+        return False
+    if x_dtype not in ("bf16", "fp16"):
+        return False
+    if not transpose:
+        return False
+    m = 1
+    for d in x_shape[:-1]:
+        m *= d
+    return m == 16
+
+
+def auto_variant(K: int, N: int) -> Tuple[str, int]:
+    """verify_qmm.py:19-22."""
+    if K >= 8192 or N <= 8192:
+        return ("mma2big_pipe", 8)
+    return ("mma2big", 1)
+
+
+def dispatch_variant(K: int, N: int, variant_env: str = "auto", kparts_env: str = "4"):
+    """verify_qmm.py:292-321: returns (variant, k_parts) or ('stock', 0) on a failed guard."""
+    variant = variant_env
+    auto_kp = None
+    if variant == "auto":
+        variant, auto_kp = auto_variant(K, N)
+    k_parts = auto_kp if auto_kp is not None else int(kparts_env)
+    if variant == "mma2big_pipe":
+        if N % 32 != 0 or K % (32 * k_parts) != 0:
+            return ("stock", 0)
+        return ("mma2big_pipe", k_parts)
+    if N % 32 != 0 or K % 32 != 0:
+        return ("stock", 0)
+    return ("mma2big", 1)
+
+
+def verify_enabled_for(config: dict, override: str = "") -> bool:
+    """runtime.py:725-753 with the env override passed in explicitly."""
+    override = override.strip()
+    if override == "1":
+        return True
+    if override == "0":
+        return False
+    try:
+        text_cfg = config.get("text_config", config) if isinstance(config, dict) else config
+        num_experts = int(text_cfg.get("num_experts", 0) or 0)
+        num_layers = int(text_cfg.get("num_hidden_layers", 0) or 0)
+    except Exception:
+        return False
+    if num_experts > 0:
+        return True
+    return num_layers >= 40
+
+
+# ----------------------------------------------------------------------------
+# GatedDeltaNet forward-with-tape and tape replay
+# ----------------------------------------------------------------------------
+
+
+def _decay(g: np.ndarray, t: int) -> np.ndarray:
+    if g.ndim == 4:
+        return g[:, t, :, None, :]
+    if g.ndim == 3:
+        return g[:, t, :, None, None]
+    raise ValueError(f"Unsupported gating shape {g.shape}")
+
+
+def gated_delta_ops_with_tape(q, k, v, g, beta, state, mask=None, dtype=np.float64):
+    """kernels.py:131-173 in NumPy.  q,k [B,T,Hk,Dk]; v [B,T,Hv,Dv]; g [B,T,Hv] or
+    [B,T,Hv,Dk]; beta [B,T,Hv]; state [B,Hv,Dv,Dk].  Returns (y, state, tape)."""
+    q = np.asarray(q, dtype=dtype)
+    k = np.asarray(k, dtype=dtype)
+    v = np.asarray(v, dtype=dtype)
+    g = np.asarray(g, dtype=dtype)
+    beta = np.asarray(beta, dtype=dtype)
+    state = np.asarray(state, dtype=dtype)
+    B, T, Hk, Dk = k.shape
+    Hv, Dv = v.shape[2:]
+    if Hv % Hk != 0:
+        raise ValueError(f"Cannot align K heads {Hk} to V heads {Hv}")
+    rf = Hv // Hk
+    if rf > 1:
+        q = np.repeat(q, rf, axis=2)
+        k = np.repeat(k, rf, axis=2)
+    ys, tape = [], []
+    for t in range(T):
+        old = state
+        decayed = state * _decay(g, t)
+        kv_mem = (decayed * k[:, t, :, None, :]).sum(axis=-1)
+        delta = (v[:, t] - kv_mem) * beta[:, t, :, None]
+        new = decayed + k[:, t, :, None, :] * delta[..., None]
+        y = (new * q[:, t, :, None, :]).sum(axis=-1)
+        if mask is not None:
+            sm = np.asarray(mask)[:, t].astype(bool)
+            new = np.where(sm[:, None, None, None], new, old)
+            delta = np.where(sm[:, None, None], delta, 0.0)
+            y = np.where(sm[:, None, None], y, 0.0)
+        state = new
+        ys.append(y)
+        tape.append(delta)
+    return np.stack(ys, axis=1), state, np.stack(tape, axis=1)
+
+
+def tape_replay_ops(tape, k, g, state, mask=None, dtype=np.float64):
+    """kernels.py:328-358 in NumPy (array-op replay; no per-step rounding).
+
+    tape [B,T,Hv,Dv]; k [B,T,Hk,Dk]; g [B,T,Hv] or [B,T,Hv,Dk]; state [B,Hv,Dv,Dk].
+    """
+    tape = np.asarray(tape, dtype=dtype)
+    k = np.asarray(k, dtype=dtype)
+    g = np.asarray(g, dtype=dtype)
+    state = np.asarray(state, dtype=dtype)
+    hk = k.shape[2]
+    hv = tape.shape[2]
+    if hv % hk != 0:
+        raise ValueError(f"Cannot align K heads {hk} to tape heads {hv}")
+    rf = hv // hk
+    if rf > 1:
+        k = np.repeat(k, rf, axis=2)
+    for t in range(int(tape.shape[1])):
+        prev = state
+        decay = _decay(g, t)
+        delta = tape[:, t, :, :, None]
+        k_t = k[:, t, :, None, :]
+        state = state * decay
+        state = state + delta * k_t
+        if mask is not None:
+            sm = np.asarray(mask)[:, t].astype(bool)[:, None, None, None]
+            state = np.where(sm, state, prev)
+    return state
+
+
+def tape_replay_kernel_semantics(tape, k, g, state, mask=None, state_dtype: str = "fp32"):
+    """kernels.py:244-293: fp32 registers, ``s = s*g; s = s + k*delta`` and a
+    round-trip through the state dtype after every (unmasked) step."""
+    tape = np.asarray(tape, dtype=np.float32)
+    k = np.asarray(k, dtype=np.float32)
+    g = np.asarray(g, dtype=np.float32)
+    s = np.asarray(state, dtype=np.float32).copy()
+    B, T, Hv, Dv = tape.shape
+    Hk = k.shape[2]
+    if Hv % Hk != 0:
+        raise ValueError(f"Cannot align K heads {Hk} to tape heads {Hv}")
+    rf = Hv // Hk
+    for b in range(B):
+        for t in range(T):
+            if mask is not None and not bool(np.asarray(mask)[b, t]):
+                continue
+            for hv in range(Hv):
+                hk = hv // rf
+                gt = g[b, t, hv] if g.ndim == 3 else g[b, t, hv][None, :]
+                sv = s[b, hv] * gt
+                sv = sv + k[b, t, hk][None, :] * tape[b, t, hv][:, None]
+                s[b, hv] = round_to(sv.astype(np.float32), state_dtype)
+    return round_to(s, state_dtype)
+
+
+def tape_replay_unrolled(tape, k, g, state, steps: int):
+    """Closed form S_a = (prod g) S0 + sum_t (prod_{u>t} g_u) delta_t (x) k_t, float64,
+    scalar-per-head gate only.  Independent of the step-by-step routines."""
+    tape = np.asarray(tape, dtype=np.float64)
+    k = np.asarray(k, dtype=np.float64)
+    g = np.asarray(g, dtype=np.float64)
+    S0 = np.asarray(state, dtype=np.float64)
+    B, T, Hv, Dv = tape.shape
+    Hk = k.shape[2]
+    rf = Hv // Hk
+    out = np.empty_like(S0)
+    for b in range(B):
+        for hv in range(Hv):
+            hk = hv // rf
+            G = np.prod(g[b, :steps, hv])
+            acc = G * S0[b, hv]
+            for t in range(steps):
+                c = np.prod(g[b, t + 1:steps, hv])
+                acc = acc + c * np.outer(tape[b, t, hv], k[b, t, hk])
+            out[b, hv] = acc
+    return out
+
+
+# ----------------------------------------------------------------------------
+# Rollback cache: conv-state rebuild, state machine, KV trim, acceptance
+# ----------------------------------------------------------------------------
+
+
+def rebuild_conv_state(snapshot_conv, qkv_tape, accepted_steps: int, conv_kernel_size: int = 4):
+    """recurrent_rollback_cache.py:129-146.  snapshot_conv [B,keep,C] or None;
+    qkv_tape [B,T,C]."""
+    keep = conv_kernel_size - 1
+    if keep <= 0:
+        return None
+    if snapshot_conv is None:
+        prefix = np.zeros((qkv_tape.shape[0], keep, qkv_tape.shape[-1]), dtype=qkv_tape.dtype)
+    else:
+        prefix = snapshot_conv
+    conv_input = np.concatenate([prefix, qkv_tape], axis=1)
+    start = accepted_steps
+    end = min(start + keep, int(conv_input.shape[1]))
+    return np.ascontiguousarray(conv_input[:, start:end, :])
+
+
+def match_acceptance_length(drafted: Sequence[int], posterior: Sequence[int]) -> int:
+    """runtime.py:101-108: sum(cumprod(drafted == posterior)); 0 for empty input."""
+    drafted = np.asarray(drafted)
+    posterior = np.asarray(posterior)
+    if drafted.shape[0] == 0:
+        return 0
+    matches = (drafted == posterior).astype(np.int32)
+    return int(np.sum(np.cumprod(matches)))
+
+
+def match_acceptance_length_loop(drafted, posterior) -> int:
+    """Plain loop: length of the longest matching prefix."""
+    n = 0
+    for a, b in zip(list(drafted), list(posterior)):
+        if int(a) != int(b):
+            break
+        n += 1
+    return n
+
+
+def kv_trim(offset: int, n: int) -> Tuple[int, int]:
+    """mlx_lm KVCache.trim as used at runtime.py:899: n=min(offset,n); offset-=n.
+    Returns (new_offset, trimmed)."""
+    n = min(int(offset), int(n))
+    return int(offset) - n, n
+
+
+def commit_cycle(start: int, verify_ids: Sequence[int], posterior: Sequence[int]):
+    """runtime.py:1381-1383, 1398-1403, 1433: one cycle's index arithmetic.
+
+    Returns dict(acceptance_len, commit_count, committed, staged_next, new_start)."""
+    verify_ids = list(int(v) for v in verify_ids)
+    posterior = list(int(v) for v in posterior)
+    acc = match_acceptance_length(verify_ids[1:], posterior[:-1])
+    commit = 1 + acc
+    return dict(
+        acceptance_len=acc,
+        commit_count=commit,
+        committed=verify_ids[:commit],
+        staged_next=posterior[acc],
+        new_start=start + commit,
+    )
+
+
+def restore_plan(layer_kinds: Sequence[str], offsets: Sequence[int], *, target_len: int,
+                 acceptance_length: int, drafted_tokens: int = 0) -> List[tuple]:
+    """runtime.py:878-907 as a pure plan: per layer what the engine does.
+
+    ``layer_kinds[i]`` is 'gdn' (has rollback) or 'kv' (has trim); returns a list of
+    ('clear',) / ('rollback', n_accepted) / ('trim', n) / ('none',) per layer."""
+    fully = drafted_tokens > 0 and acceptance_length == drafted_tokens
+    plan = []
+    for kind, off in zip(layer_kinds, offsets):
+        if kind == "gdn":
+            plan.append(("clear",) if fully else ("rollback", int(acceptance_length)))
+        elif kind == "kv":
+            off = int(off or 0)
+            plan.append(("trim", off - target_len) if off > target_len else ("none",))
+        else:
+            raise ValueError(kind)
+    return plan
+
+
+class RollbackCacheModel:
+    """recurrent_rollback_cache.py:96-171 as a NumPy state machine."""
+
+    def __init__(self, conv_kernel_size: int = 4):
+        self.cache = [None, None]
+        self.conv_kernel_size = conv_kernel_size
+        self.clear_transients()
+
+    def clear_transients(self):
+        self._armed = False
+        self._tape = self._tape_k = self._tape_g = self._tape_qkv = None
+        self._snapshot = None
+
+    def arm_rollback(self, prefix_len: int = 0):
+        self._armed = True
+        self._tape = self._tape_k = self._tape_g = self._tape_qkv = None
+        self._snapshot = list(self.cache)
+
+    def record_tape(self, *, tape, k, g, qkv):
+        self._tape, self._tape_k, self._tape_g, self._tape_qkv = tape, k, g, qkv
+
+    def rollback(self, n_accepted: int):
+        if self._snapshot is None:
+            self.clear_transients()
+            return
+        self.cache = list(self._snapshot)
+        if (self._tape is not None and self._tape_k is not None
+                and self._tape_g is not None and self.cache[1] is not None):
+            steps = int(n_accepted) + 1
+            self.cache[1] = tape_replay_ops(
+                self._tape[:, :steps], self._tape_k[:, :steps], self._tape_g[:, :steps], self.cache[1])
+            if self._tape_qkv is None:
+                pass
+            else:
+                self.cache[0] = rebuild_conv_state(
+                    self._snapshot[0], self._tape_qkv, steps, self.conv_kernel_size)
+        self.clear_transients()

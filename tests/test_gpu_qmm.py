@@ -1,0 +1,241 @@
+"""Parity of the gfx950 M=16 int4 qmm against the CPU oracle (exact fp64 closed form
+and the reference-kernel arithmetic), through the Python surface and the raw C ABI.
+
+Tolerances:
+  north-star bar   max|y - y_exact| <= 2e-2 * max|row|   and   rel-L2 <= 5e-3   (bf16)
+  reference's own  max_abs <= 8e-3 (bf16) / 4e-3 (fp16), max_abs/(max|y_ref|+1e-3) <= 2e-2
+                   on x, w ~ N(0,1)/sqrt(K)   (tests/test_verify_qmm_parity.py:83-109)
+"""
+import numpy as np
+import pytest
+import torch
+
+import dflash_mlx_amd._native as nat
+from dflash_mlx_amd import verify_qmm as VQ
+from dflash_mlx_amd.quantized import QuantizedLinear, quantize, quantized_matmul
+from dflash_mlx_amd.verify_linear import VerifyQuantizedLinear
+from dflash_mlx_amd.workloads import make_qmm_case, seed_for
+from oracle import dflash_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _bits(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _f32(t):
+    return t.detach().cpu().float().numpy()
+
+
+def _oracle_exact(c_oracle, case):
+    assert case.x.dtype == torch.bfloat16
+    y32, _ = c_oracle.qmm_m16(_bits(case.x), case.w.cpu().numpy().view(np.uint32), _bits(case.scales),
+                              _bits(case.biases), case.group_size, flavour=0)
+    return y32.astype(np.float64)
+
+
+def _check_north_star(y, exact):
+    err = np.abs(y - exact)
+    row_inf = np.max(np.abs(exact), axis=1, keepdims=True)
+    assert np.all(err <= 2e-2 * row_inf + 1e-30), f"max-abs ratio {np.max(err / row_inf):.3g}"
+    rel = np.linalg.norm(y - exact) / max(np.linalg.norm(exact), 1e-30)
+    assert rel <= 5e-3, f"rel-L2 {rel:.3g}"
+    return rel
+
+
+def _run(case, variant=None, k_parts=None, monkeypatch=None):
+    d = case.to(DEV)
+    y = VQ.verify_matmul(d.x, d.w, d.scales, d.biases, group_size=d.group_size, bits=4)
+    torch.cuda.synchronize()
+    return y
+
+
+def test_config0_single_call(verify_env, native_lib, c_oracle):
+    """BASELINE config[0]: 16x4096x4096, group 64 (auto dispatch -> pipe x8)."""
+    case = make_qmm_case(4096, 4096, seed_for(0))
+    y = _f32(_run(case)).astype(np.float64)
+    exact = _oracle_exact(c_oracle, case)
+    rel = _check_north_star(y, exact)
+    # the kernel keeps exact affine weights, so it sits at the bf16 output-rounding floor
+    assert rel < 2.5e-3
+    assert np.max(np.abs(y - O.round_bf16(exact.astype(np.float32)))) <= 2 ** -7 * np.max(np.abs(exact))
+
+
+@pytest.mark.parametrize("K,N", [(5120, 17408), (17408, 5120), (5120, 7168), (4096, 12288)])
+def test_real_projection_shapes(verify_env, native_lib, c_oracle, K, N):
+    """27B / 9B projection shapes at full size, both dispatch branches."""
+    case = make_qmm_case(K, N, seed_for(3, K % 97))
+    y = _f32(_run(case)).astype(np.float64)
+    _check_north_star(y, _oracle_exact(c_oracle, case))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("K,N", [(5120, 17408), (17408, 5120)])
+def test_reference_tolerances_on_reference_style_data(verify_env, native_lib, dtype, K, N):
+    """The reference's own acceptance test: data ~ N(0,1)/sqrt(K) quantised from floats,
+    compared with the stock operator (here: the oracle's reference-kernel arithmetic)."""
+    g = torch.Generator().manual_seed(K + N)
+    scale = 1.0 / np.sqrt(K)
+    x = (torch.randn(16, K, generator=g) * scale).to(dtype)
+    w_fp = (torch.randn(N, K, generator=g) * scale).to(dtype)
+    wq, s, b = quantize(w_fp, 64, 4)
+    y = VQ.verify_matmul(x.to(DEV), wq.to(DEV), s.to(DEV), b.to(DEV), group_size=64, bits=4)
+    name = "bf16" if dtype == torch.bfloat16 else "fp16"
+    ref = O.qmm_kernel_semantics(x.float().numpy(), wq.numpy().view(np.uint32), s.float().numpy(),
+                                 b.float().numpy(), 64, dtype=name,
+                                 k_parts=8 if VQ._auto_variant(K, N)[0] == "mma2big_pipe" else 1)
+    yv = _f32(y)
+    max_abs = float(np.max(np.abs(yv - ref)))
+    max_rel = max_abs / (float(np.max(np.abs(ref))) + 1e-3)
+    assert max_abs <= (8e-3 if dtype == torch.bfloat16 else 4e-3), max_abs
+    assert max_rel <= 2e-2, max_rel
+
+
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("variant,kp", [("mma2big", 1), ("mma2big_pipe", 1), ("mma2big_pipe", 2),
+                                        ("mma2big_pipe", 4), ("mma2big_pipe", 8)])
+def test_group_sizes_and_variants(verify_env, native_lib, c_oracle, gs, variant, kp):
+    verify_env.setenv("DFLASH_VERIFY_VARIANT", variant)
+    verify_env.setenv("DFLASH_VERIFY_QMM_KPARTS", str(kp))
+    for K, N in [(1024, 96), (256, 32), (2304, 160)]:
+        case = make_qmm_case(K, N, 100 + gs + kp, group_size=gs)
+        y = _f32(_run(case)).astype(np.float64)
+        _check_north_star(y, _oracle_exact(c_oracle, case))
+
+
+def test_fp16_activations_and_scales(verify_env, native_lib):
+    for sdt in (torch.float16, torch.bfloat16):
+        case = make_qmm_case(1024, 128, 7, dtype=torch.float16)
+        case.scales = case.scales.to(sdt)
+        case.biases = (-8.0 * case.scales.float()).to(sdt)
+        y = _f32(_run(case)).astype(np.float64)
+        exact = O.qmm_exact(case.x.float().numpy(), case.w.numpy().view(np.uint32),
+                            case.scales.float().numpy(), case.biases.float().numpy(), 64)
+        err = np.abs(y - exact)
+        assert np.all(err <= 2e-3 * np.max(np.abs(exact), axis=1, keepdims=True))
+        assert np.linalg.norm(y - exact) / np.linalg.norm(exact) <= 1e-3
+
+
+def test_known_answers_on_device(verify_env, native_lib):
+    K, N, gs = 512, 64, 64
+    case = make_qmm_case(K, N, 11)
+    # (1) all codes 8 with bias = -8*scale: every weight is zero
+    zero = make_qmm_case(K, N, 11)
+    zero.w = torch.full_like(zero.w, 0x88888888 - 2 ** 32)
+    y = _f32(_run(zero))
+    bound = 1e-5 * float(case.scales.float().max()) * float(case.x.float().abs().sum(dim=1).max())
+    assert np.max(np.abs(y)) <= bound
+    # (2) one-hot rows read single weights: y[m, n] == bf16(s*q + b) exactly
+    ks = torch.randint(0, K, (16,), generator=torch.Generator().manual_seed(5))
+    hot = make_qmm_case(K, N, 11)
+    hot.x = torch.zeros_like(hot.x)
+    hot.x[torch.arange(16), ks] = 1.0
+    y = _f32(_run(hot))
+    wd = O.dequant_affine(hot.w.numpy().view(np.uint32), hot.scales.float().numpy(), hot.biases.float().numpy(), gs)
+    want = O.round_bf16(wd[:, ks.numpy()].T.astype(np.float32))
+    assert np.array_equal(y, want)
+    # (3) nibble order: codes 0..7 in every word, s=1, b=0, x = e_k  ->  y = k % 8
+    seq = make_qmm_case(K, N, 11)
+    seq.w = torch.full_like(seq.w, 0x76543210)
+    seq.scales = torch.ones_like(seq.scales)
+    seq.biases = torch.zeros_like(seq.biases)
+    seq.x = hot.x
+    y = _f32(_run(seq))
+    assert np.array_equal(y, np.repeat((ks.numpy() % 8)[:, None], N, axis=1).astype(np.float32))
+
+
+def test_deterministic_and_workspace_reuse(verify_env, native_lib, c_oracle):
+    a = make_qmm_case(4096, 4096, 21).to(DEV)
+    b = make_qmm_case(1024, 512, 22).to(DEV)
+    ya = [VQ.verify_matmul(a.x, a.w, a.scales, a.biases) for _ in range(3)]
+    yb = VQ.verify_matmul(b.x, b.w, b.scales, b.biases)
+    ya.append(VQ.verify_matmul(a.x, a.w, a.scales, a.biases))
+    torch.cuda.synchronize()
+    for y in ya[1:]:
+        assert torch.equal(y, ya[0])
+    _check_north_star(_f32(yb).astype(np.float64), _oracle_exact(c_oracle, b.to("cpu")))
+
+
+def test_n_tiles_are_independent_full_size(verify_env, native_lib):
+    """Size-independent property at a full 27B shape: any N-slice of W gives the same
+    bits as the matching slice of the full product."""
+    case = make_qmm_case(5120, 17408, 31).to(DEV)
+    full = VQ.verify_matmul(case.x, case.w, case.scales, case.biases)
+    for n0, n1 in [(0, 32), (4096, 4096 + 512), (17408 - 64, 17408)]:
+        part = VQ.verify_matmul(case.x, case.w[n0:n1], case.scales[n0:n1], case.biases[n0:n1])
+        assert torch.equal(part, full[:, n0:n1])
+
+
+def test_linearity_full_size(verify_env, native_lib):
+    case = make_qmm_case(17408, 5120, 32).to(DEV)
+    x2 = torch.randn_like(case.x.float()).to(torch.bfloat16)
+    # 2*x and x+x2 are formed in bf16 so that every operand is exactly representable
+    xs = (case.x.float() + x2.float()).to(torch.bfloat16)
+    exact_sum = xs.float() - case.x.float() - x2.float()
+    y1 = VQ.verify_matmul(case.x, case.w, case.scales, case.biases).float()
+    y2 = VQ.verify_matmul(x2, case.w, case.scales, case.biases).float()
+    ys = VQ.verify_matmul(xs, case.w, case.scales, case.biases).float()
+    yr = VQ.verify_matmul(exact_sum.to(torch.bfloat16), case.w, case.scales, case.biases).float()
+    resid = (ys - y1 - y2 - yr).abs().max().item()
+    assert resid <= 4 * 2 ** -8 * max(y1.abs().max().item(), y2.abs().max().item())
+
+
+def test_leading_shapes_and_stock_fallbacks_on_device(verify_env, native_lib):
+    case = make_qmm_case(512, 64, 41).to(DEV)
+    y = VQ.verify_matmul(case.x, case.w, case.scales, case.biases)
+    for shape in [(1, 16, 512), (4, 4, 512), (2, 2, 4, 512)]:
+        yr = VQ.verify_matmul(case.x.reshape(shape), case.w, case.scales, case.biases)
+        assert yr.shape == (*shape[:-1], 64) and torch.equal(yr.reshape(16, 64), y)
+    # M != 16 and fp32 activations use the stock operator
+    x8 = case.x[:8]
+    assert torch.equal(VQ.verify_matmul(x8, case.w, case.scales, case.biases),
+                       quantized_matmul(x8, case.w, case.scales, case.biases))
+    xf = case.x.float()
+    assert torch.equal(VQ.verify_matmul(xf, case.w, case.scales, case.biases),
+                       quantized_matmul(xf, case.w, case.scales, case.biases))
+    verify_env.setenv("DFLASH_VERIFY_QMM", "0")
+    assert torch.equal(VQ.verify_matmul(case.x, case.w, case.scales, case.biases),
+                       quantized_matmul(case.x, case.w, case.scales, case.biases))
+
+
+def test_verify_linear_on_device(verify_env, native_lib):
+    """tests/test_verify_linear_parity.py:50-72 - M != 16 identical to stock, M == 16
+    identical to a direct verify_matmul call."""
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(512, 1024, bias=False)
+    with torch.no_grad():
+        lin.weight.mul_(0.1 / lin.weight.std())
+    ql = QuantizedLinear.from_linear(lin.to(torch.bfloat16), 64, 4).to(DEV)
+    v = VerifyQuantizedLinear.from_quantized(ql)
+    for M in (1, 8, 32):
+        x = (torch.randn(M, 512, device=DEV) * 0.5).to(torch.bfloat16)
+        assert torch.equal(ql(x), v(x))
+    x = (torch.randn(16, 512, device=DEV) * 0.5).to(torch.bfloat16)
+    direct = VQ.verify_matmul(x, ql.weight, ql.scales, ql.biases, transpose=True, group_size=64, bits=4)
+    assert torch.equal(direct, v(x))
+    stock = ql(x).float()
+    assert (direct.float() - stock).abs().max() <= 2e-2 * stock.abs().max()
+    # a module moved after construction still dispatches on its current buffers
+    v2 = VerifyQuantizedLinear.from_quantized(QuantizedLinear.from_linear(lin.to(torch.bfloat16), 64, 4)).to(DEV)
+    assert torch.equal(v2(x), direct)
+
+
+def test_c_abi_direct_n16_and_errors(native_lib):
+    """N % 32 != 0 is outside the Python gate but inside the C ABI contract (N % 16)."""
+    L = native_lib
+    case = make_qmm_case(512, 48, 51).to(DEV)
+    y = torch.empty((16, 48), dtype=torch.bfloat16, device=DEV)
+    ws = torch.zeros(L.dflash_qmm_m16_workspace_bytes(512, 48, 64, 1, 4), dtype=torch.uint8, device=DEV)
+    for variant, kp in ((0, 1), (1, 4)):
+        y.zero_()
+        rc = L.dflash_qmm_m16(case.x.data_ptr(), case.w.data_ptr(), case.scales.data_ptr(),
+                              case.biases.data_ptr(), y.data_ptr(), ws.data_ptr(), ws.numel(),
+                              512, 48, 64, nat.BF16, nat.BF16, variant, kp, None)
+        assert rc == 0, L.dflash_last_error()
+        torch.cuda.synchronize()
+        exact = O.qmm_exact(case.x.float().cpu().numpy(), case.w.cpu().numpy().view(np.uint32),
+                            case.scales.float().cpu().numpy(), case.biases.float().cpu().numpy(), 64)
+        _check_north_star(_f32(y).astype(np.float64), exact)
+    assert int(ws[:65536].view(torch.int32).abs().sum()) == 0   # counter block handed back zeroed
