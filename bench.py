@@ -1,0 +1,314 @@
+#!/usr/bin/env python3
+"""Benchmark of the target-verify hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 27b|9b]
+
+One "step" is one pass of the M=16 int4 verify_qmm over every projection of the dense
+stack (27B-shaped by default: 64 layers x {qkv, o, gate, up, down} = 320 calls through
+``verify_matmul``, x re-drawn per call, all operands resident in HBM), replayed from a
+HIP graph so that host launch overhead is not what is measured.  The printed value is
+aggregate weight bytes (packed codes + scales + biases) per second.
+
+Also measured and reported in the same JSON line:
+  roofline      algorithmic bytes of the qmm kernel per launch / average launch
+                duration (HIP events around the timed region), against 8 TB/s HBM
+  replay        GDN tape-replay rollback, 48 layers x 32 heads, 16 steps, one launch
+  cpu_baseline  the oracle's C port of the reference arithmetic on the host cores,
+                on a bounded sample of the same workload
+
+Exactly one JSON line goes to stdout; progress goes to stderr.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build_stack(stack: str, device: str):
+    """All operands of one pass over the stack, generated on the device."""
+    import torch
+
+    from dflash_mlx_amd.workloads import make_qmm_case, seed_for, stack_linears
+
+    linears, layers, cfg = stack_linears(stack)
+    calls = []
+    for layer in range(layers):
+        for i, (_, K, N) in enumerate(linears):
+            calls.append(make_qmm_case(K, N, seed_for(cfg, layer) * 8 + i, device=device))
+    torch.cuda.synchronize()
+    return calls
+
+
+def run_pass(calls):
+    from dflash_mlx_amd.verify_qmm import verify_matmul
+
+    return [verify_matmul(c.x, c.w, c.scales, c.biases, group_size=c.group_size, bits=4) for c in calls]
+
+
+def time_region(fn, steps: int):
+    """Wall time and HIP-event time (ms) of ``steps`` invocations of fn."""
+    import torch
+
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return wall_ms, start.elapsed_time(stop)
+
+
+def capture(fn):
+    """Run ``fn`` once on a side stream (so that every lazily created buffer exists), then
+    record it into a HIP graph on that stream.  Returns (graph, outputs of the capture)."""
+    import torch
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            out = fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    return graph, out
+
+
+def bench_qmm_stack(stack: str, steps: int, warmup: int, device: str):
+    import torch
+
+    from dflash_mlx_amd.workloads import stack_bytes
+
+    calls = build_stack(stack, device)
+    weight_bytes, total_bytes = stack_bytes(stack)
+    log(f"[bench] {stack} stack: {len(calls)} qmm calls/step, {weight_bytes / 1e9:.3f} GB weights")
+
+    eager = run_pass(calls)  # also creates the split-K workspace outside of graph capture
+    torch.cuda.synchronize()
+
+    graph, captured = capture(lambda: run_pass(calls))
+
+    # every replay must reproduce the eager result bit for bit
+    for r in range(2):
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(eager, captured):
+            if not torch.equal(a, b):
+                raise RuntimeError(f"graph replay {r} differs from the eager result")
+
+    for _ in range(warmup):
+        graph.replay()
+    wall_ms, ev_ms = time_region(graph.replay, steps)
+    ms_per_step = wall_ms / steps
+    # eager launches through the Python surface, for the record
+    e_wall, _ = time_region(lambda: run_pass(calls), max(1, min(steps, 3)))
+    res = dict(
+        calls_per_step=len(calls), weight_bytes=weight_bytes, total_bytes=total_bytes,
+        ms_per_step=ms_per_step, event_ms_per_step=ev_ms / steps,
+        weight_gbps=weight_bytes / (ms_per_step * 1e-3) / 1e9,
+        avg_launch_us=ev_ms / steps / len(calls) * 1e3,
+        bytes_per_launch=total_bytes / len(calls),
+        eager_ms_per_step=e_wall / max(1, min(steps, 3)),
+    )
+    del graph, captured, eager, calls
+    torch.cuda.empty_cache()
+    return res
+
+
+def bench_single_call(device: str, launches: int = 200):
+    """config[0]: one 16x4096x4096 call, cold (ring of distinct weight sets larger than
+    the 256 MB Infinity Cache) and hot (same weights every launch)."""
+    import torch
+
+    from dflash_mlx_amd.verify_qmm import verify_matmul
+    from dflash_mlx_amd.workloads import make_qmm_case, qmm_algorithmic_bytes, seed_for
+
+    ring = [make_qmm_case(4096, 4096, seed_for(0) + i, device=device) for i in range(64)]
+    _, total = qmm_algorithmic_bytes(4096, 4096)
+    out = {}
+    for name, cases in (("cold", ring), ("hot", ring[:1])):
+        def one_round():
+            for i in range(launches):
+                c = cases[i % len(cases)]
+                verify_matmul(c.x, c.w, c.scales, c.biases)
+        g, _ = capture(one_round)
+        g.replay()
+        _, ev_ms = time_region(g.replay, 3)
+        us = ev_ms / 3 / launches * 1e3
+        out[name] = dict(us_per_call=us, gbps=total / us / 1e3, frac_hbm=total / (us * 1e-6) / HBM_PEAK)
+        del g
+    del ring
+    torch.cuda.empty_cache()
+    return out
+
+
+def bench_replay(device: str, steps: int, warmup: int):
+    """config[2]: 48 layers x 32 value heads, fp32 128x128 state, 16 recorded steps, all
+    applied; one launch per rollback.  Four state sets (800 MB) are rotated so that the
+    Infinity Cache cannot hold the working set."""
+    import torch
+
+    from dflash_mlx_amd.cache import KVCache
+    from dflash_mlx_amd.kernels import replay_launch
+    from dflash_mlx_amd.workloads import make_replay_case, replay_algorithmic_bytes
+
+    L, H, T = 48, 32, 16
+    sets = [make_replay_case(L, steps=T, seed=7000 + i, device=device) for i in range(4)]
+    outs = [torch.empty_like(s.state) for s in sets]
+    steps_dev = sets[0].steps
+
+    def one_pass(i):
+        c = sets[i % 4]
+        replay_launch(c.tape, c.k, c.g, c.state, outs[i % 4], steps=steps_dev, T_alloc=T, slots=L)
+
+    for i in range(max(warmup, 4)):
+        one_pass(i)
+    n = max(steps * 10, 40)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for i in range(n):
+        one_pass(i)
+    stop.record()
+    torch.cuda.synchronize()
+    us = start.elapsed_time(stop) / n * 1e3
+    total = replay_algorithmic_bytes(128, 128, T) * L * H
+    # KV trim of the 16 full-attention layers: offset arithmetic, no device work
+    kv = [KVCache() for _ in range(16)]
+    for c in kv:
+        c.offset = 4096 + 16
+    t0 = time.perf_counter_ns()
+    for c in kv:
+        c.trim(c.offset - (4096 + 7))
+    trim_ns = time.perf_counter_ns() - t0
+    assert all(c.offset == 4096 + 7 for c in kv)
+    del sets, outs
+    torch.cuda.empty_cache()
+    return dict(us_per_rollback=us, us_per_layer=us / L, gbps=total / us / 1e3,
+                frac_hbm=total / (us * 1e-6) / HBM_PEAK, bytes=total, layers=L, heads=H,
+                steps=T, kv_trim_host_ns_16_layers=trim_ns)
+
+
+def bench_cpu_baseline(stack: str, budget_s: float = 15.0):
+    """The oracle's C port of the reference kernel arithmetic (bf16-rounded dequantised
+    weights, fp32 accumulation) on the host cores, over as many linears of one layer of
+    the same stack as fit the time budget."""
+    from dflash_mlx_amd.workloads import make_qmm_case, qmm_algorithmic_bytes, seed_for, stack_linears
+    from oracle.c_binding import load_c_oracle
+    import numpy as np
+    import torch
+
+    orc = load_c_oracle(build_if_missing=True)
+    linears, _, cfg = stack_linears(stack)
+    done_bytes, spent, used = 0, 0.0, []
+    for i, (name, K, N) in enumerate(linears):
+        c = make_qmm_case(K, N, seed_for(cfg, 0) * 8 + i)
+        args = (c.x.view(torch.int16).numpy().view(np.uint16), c.w.numpy().view(np.uint32),
+                c.scales.view(torch.int16).numpy().view(np.uint16),
+                c.biases.view(torch.int16).numpy().view(np.uint16), 64)
+        t0 = time.perf_counter()
+        orc.qmm_m16(*args, flavour=1, k_parts=1)
+        dt = time.perf_counter() - t0
+        spent += dt
+        done_bytes += qmm_algorithmic_bytes(K, N)[0]
+        used.append(name)
+        if spent > budget_s:
+            break
+    return dict(value=done_bytes / spent / 1e9, unit="GB/s", cores=orc.num_threads(), kind="port",
+                sample=f"{'+'.join(used)} of layer 0 of the {stack} stack ({done_bytes / 1e6:.1f} MB of "
+                       f"weights, {spent:.1f} s), C/OpenMP port of the reference kernel arithmetic")
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="27b", choices=["27b", "9b"])
+    ap.add_argument("--skip-cpu", action="store_true", help="leave out the cpu_baseline leg")
+    ap.add_argument("--skip-extra", action="store_true", help="only the headline stack")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: the verify hot path is a single-device path and this "
+              "build has no multi-GPU leg; run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import dflash_mlx_amd._native as nat
+
+    nat.lib()  # no library, no benchmark: there is no fallback path to time
+    os.environ["DFLASH_VERIFY_QMM"] = "1"
+    os.environ.pop("DFLASH_VERIFY_VARIANT", None)
+    device = "cuda:0"
+    torch.cuda.set_device(0)
+
+    main_res = bench_qmm_stack(args.workload, args.steps, args.warmup, device)
+    log(f"[bench] {args.workload}: {main_res['ms_per_step']:.3f} ms/step, "
+        f"{main_res['weight_gbps']:.0f} GB/s weights, {main_res['avg_launch_us']:.2f} us/launch")
+    extra = {}
+    if not args.skip_extra:
+        other = "9b" if args.workload == "27b" else "27b"
+        o = bench_qmm_stack(other, args.steps, args.warmup, device)
+        extra[f"stack_{other}"] = dict(ms_per_step=round(o["ms_per_step"], 4),
+                                       weight_gbps=round(o["weight_gbps"], 1),
+                                       frac_hbm=round(o["total_bytes"] / (o["event_ms_per_step"] * 1e-3) / HBM_PEAK, 4))
+        extra["single_call_16x4096x4096"] = {k: {kk: round(vv, 4) for kk, vv in v.items()}
+                                             for k, v in bench_single_call(device).items()}
+        rp = bench_replay(device, args.steps, args.warmup)
+        extra["gdn_tape_replay"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in rp.items()}
+        log(f"[bench] replay: {rp['us_per_layer']:.3f} us/layer, {rp['gbps']:.0f} GB/s")
+
+    achieved = main_res["bytes_per_launch"] / (main_res["avg_launch_us"] * 1e-6) / 1e9
+    roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK / 1e9, unit="GB/s",
+                    frac=round(achieved * 1e9 / HBM_PEAK, 4), traffic=None,
+                    kernel="qmm_m16_kernel", bytes_per_launch=round(main_res["bytes_per_launch"]),
+                    avg_launch_us=round(main_res["avg_launch_us"], 3))
+    cpu = None if args.skip_cpu else bench_cpu_baseline(args.workload)
+
+    out = {
+        "metric": "verify_qmm M=16 GB/s (% HBM peak); GDN tape-replay us/layer at 16 steps",
+        "value": round(main_res["weight_gbps"], 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(main_res["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 x int4 (fp32 accumulate)",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}-shaped dense int4 verify stack, M=16, group 64, "
+                               f"{main_res['calls_per_step']} verify_matmul calls per step (HIP graph replay)",
+                   "weight_bytes_per_step": main_res["weight_bytes"],
+                   "eager_ms_per_step": round(main_res["eager_ms_per_step"], 3)},
+        "pct_hbm_peak": round(100.0 * main_res["weight_gbps"] * 1e9 / HBM_PEAK, 2),
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -12,10 +12,11 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
+QMM_KERNEL_AUTO, QMM_KERNEL_TILE, QMM_KERNEL_STREAM = 0, 1, 2
 
 # every symbol include/dflash_mi355.h declares
 EXPORTED_SYMBOLS = (
@@ -42,10 +43,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.dflash_last_error.restype = c.c_char_p
     lib.dflash_last_error.argtypes = []
     lib.dflash_qmm_m16_workspace_bytes.restype = c.c_size_t
-    lib.dflash_qmm_m16_workspace_bytes.argtypes = [c.c_int] * 5
+    lib.dflash_qmm_m16_workspace_bytes.argtypes = [c.c_int] * 6
     lib.dflash_qmm_m16.restype = c.c_int
     lib.dflash_qmm_m16.argtypes = (
-        [c.c_void_p] * 6 + [c.c_size_t] + [c.c_int] * 7 + [c.c_void_p]
+        [c.c_void_p] * 6 + [c.c_size_t] + [c.c_int] * 8 + [c.c_void_p]
     )
     lib.dflash_tape_replay.restype = c.c_int
     lib.dflash_tape_replay.argtypes = (

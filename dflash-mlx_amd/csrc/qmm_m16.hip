@@ -183,11 +183,15 @@ __global__ __launch_bounds__(kThreads) void qmm_m16_kernel(
     return;
   }
 
+  // Partial tiles travel as agent-scope relaxed atomics (written through to / read from
+  // the level all XCDs share); the barrier's vmcnt(0) retires the stores before the
+  // counter is bumped.  A release fence instead would write back the whole L2 per
+  // workgroup, which costs tens of microseconds.
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    partials[((size_t)part * 16 + m) * N + n0 + 16 * t + col] = v[t];
+    __hip_atomic_store(&partials[((size_t)part * 16 + m) * N + n0 + 16 * t + col], v[t],
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  __threadfence();
   __syncthreads();
   if (threadIdx.x == 0) {
     // wrapping increment: the k_parts-th arrival sees k_parts-1 and puts the counter
@@ -197,12 +201,12 @@ __global__ __launch_bounds__(kThreads) void qmm_m16_kernel(
   }
   __syncthreads();
   if (!is_last) return;
-  __threadfence();
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     float sum = 0.f;
     for (int p = 0; p < k_parts; ++p) {
-      sum += __builtin_nontemporal_load(&partials[((size_t)p * 16 + m) * N + n0 + 16 * t + col]);
+      sum += __hip_atomic_load(&partials[((size_t)p * 16 + m) * N + n0 + 16 * t + col],
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     y[(size_t)m * N + n0 + 16 * t + col] = (uint16_t)A::from_f32(sum);
   }
@@ -248,18 +252,34 @@ constexpr int kMaxCounterTiles = (int)(kCounterBytes / sizeof(uint32_t));
 }  // namespace
 }  // namespace dflash
 
+namespace dflash {
+// qmm_m16_stream.hip
+bool qmm_stream_eligible(int K, int N, int group_size);
+size_t qmm_stream_workspace_bytes(int N, int grid);
+int qmm_stream_grid();
+int qmm_stream_launch(const void* x, const uint32_t* w, const void* scales, const void* biases,
+                      void* y, void* workspace, size_t workspace_bytes, int K, int N,
+                      int act_dtype, int sb_dtype, hipStream_t stream);
+}  // namespace dflash
+
 extern "C" size_t dflash_qmm_m16_workspace_bytes(int K, int N, int group_size, int variant,
-                                                 int k_parts) {
-  (void)K;
-  (void)group_size;
-  if (variant != DFLASH_QMM_MMA2BIG_PIPE || k_parts <= 1 || N <= 0) return 0;
-  return dflash::kCounterBytes + (size_t)k_parts * 16 * (size_t)N * sizeof(float);
+                                                 int k_parts, int kernel) {
+  size_t need = 0;
+  if (N <= 0) return 0;
+  if (kernel != DFLASH_QMM_KERNEL_STREAM && variant == DFLASH_QMM_MMA2BIG_PIPE && k_parts > 1) {
+    need = dflash::kCounterBytes + (size_t)k_parts * 16 * (size_t)N * sizeof(float);
+  }
+  if (kernel != DFLASH_QMM_KERNEL_TILE && dflash::qmm_stream_eligible(K, N, group_size)) {
+    const size_t s = dflash::qmm_stream_workspace_bytes(N, dflash::qmm_stream_grid());
+    need = s > need ? s : need;
+  }
+  return need;
 }
 
 extern "C" int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* scales,
                               const void* biases, void* y, void* workspace, size_t workspace_bytes,
                               int K, int N, int group_size, int act_dtype, int sb_dtype,
-                              int variant, int k_parts, void* stream) {
+                              int variant, int k_parts, int kernel, void* stream) {
   using namespace dflash;
   DFLASH_REQUIRE(x && w_q && scales && biases && y, DFLASH_ERR_ARG, "dflash_qmm_m16: null operand");
   DFLASH_REQUIRE(act_dtype == DFLASH_BF16 || act_dtype == DFLASH_FP16, DFLASH_ERR_ARG,
@@ -273,15 +293,26 @@ extern "C" int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* sc
   DFLASH_REQUIRE(K > 0 && N > 0 && N % 16 == 0 && K % group_size == 0, DFLASH_ERR_SHAPE,
                  "dflash_qmm_m16: need N %% 16 == 0 and K %% group_size == 0 (K=%d N=%d gs=%d)", K,
                  N, group_size);
+  DFLASH_REQUIRE(kernel == DFLASH_QMM_KERNEL_AUTO || kernel == DFLASH_QMM_KERNEL_TILE ||
+                     kernel == DFLASH_QMM_KERNEL_STREAM,
+                 DFLASH_ERR_ARG, "dflash_qmm_m16: unknown kernel selector %d", kernel);
   if (variant == DFLASH_QMM_MMA2BIG) k_parts = 1;
   DFLASH_REQUIRE(k_parts >= 1 && K % (32 * k_parts) == 0, DFLASH_ERR_SHAPE,
                  "dflash_qmm_m16: K=%d is not a multiple of 32*k_parts (k_parts=%d)", K, k_parts);
   DFLASH_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)w_q % 16) == 0, DFLASH_ERR_ARG,
                  "dflash_qmm_m16: x and w_q must be 16-byte aligned");
+  if (kernel != DFLASH_QMM_KERNEL_TILE && qmm_stream_eligible(K, N, group_size)) {
+    return qmm_stream_launch(x, w_q, scales, biases, y, workspace, workspace_bytes, K, N, act_dtype,
+                             sb_dtype, (hipStream_t)stream);
+  }
+  DFLASH_REQUIRE(kernel != DFLASH_QMM_KERNEL_STREAM, DFLASH_ERR_SHAPE,
+                 "dflash_qmm_m16: the streaming kernel needs group_size 64 and K %% 1024 == 0 "
+                 "(K=%d gs=%d)", K, group_size);
   float* partials = nullptr;
   uint32_t* counters = nullptr;
   if (k_parts > 1) {
-    const size_t need = dflash_qmm_m16_workspace_bytes(K, N, group_size, variant, k_parts);
+    const size_t need = dflash_qmm_m16_workspace_bytes(K, N, group_size, variant, k_parts,
+                                                       DFLASH_QMM_KERNEL_TILE);
     DFLASH_REQUIRE(workspace && workspace_bytes >= need, DFLASH_ERR_WORKSPACE,
                    "dflash_qmm_m16: workspace of %zu bytes needed, %zu given", need,
                    workspace ? workspace_bytes : (size_t)0);

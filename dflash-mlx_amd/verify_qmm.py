@@ -12,6 +12,8 @@ and shape dispatch, with the device work done by the gfx950 kernel behind
   silently, as in the reference.
 * ``DFLASH_VERIFY_VARIANT`` in {auto, mma2big, mma2big_pipe} and
   ``DFLASH_VERIFY_QMM_KPARTS`` select the variant (:15-22, 292-297).
+* ``DFLASH_QMM_KERNEL`` in {auto, tile, stream} picks the device kernel (no counterpart
+  in the reference; auto uses the streaming kernel for group 64 and K % 512 == 0).
 * An eligible call needs device tensors and the built HIP library; there is no
   software fallback for it.
 """
@@ -27,6 +29,15 @@ from .quantized import quantized_matmul
 
 _DTYPE_CODE = {torch.bfloat16: _native.BF16, torch.float16: _native.FP16}
 _VARIANT_CODE = {"mma2big": _native.QMM_MMA2BIG, "mma2big_pipe": _native.QMM_MMA2BIG_PIPE}
+_KERNEL_CODE = {"auto": _native.QMM_KERNEL_AUTO, "tile": _native.QMM_KERNEL_TILE,
+                "stream": _native.QMM_KERNEL_STREAM}
+
+
+def _kernel_select() -> int:
+    """``DFLASH_QMM_KERNEL`` in {auto, tile, stream}: which device kernel serves eligible
+    calls (auto: the streaming kernel wherever it applies, the tile kernel elsewhere)."""
+    return _KERNEL_CODE.get(os.environ.get("DFLASH_QMM_KERNEL", "auto").strip().lower(),
+                            _native.QMM_KERNEL_AUTO)
 
 
 def is_enabled() -> bool:
@@ -67,7 +78,7 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
     ws = _WORKSPACES.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 1 << 22), dtype=torch.uint8, device=device)
+        ws = torch.zeros(max(nbytes, 1 << 23), dtype=torch.uint8, device=device)
         _WORKSPACES[key] = ws
     return ws
 
@@ -84,14 +95,16 @@ def _launch(x2: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: tor
     y = torch.empty((16, N), dtype=x2.dtype, device=x2.device)
     stream = torch.cuda.current_stream(x2.device).cuda_stream
     vcode = _VARIANT_CODE[variant]
-    need = lib.dflash_qmm_m16_workspace_bytes(K, N, group_size, vcode, k_parts)
+    kernel = _kernel_select()
+    need = lib.dflash_qmm_m16_workspace_bytes(K, N, group_size, vcode, k_parts, kernel)
     ws_ptr, ws_bytes = None, 0
     if need:
         ws = _workspace(x2.device, stream, need)
         ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
     rc = lib.dflash_qmm_m16(x2.data_ptr(), w.data_ptr(), scales.data_ptr(), biases.data_ptr(),
                             y.data_ptr(), ws_ptr, ws_bytes, K, N, group_size,
-                            _DTYPE_CODE[x2.dtype], _DTYPE_CODE[scales.dtype], vcode, k_parts, stream)
+                            _DTYPE_CODE[x2.dtype], _DTYPE_CODE[scales.dtype], vcode, k_parts, kernel,
+                            stream)
     _native.check(rc, "dflash_qmm_m16")
     return y
 

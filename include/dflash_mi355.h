@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 1
+#define DFLASH_ABI_VERSION 2
 
 enum {
   DFLASH_OK = 0,
@@ -40,6 +40,15 @@ enum { DFLASH_BF16 = 0, DFLASH_FP16 = 1, DFLASH_FP32 = 2 };
 
 /* Shape dispatch of dflash_mlx/verify_qmm.py:19-22, 299-331. */
 enum { DFLASH_QMM_MMA2BIG = 0, DFLASH_QMM_MMA2BIG_PIPE = 1 };
+
+/*
+ * Which device kernel serves a qmm call.  TILE: one workgroup per 32 output columns and
+ * per K slice, K cut into k_parts slices for the pipe variant.  STREAM: persistent
+ * workgroups that divide the weight matrix evenly and stream it through LDS; needs
+ * group_size 64 and K % 1024 == 0, and decides the K split itself (variant and k_parts
+ * then only name the caller's dispatch decision).  AUTO: STREAM where it applies.
+ */
+enum { DFLASH_QMM_KERNEL_AUTO = 0, DFLASH_QMM_KERNEL_TILE = 1, DFLASH_QMM_KERNEL_STREAM = 2 };
 
 int dflash_abi_version(void);
 const char* dflash_last_error(void);
@@ -66,11 +75,12 @@ const char* dflash_last_error(void);
  * for the pipe variant K % (32*k_parts) == 0.  Results are deterministic
  * (bit-identical from run to run for identical inputs).
  */
-size_t dflash_qmm_m16_workspace_bytes(int K, int N, int group_size, int variant, int k_parts);
+size_t dflash_qmm_m16_workspace_bytes(int K, int N, int group_size, int variant, int k_parts,
+                                      int kernel);
 
 int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* scales, const void* biases,
                    void* y, void* workspace, size_t workspace_bytes, int K, int N, int group_size,
-                   int act_dtype, int sb_dtype, int variant, int k_parts, void* stream);
+                   int act_dtype, int sb_dtype, int variant, int k_parts, int kernel, void* stream);
 
 /*
  * GatedDeltaNet tape replay: for every slot s and value head hv apply the first

@@ -40,6 +40,6 @@ def verify_env(monkeypatch):
     """Environment of an enabled verify kernel with default dispatch."""
     monkeypatch.setenv("DFLASH_VERIFY_QMM", "1")
     for name in ("DFLASH_VERIFY_VARIANT", "DFLASH_VERIFY_QMM_KPARTS", "DFLASH_VERIFY_MAX_N",
-                 "DFLASH_VERIFY_INCLUDE", "DFLASH_VERIFY_LINEAR", "DFLASH_REPLAY_EXACT"):
+                 "DFLASH_VERIFY_INCLUDE", "DFLASH_VERIFY_LINEAR", "DFLASH_REPLAY_EXACT", "DFLASH_QMM_KERNEL"):
         monkeypatch.delenv(name, raising=False)
     return monkeypatch

@@ -21,6 +21,14 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+@pytest.fixture(autouse=True, params=["auto", "tile"])
+def kernel_mode(request, verify_env):
+    """Every test runs once with the streaming kernel where it applies (auto) and once
+    with the tile kernel forced."""
+    verify_env.setenv("DFLASH_QMM_KERNEL", request.param)
+    return request.param
+
+
 def _bits(t):
     return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
 
@@ -158,14 +166,21 @@ def test_deterministic_and_workspace_reuse(verify_env, native_lib, c_oracle):
     _check_north_star(_f32(yb).astype(np.float64), _oracle_exact(c_oracle, b.to("cpu")))
 
 
-def test_n_tiles_are_independent_full_size(verify_env, native_lib):
-    """Size-independent property at a full 27B shape: any N-slice of W gives the same
-    bits as the matching slice of the full product."""
+def test_n_tiles_are_independent_full_size(verify_env, native_lib, kernel_mode):
+    """Size-independent property at a full 27B shape: any N-slice of W gives the matching
+    slice of the full product - the same bits with the tile kernel (fixed K split), and to
+    within one output rounding with the streaming kernel, whose K split follows the even
+    division of the whole matrix among workgroups and therefore changes with N."""
     case = make_qmm_case(5120, 17408, 31).to(DEV)
     full = VQ.verify_matmul(case.x, case.w, case.scales, case.biases)
     for n0, n1 in [(0, 32), (4096, 4096 + 512), (17408 - 64, 17408)]:
         part = VQ.verify_matmul(case.x, case.w[n0:n1], case.scales[n0:n1], case.biases[n0:n1])
-        assert torch.equal(part, full[:, n0:n1])
+        if kernel_mode == "tile":
+            assert torch.equal(part, full[:, n0:n1])
+        else:
+            ref = full[:, n0:n1].float()
+            assert (part.float() - ref).abs().max() <= 2 ** -7 * ref.abs().max()
+            assert (part == full[:, n0:n1]).float().mean() > 0.95
 
 
 def test_linearity_full_size(verify_env, native_lib):
@@ -225,14 +240,16 @@ def test_verify_linear_on_device(verify_env, native_lib):
 def test_c_abi_direct_n16_and_errors(native_lib):
     """N % 32 != 0 is outside the Python gate but inside the C ABI contract (N % 16)."""
     L = native_lib
-    case = make_qmm_case(512, 48, 51).to(DEV)
+    case = make_qmm_case(1024, 48, 51).to(DEV)
     y = torch.empty((16, 48), dtype=torch.bfloat16, device=DEV)
-    ws = torch.zeros(L.dflash_qmm_m16_workspace_bytes(512, 48, 64, 1, 4), dtype=torch.uint8, device=DEV)
-    for variant, kp in ((0, 1), (1, 4)):
+    ws = torch.zeros(L.dflash_qmm_m16_workspace_bytes(1024, 48, 64, 1, 4, nat.QMM_KERNEL_AUTO),
+                     dtype=torch.uint8, device=DEV)
+    for variant, kp, kernel in ((0, 1, nat.QMM_KERNEL_TILE), (1, 4, nat.QMM_KERNEL_TILE),
+                                (0, 1, nat.QMM_KERNEL_STREAM), (1, 4, nat.QMM_KERNEL_AUTO)):
         y.zero_()
         rc = L.dflash_qmm_m16(case.x.data_ptr(), case.w.data_ptr(), case.scales.data_ptr(),
                               case.biases.data_ptr(), y.data_ptr(), ws.data_ptr(), ws.numel(),
-                              512, 48, 64, nat.BF16, nat.BF16, variant, kp, None)
+                              1024, 48, 64, nat.BF16, nat.BF16, variant, kp, kernel, None)
         assert rc == 0, L.dflash_last_error()
         torch.cuda.synchronize()
         exact = O.qmm_exact(case.x.float().cpu().numpy(), case.w.cpu().numpy().view(np.uint32),
