@@ -31,6 +31,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
+# HBM bytes per launch of the qmm kernel on each stack (mean over its launches), from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file scaled by the same counters'
+# reading for a 1 GiB copy (x2.000 / x1.000); None where not measured for the current kernel.
+MEASURED_TRAFFIC_BYTES = {"27b": 55.03e6, "9b": None}
 
 
 def log(*a):
@@ -207,34 +211,35 @@ def bench_replay(device: str, steps: int, warmup: int):
                 steps=T, kv_trim_host_ns_16_layers=trim_ns)
 
 
-def bench_cpu_baseline(stack: str, budget_s: float = 15.0):
+def bench_cpu_baseline(stack: str, budget_s: float = 12.0):
     """The oracle's C port of the reference kernel arithmetic (bf16-rounded dequantised
-    weights, fp32 accumulation) on the host cores, over as many linears of one layer of
-    the same stack as fit the time budget."""
+    weights, fp32 accumulation) on the host cores: whole layers of the same stack, one
+    after the other, until the time budget is used up."""
     from dflash_mlx_amd.workloads import make_qmm_case, qmm_algorithmic_bytes, seed_for, stack_linears
     from oracle.c_binding import load_c_oracle
     import numpy as np
     import torch
 
     orc = load_c_oracle(build_if_missing=True)
-    linears, _, cfg = stack_linears(stack)
-    done_bytes, spent, used = 0, 0.0, []
-    for i, (name, K, N) in enumerate(linears):
-        c = make_qmm_case(K, N, seed_for(cfg, 0) * 8 + i)
-        args = (c.x.view(torch.int16).numpy().view(np.uint16), c.w.numpy().view(np.uint32),
-                c.scales.view(torch.int16).numpy().view(np.uint16),
-                c.biases.view(torch.int16).numpy().view(np.uint16), 64)
-        t0 = time.perf_counter()
-        orc.qmm_m16(*args, flavour=1, k_parts=1)
-        dt = time.perf_counter() - t0
-        spent += dt
-        done_bytes += qmm_algorithmic_bytes(K, N)[0]
-        used.append(name)
+    linears, layers, cfg = stack_linears(stack)
+    done_bytes, spent, n_layers = 0, 0.0, 0
+    for layer in range(layers):
+        for i, (name, K, N) in enumerate(linears):
+            c = make_qmm_case(K, N, seed_for(cfg, layer) * 8 + i)
+            args = (c.x.view(torch.int16).numpy().view(np.uint16), c.w.numpy().view(np.uint32),
+                    c.scales.view(torch.int16).numpy().view(np.uint16),
+                    c.biases.view(torch.int16).numpy().view(np.uint16), 64)
+            t0 = time.perf_counter()
+            orc.qmm_m16(*args, flavour=1, k_parts=1)
+            spent += time.perf_counter() - t0
+            done_bytes += qmm_algorithmic_bytes(K, N)[0]
+        n_layers += 1
         if spent > budget_s:
             break
-    return dict(value=done_bytes / spent / 1e9, unit="GB/s", cores=orc.num_threads(), kind="port",
-                sample=f"{'+'.join(used)} of layer 0 of the {stack} stack ({done_bytes / 1e6:.1f} MB of "
-                       f"weights, {spent:.1f} s), C/OpenMP port of the reference kernel arithmetic")
+    return dict(value=round(done_bytes / spent / 1e9, 3), unit="GB/s", cores=orc.num_threads(), kind="port",
+                sample=f"{n_layers} of {layers} layers of the {stack} stack ({done_bytes / 1e9:.2f} GB of "
+                       f"weights in {spent:.1f} s of compute; input generation not timed), C/OpenMP port "
+                       f"of the reference kernel arithmetic")
 
 
 def main() -> int:
@@ -245,6 +250,9 @@ def main() -> int:
     ap.add_argument("--workload", default="27b", choices=["27b", "9b"])
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the cpu_baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the headline stack")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run three 1 GiB device-to-device copies (a kernel of known traffic, "
+                         "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings) and exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the verify hot path is a single-device path and this "
@@ -252,6 +260,15 @@ def main() -> int:
         return 2
 
     import torch
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": 1 << 30, "copy_bytes_written": 1 << 30, "copies": 3}))
+        return 0
 
     import dflash_mlx_amd._native as nat
 
@@ -279,8 +296,8 @@ def main() -> int:
 
     achieved = main_res["bytes_per_launch"] / (main_res["avg_launch_us"] * 1e-6) / 1e9
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK / 1e9, unit="GB/s",
-                    frac=round(achieved * 1e9 / HBM_PEAK, 4), traffic=None,
-                    kernel="qmm_m16_kernel", bytes_per_launch=round(main_res["bytes_per_launch"]),
+                    frac=round(achieved * 1e9 / HBM_PEAK, 4), traffic=MEASURED_TRAFFIC_BYTES.get(args.workload),
+                    kernel="qmm_stream_kernel", bytes_per_launch=round(main_res["bytes_per_launch"]),
                     avg_launch_us=round(main_res["avg_launch_us"], 3))
     cpu = None if args.skip_cpu else bench_cpu_baseline(args.workload)
 
