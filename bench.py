@@ -164,6 +164,51 @@ def bench_single_call(device: str, launches: int = 200):
     return out
 
 
+def bench_moe(device: str, steps: int, warmup: int, layers: int = 40):
+    """config[4]: MoE-shaped verify step at M=16 - 256 experts of intermediate 512 (gate/up
+    2048->512, down 512->2048), top-8 routing, gathered per-expert qmm, plus a shared expert
+    through verify_matmul; `layers` layers replayed from a HIP graph.  Algorithmic bytes
+    count the weights of the experts the seeded routing actually touches."""
+    import torch
+
+    from dflash_mlx_amd.verify_qmm import gather_qmm, verify_matmul
+    from dflash_mlx_amd.workloads import make_moe_case, make_qmm_case, qmm_algorithmic_bytes, seed_for
+
+    per_expert = 3 * qmm_algorithmic_bytes(2048, 512)[0]
+    calls, total = [], 0
+    for layer in range(layers):
+        gate = make_moe_case(2048, 512, seed_for(4, layer) * 8, device=device)
+        up = make_moe_case(2048, 512, seed_for(4, layer) * 8 + 1, device=device)
+        up.expert_ids = gate.expert_ids
+        down = make_moe_case(512, 2048, seed_for(4, layer) * 8 + 2, device=device)
+        down.expert_ids = gate.expert_ids
+        shared = [make_qmm_case(2048, 512, seed_for(4, layer) * 8 + 3, device=device),
+                  make_qmm_case(2048, 512, seed_for(4, layer) * 8 + 4, device=device),
+                  make_qmm_case(512, 2048, seed_for(4, layer) * 8 + 5, device=device)]
+        calls.append((gate, up, down, shared))
+        total += (int(torch.unique(gate.expert_ids).numel()) + 1) * per_expert
+    torch.cuda.synchronize()
+
+    def one_pass():
+        out = []
+        for gate, up, down, shared in calls:
+            for c in (gate, up, down):
+                out.append(gather_qmm(c.x, c.w, c.scales, c.biases, c.expert_ids, group_size=64))
+            for c in shared:
+                out.append(verify_matmul(c.x, c.w, c.scales, c.biases))
+        return out
+
+    g, _ = capture(one_pass)
+    for _ in range(max(1, warmup)):
+        g.replay()
+    wall_ms, ev_ms = time_region(g.replay, steps)
+    ms = wall_ms / steps
+    del g, calls
+    torch.cuda.empty_cache()
+    return dict(layers=layers, ms_per_step=ms, weight_bytes=total, weight_gbps=total / (ms * 1e-3) / 1e9,
+                frac_hbm=total / (ms * 1e-3) / HBM_PEAK)
+
+
 def bench_replay(device: str, steps: int, warmup: int):
     """config[2]: 48 layers x 32 value heads, fp32 128x128 state, 16 recorded steps, all
     applied; one launch per rollback.  Four state sets (800 MB) are rotated so that the
@@ -290,6 +335,9 @@ def main() -> int:
                                        frac_hbm=round(o["total_bytes"] / (o["event_ms_per_step"] * 1e-3) / HBM_PEAK, 4))
         extra["single_call_16x4096x4096"] = {k: {kk: round(vv, 4) for kk, vv in v.items()}
                                              for k, v in bench_single_call(device).items()}
+        mo = bench_moe(device, args.steps, args.warmup)
+        extra["moe_35b_a3b_stack"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in mo.items()}
+        log(f"[bench] moe: {mo['ms_per_step']:.3f} ms/step, {mo['weight_gbps']:.0f} GB/s")
         rp = bench_replay(device, args.steps, args.warmup)
         extra["gdn_tape_replay"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in rp.items()}
         log(f"[bench] replay: {rp['us_per_layer']:.3f} us/layer, {rp['gbps']:.0f} GB/s")

@@ -24,6 +24,7 @@ EXPORTED_SYMBOLS = (
     "dflash_last_error",
     "dflash_qmm_m16_workspace_bytes",
     "dflash_qmm_m16",
+    "dflash_qmm_m16_gather",
     "dflash_tape_replay",
     "dflash_conv_state_rebuild",
 )
@@ -48,6 +49,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.dflash_qmm_m16.argtypes = (
         [c.c_void_p] * 6 + [c.c_size_t] + [c.c_int] * 8 + [c.c_void_p]
     )
+    lib.dflash_qmm_m16_gather.restype = c.c_int
+    lib.dflash_qmm_m16_gather.argtypes = [c.c_void_p] * 6 + [c.c_int] * 7 + [c.c_void_p]
     lib.dflash_tape_replay.restype = c.c_int
     lib.dflash_tape_replay.argtypes = (
         [c.c_void_p] * 6 + [c.c_int] + [c.c_void_p] + [c.c_int] * 12 + [c.c_void_p]

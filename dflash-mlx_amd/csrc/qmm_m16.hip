@@ -242,6 +242,148 @@ int launch_gs(int act_dtype, int sb_dtype, const void* x, const uint32_t* w, con
   return launch<GS, true, true>(x, w, scales, biases, y, partials, counters, K, N, k_parts, stream);
 }
 
+// ---------------------------------------------------------------------------
+// Gathered per-expert form: row p of x is multiplied by the weights of expert
+// expert_ids[p].  One workgroup per (column block, expert); a workgroup whose
+// expert owns no row exits at once.  Rows of one expert are collected in ascending
+// row order (so results do not depend on scheduling), processed 16 at a time as the
+// M dimension of the same MFMA tile, rows beyond the expert's count are zero.
+// ---------------------------------------------------------------------------
+constexpr int kMaxGatherRows = 2048;
+
+template <int GS, bool ACT_FP16, bool SB_FP16, int NT>
+__global__ __launch_bounds__(kThreads) void qmm_m16_gather_kernel(
+    const uint16_t* __restrict__ x, const int32_t* __restrict__ expert_ids,
+    const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
+    const uint16_t* __restrict__ biases, uint16_t* __restrict__ y, int P, int K, int N) {
+  using A = Act<ACT_FP16>;
+  constexpr int WPL = GS / 32;
+  __shared__ int rows[kMaxGatherRows];
+  __shared__ int n_rows;
+  __shared__ float red[kWaves][NT][4][64];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int col = lane & 15;
+  const int kblk = lane >> 4;
+  const int n0 = blockIdx.x * (16 * NT);
+  const int e = blockIdx.y;
+
+  // wave 0 lists the rows of expert e in ascending order
+  if (wave == 0) {
+    int count = 0;
+    for (int base = 0; base < P; base += 64) {
+      const int pidx = base + lane;
+      const bool mine = pidx < P && expert_ids[pidx] == e;
+      const unsigned long long m = __ballot(mine);
+      if (mine) rows[count + __popcll(m & ((1ull << lane) - 1ull))] = pidx;
+      count += __popcll(m);
+    }
+    if (lane == 0) n_rows = count;
+  }
+  __syncthreads();
+  const int count = n_rows;
+  if (count == 0) return;
+
+  const int G = K / GS;
+  const int words_per_row = K >> 3;
+  const uint32_t* we = w + (size_t)e * N * words_per_row;
+  const uint16_t* se = scales + (size_t)e * N * G;
+  const uint16_t* be = biases + (size_t)e * N * G;
+  const uint4 ones = make_uint4(A::kOnes, A::kOnes, A::kOnes, A::kOnes);
+  const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+
+  for (int base = 0; base < count; base += 16) {
+    const int my_row = base + col < count ? rows[base + col] : -1;
+    const uint16_t* xrow = x + (size_t)(my_row < 0 ? 0 : my_row) * K + kblk * (GS / 4);
+    f32x4_t acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int g = wave; g < G; g += kWaves) {
+      uint4 a[WPL];
+#pragma unroll
+      for (int j = 0; j < WPL; ++j) {
+        const uint4 v = *reinterpret_cast<const uint4*>(xrow + (size_t)g * GS + 8 * j);
+        a[j] = permute_x(my_row < 0 ? zero4 : v);
+      }
+      f32x4_t xs = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < WPL; ++j) xs = A::mfma(a[j], ones, xs);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const int n = n0 + 16 * t + col;
+        const uint32_t* wp = we + (size_t)n * words_per_row + (size_t)g * (GS / 8) + kblk * WPL;
+        uint32_t wd[WPL];
+        if constexpr (WPL == 1) {
+          wd[0] = wp[0];
+        } else if constexpr (WPL == 2) {
+          const uint2 v = *reinterpret_cast<const uint2*>(wp);
+          wd[0] = v.x;
+          wd[1] = v.y;
+        } else {
+          const uint4 v = *reinterpret_cast<const uint4*>(wp);
+          wd[0] = v.x;
+          wd[1] = v.y;
+          wd[2] = v.z;
+          wd[3] = v.w;
+        }
+        f32x4_t c = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < WPL; ++j) c = A::mfma(a[j], unpack_codes<ACT_FP16>(wd[j]), c);
+        const float s = sb_to_f32<SB_FP16>(se[(size_t)n * G + g]);
+        const float b = sb_to_f32<SB_FP16>(be[(size_t)n * G + g]);
+        const float bb = b - A::kOffset * s;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[t][r] += s * c[r] + bb * xs[r];
+      }
+    }
+    __syncthreads();  // red[] of the previous 16 rows has been read
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][t][r][lane] = acc[t][r];
+    __syncthreads();
+    const int r = wave;
+    const int m = base + 4 * (lane >> 4) + r;
+    if (m < count) {
+      const int out_row = rows[m];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const float v = (red[0][t][r][lane] + red[1][t][r][lane]) + (red[2][t][r][lane] + red[3][t][r][lane]);
+        y[(size_t)out_row * N + n0 + 16 * t + col] = (uint16_t)A::from_f32(v);
+      }
+    }
+  }
+}
+
+template <int GS>
+int launch_gather_gs(int act_dtype, int sb_dtype, const void* x, const int32_t* ids, const uint32_t* w,
+                     const void* scales, const void* biases, void* y, int P, int K, int N, int E,
+                     hipStream_t stream) {
+  const bool a16 = act_dtype == DFLASH_FP16, s16 = sb_dtype == DFLASH_FP16;
+  const dim3 block(kThreads);
+#define DFLASH_GATHER_LAUNCH(A16, S16)                                                             \
+  do {                                                                                             \
+    if (N % 32 == 0) {                                                                             \
+      hipLaunchKernelGGL((qmm_m16_gather_kernel<GS, A16, S16, 2>), dim3(N / 32, E), block, 0,      \
+                         stream, (const uint16_t*)x, ids, w, (const uint16_t*)scales,              \
+                         (const uint16_t*)biases, (uint16_t*)y, P, K, N);                          \
+    } else {                                                                                       \
+      hipLaunchKernelGGL((qmm_m16_gather_kernel<GS, A16, S16, 1>), dim3(N / 16, E), block, 0,      \
+                         stream, (const uint16_t*)x, ids, w, (const uint16_t*)scales,              \
+                         (const uint16_t*)biases, (uint16_t*)y, P, K, N);                          \
+    }                                                                                              \
+  } while (0)
+  if (!a16 && !s16) DFLASH_GATHER_LAUNCH(false, false);
+  if (!a16 && s16) DFLASH_GATHER_LAUNCH(false, true);
+  if (a16 && !s16) DFLASH_GATHER_LAUNCH(true, false);
+  if (a16 && s16) DFLASH_GATHER_LAUNCH(true, true);
+#undef DFLASH_GATHER_LAUNCH
+  DFLASH_HIP_OK(hipGetLastError());
+  return DFLASH_OK;
+}
+
 // Layout of the workspace: [arrival counters, fixed 64 KiB][partials: k_parts*16*N fp32].
 // The counter block has the same size for every shape so that calls of different
 // shapes sharing one workspace never put partial sums where another call keeps its
@@ -330,5 +472,39 @@ extern "C" int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* sc
       return launch_gs<64>(act_dtype, sb_dtype, x, w_q, scales, biases, y, partials, counters, K, N, k_parts, s);
     default:
       return launch_gs<128>(act_dtype, sb_dtype, x, w_q, scales, biases, y, partials, counters, K, N, k_parts, s);
+  }
+}
+
+extern "C" int dflash_qmm_m16_gather(const void* x, const int32_t* expert_ids, const uint32_t* w_q,
+                                     const void* scales, const void* biases, void* y, int P, int K,
+                                     int N, int E, int group_size, int act_dtype, int sb_dtype,
+                                     void* stream) {
+  using namespace dflash;
+  DFLASH_REQUIRE(x && expert_ids && w_q && scales && biases && y, DFLASH_ERR_ARG,
+                 "dflash_qmm_m16_gather: null operand");
+  DFLASH_REQUIRE(act_dtype == DFLASH_BF16 || act_dtype == DFLASH_FP16, DFLASH_ERR_ARG,
+                 "dflash_qmm_m16_gather: act_dtype %d is not bf16/fp16", act_dtype);
+  DFLASH_REQUIRE(sb_dtype == DFLASH_BF16 || sb_dtype == DFLASH_FP16, DFLASH_ERR_ARG,
+                 "dflash_qmm_m16_gather: sb_dtype %d is not bf16/fp16", sb_dtype);
+  DFLASH_REQUIRE(group_size == 32 || group_size == 64 || group_size == 128, DFLASH_ERR_SHAPE,
+                 "dflash_qmm_m16_gather: group_size %d not in {32,64,128}", group_size);
+  DFLASH_REQUIRE(K > 0 && N > 0 && E > 0 && P >= 0 && N % 16 == 0 && K % group_size == 0,
+                 DFLASH_ERR_SHAPE,
+                 "dflash_qmm_m16_gather: need N %% 16 == 0 and K %% group_size == 0 (K=%d N=%d gs=%d)",
+                 K, N, group_size);
+  DFLASH_REQUIRE(P <= kMaxGatherRows, DFLASH_ERR_SHAPE,
+                 "dflash_qmm_m16_gather: at most %d rows per call, got %d", kMaxGatherRows, P);
+  DFLASH_REQUIRE(E <= 65535, DFLASH_ERR_SHAPE, "dflash_qmm_m16_gather: too many experts (%d)", E);
+  DFLASH_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)w_q % 16) == 0 && (K * 2) % 16 == 0,
+                 DFLASH_ERR_ARG, "dflash_qmm_m16_gather: x and w_q must be 16-byte aligned");
+  if (P == 0) return DFLASH_OK;
+  hipStream_t s = (hipStream_t)stream;
+  switch (group_size) {
+    case 32:
+      return launch_gather_gs<32>(act_dtype, sb_dtype, x, expert_ids, w_q, scales, biases, y, P, K, N, E, s);
+    case 64:
+      return launch_gather_gs<64>(act_dtype, sb_dtype, x, expert_ids, w_q, scales, biases, y, P, K, N, E, s);
+    default:
+      return launch_gather_gs<128>(act_dtype, sb_dtype, x, expert_ids, w_q, scales, biases, y, P, K, N, E, s);
   }
 }

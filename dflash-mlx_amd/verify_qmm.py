@@ -147,3 +147,31 @@ def verify_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases
 
 # the name the hot path is known by
 verify_qmm = verify_matmul
+
+
+def gather_qmm(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
+               expert_ids: torch.Tensor, *, group_size: int = 64, bits: int = 4) -> torch.Tensor:
+    """Per-row expert selection for MoE layers: ``y[p] = x[p] @ dequant(w[expert_ids[p]]).T``.
+
+    ``x [P, K]`` bf16/fp16, ``w [E, N, K/8]`` packed, ``scales``/``biases [E, N, K/group]``,
+    ``expert_ids [P]`` integer.  Not part of the reference (its experts use mlx_lm's switch
+    layers); provided for the MoE-shaped verify step.  Device tensors only."""
+    if bits != 4:
+        raise NotImplementedError("only 4-bit codes are implemented")
+    if not x.is_cuda:
+        raise _native.NativeLibraryError("gather_qmm runs on the GPU only")
+    lib = _native.lib()
+    x2 = x.reshape(-1, x.shape[-1]).contiguous()
+    ids = expert_ids.reshape(-1).to(torch.int32).contiguous()
+    w_q, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
+    P, K = int(x2.shape[0]), int(x2.shape[1])
+    E, N = int(w_q.shape[0]), int(w_q.shape[1])
+    if ids.numel() != P:
+        raise ValueError("one expert id per row of x is required")
+    y = torch.empty((P, N), dtype=x2.dtype, device=x2.device)
+    stream = torch.cuda.current_stream(x2.device).cuda_stream
+    rc = lib.dflash_qmm_m16_gather(x2.data_ptr(), ids.data_ptr(), w_q.data_ptr(), scales.data_ptr(),
+                                   biases.data_ptr(), y.data_ptr(), P, K, N, E, group_size,
+                                   _DTYPE_CODE[x2.dtype], _DTYPE_CODE[scales.dtype], stream)
+    _native.check(rc, "dflash_qmm_m16_gather")
+    return y.reshape(*x.shape[:-1], N)

@@ -142,3 +142,32 @@ def make_replay_case(layers: int = 48, *, batch: int = 1, T: int = 16, Hk: int =
         steps = int(torch.randint(0, T + 1, (1,), generator=g, device=device).item())
     st = torch.full((L * B,), int(steps), dtype=torch.int32, device=device)
     return ReplayCase(state, tape, k, gate, st)
+
+
+@dataclass
+class MoeCase:
+    x: torch.Tensor           # [P, K] rows already gathered per (token, expert) pair
+    expert_ids: torch.Tensor  # [P] int32
+    w: torch.Tensor           # [E, N, K/8] int32 words
+    scales: torch.Tensor      # [E, N, K/gs]
+    biases: torch.Tensor      # [E, N, K/gs]
+    group_size: int
+
+    def to(self, device) -> "MoeCase":
+        return MoeCase(self.x.to(device), self.expert_ids.to(device), self.w.to(device),
+                       self.scales.to(device), self.biases.to(device), self.group_size)
+
+
+def make_moe_case(K: int, N: int, seed: int, *, experts: int = 256, tokens: int = 16, top_k: int = 8,
+                  group_size: int = GROUP_SIZE, device: Union[str, torch.device] = "cpu") -> MoeCase:
+    """BASELINE config[4] routing: softmax over router logits ~ N(0,1), top-k experts per
+    token; one row per (token, expert) pair, token-major."""
+    g = _gen(seed, device)
+    logits = torch.randn((tokens, experts), generator=g, device=device, dtype=torch.float32)
+    ids = torch.topk(torch.softmax(logits, dim=-1), top_k, dim=-1).indices.to(torch.int32).reshape(-1)
+    x = torch.randn((tokens * top_k, K), generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    w = torch.randint(-2 ** 31, 2 ** 31, (experts, N, K // 8), generator=g, device=device, dtype=torch.int32)
+    s = ((torch.randn((experts, N, K // group_size), generator=g, device=device, dtype=torch.float32) * 0.02).abs()
+         + 1e-4).to(torch.bfloat16)
+    b = (-8.0 * s.to(torch.float32)).to(torch.bfloat16)
+    return MoeCase(x, ids, w, s, b, group_size)

@@ -83,6 +83,22 @@ int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* scales, const
                    int act_dtype, int sb_dtype, int variant, int k_parts, int kernel, void* stream);
 
 /*
+ * Gathered per-expert M<=16-per-expert qmm for MoE layers: y[p,:] = x[p,:] . (s*q + b)^T of
+ * expert expert_ids[p].  No counterpart in the reference tree: its MoE experts go through
+ * mlx_lm's switch layers (third-party `mx.gather_qmm`), which `install_verify_linears`
+ * (dflash_mlx/verify_linear.py:160) never swaps.  Rows of an expert are handled 16 at a time
+ * as one MFMA tile; experts without rows cost one early-exit workgroup per column block.
+ *
+ *   x [P, K] act_dtype      expert_ids [P] int32 in [0, E)
+ *   w_q [E, N, K/8] uint32  scales, biases [E, N, K/group_size] sb_dtype     y [P, N] act_dtype
+ * Requirements: P <= 2048, group_size in {32,64,128}, N % 16 == 0, K % group_size == 0.
+ * Rows whose expert id is outside [0, E) are left unwritten.
+ */
+int dflash_qmm_m16_gather(const void* x, const int32_t* expert_ids, const uint32_t* w_q,
+                          const void* scales, const void* biases, void* y, int P, int K, int N,
+                          int E, int group_size, int act_dtype, int sb_dtype, void* stream);
+
+/*
  * GatedDeltaNet tape replay: for every slot s and value head hv apply the first
  * steps[s] recorded steps to the recurrent state,
  *     S[dv][dk] <- g_t * S[dv][dk] + k_t[dk] * delta_t[dv],   t = 0 .. steps[s]-1,
