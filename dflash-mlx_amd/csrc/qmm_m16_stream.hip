@@ -16,12 +16,12 @@
 //    (96 KiB per CU) in flight while the fifth is consumed - HBM latency times bandwidth
 //    is ~100 KiB per CU on this part.  Granules are XOR-swizzled inside a row so that the
 //    MFMA-shaped reads spread evenly over the LDS banks.
-//  * Work every wave would otherwise repeat is done once per unit, one unit ahead, by
-//    waves 0-3: putting the x fragments into MFMA slot order (in place) and the per-group
-//    row sums of x (an MFMA against ones, already in accumulator layout).
-//  * Within a unit, wave w owns rows 16w..16w+15 (one MFMA tile) for all four
-//    quantisation groups, so its accumulators never need a cross-wave reduction and a
-//    finished row block goes from registers straight to memory.
+//  * Within a unit, wave w works on ONE quantisation group (w & 3) for 64 rows (four MFMA
+//    tiles, rows 64*(w >> 2) ..): the x fragments and the row sums of x (an MFMA against
+//    ones, already in accumulator layout) are then shared by its four tiles, which keeps
+//    the LDS read traffic per unit at a quarter of what "one tile, all groups" costs.  The
+//    four waves that cover the same rows add their accumulators through LDS only when a
+//    row block ends; after that wave w holds tile w and writes it out.
 //  * A workgroup whose range covers all of K for a row block writes y directly.
 //    Row blocks shared between workgroups go through fp32 partial tiles in the
 //    workspace; the last contributor to arrive (wrapping agent-scope counter)
@@ -35,13 +35,15 @@
 // through hand-written instruction blocks and synchronises with a bare s_barrier plus
 // an explicit vmcnt wait (loads retire in issue order and every wave issues the same
 // number of them per unit: one for x, two for codes, plus one with each scale/bias chunk).
+// The row-block epilogue (a few times per workgroup) uses ordinary code.
 #include "dflash_common.h"
 
 namespace dflash {
 namespace stream {
 
-constexpr int kWaves = 8;
-constexpr int kThreads = kWaves * 64;
+constexpr int kWaves = 8;  // arithmetic waves
+constexpr int kLoaders = 4;  // extra waves that only issue loads
+constexpr int kThreads = (kWaves + kLoaders) * 64;
 constexpr int kRows = 128;   // rows per unit (16 per wave)
 constexpr int kUnitK = 256;  // k per unit (four groups of 64)
 constexpr int kGS = 64;
@@ -51,9 +53,6 @@ constexpr int kWBytes = kRows * (kUnitK / 2);  // 16 KiB: 128 B per row
 constexpr int kXBytes = 16 * kUnitK * 2;       // 8 KiB
 constexpr int kXOffset = kWBytes;
 constexpr int kSlotBytes = kWBytes + kXBytes;  // 24 KiB
-// row sums of x per group in accumulator layout, for the unit in use and the next one
-constexpr int kXsBytes = kGroups * 64 * 16;    // 4 KiB
-constexpr int kXsOffset = kDepth * kSlotBytes;
 // Scales and biases are staged per chunk of kChunk units (32 bytes per row and array):
 // fetching them unit by unit would cost two 8-byte requests per row and unit, twice the
 // number of memory requests the codes themselves need.
@@ -61,8 +60,8 @@ constexpr int kChunk = 4;
 constexpr int kSbDepth = 3;
 constexpr int kSbArrayBytes = kRows * kChunk * kGroups * 2;  // 4 KiB
 constexpr int kSbSlotBytes = 2 * kSbArrayBytes;              // scales then biases
-constexpr int kSbOffset = kXsOffset + 2 * kXsBytes;
-constexpr int kLdsBytes = kSbOffset + kSbDepth * kSbSlotBytes;  // 152 KiB
+constexpr int kSbOffset = kDepth * kSlotBytes;
+constexpr int kLdsBytes = kSbOffset + kSbDepth * kSbSlotBytes;  // 144 KiB
 constexpr int kPartialFloats = 16 * kRows;
 
 template <bool FP16>
@@ -126,71 +125,122 @@ typedef __attribute__((address_space(1))) const void global_cvoid_t;
 __device__ __forceinline__ void load16_to_lds(const void* gptr, char* lds_base) {
   __builtin_amdgcn_global_load_lds((global_cvoid_t*)gptr, (lds_void_t*)lds_base, 16, 0, 0);
 }
+// The same with the non-temporal cache policy (aux bit 1 = nt on gfx94x/gfx950): the codes
+// are read exactly once, so they should not push x and the scale/bias lines, which are
+// re-read, out of the L2.
+__device__ __forceinline__ void load16_to_lds_stream(const void* gptr, char* lds_base) {
+  __builtin_amdgcn_global_load_lds((global_cvoid_t*)gptr, (lds_void_t*)lds_base, 16, 0, 2);
+}
 
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(uintptr_t)(const lds_void_t*)p;
 }
 
-// Preparation of one group of the next unit (waves 0-3): fragments j = 0, 1 of this lane
-// are put into MFMA slot order in place, and the group's row sums of x land in `xs_addr`.
-template <bool FP16>
-__device__ __forceinline__ void prepare_group(uint32_t frag_addr, uint32_t xs_addr, uint4 ones) {
+// One unit's operands of a worker wave (group g, rows 64h + 16j + col for tiles j = 0..3):
+//   f0, f1  x fragments (natural order) feeding MFMA 0 / 1
+//   wq[j]   packed codes of tile j: .x feeds MFMA 0, .y MFMA 1
+//   sv, bv  scale / bias of this lane's row in tile j, 16 bits zero-extended
+struct Operands {
   u32x4_t f0, f1;
-  asm volatile(
-      "ds_read_b128 %0, %2\n"
-      "ds_read_b128 %1, %2 offset:256\n"
-      "s_waitcnt lgkmcnt(0)\n"
-      : "=&v"(f0), "=&v"(f1)
-      : "v"(frag_addr)
-      : "memory");
-  const u32x4_t a0 = permute_x(f0), a1 = permute_x(f1);
-  f32x4_t xs = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  xs = Act<FP16>::mfma(as_uint4(a0), ones, xs);
-  xs = Act<FP16>::mfma(as_uint4(a1), ones, xs);
-  asm volatile(
-      "ds_write_b128 %0, %2\n"
-      "ds_write_b128 %0, %3 offset:256\n"
-      "ds_write_b128 %1, %4\n"
-      :
-      : "v"(frag_addr), "v"(xs_addr), "v"(a0), "v"(a1), "v"(xs)
-      : "memory");
-}
-
-// One unit's operands of a wave.  Completion of the unit is established by the caller.
-//   af[2g+j] x fragment (slot order) feeding MFMA j of group g
-//   xs[g]    row sums of x over group g, accumulator layout
-//   wq[g]    packed codes of group g: .x feeds MFMA 0, .y MFMA 1
-//   sc, bi   the four scales / biases of this lane's row, two 16-bit values per dword
-__device__ __forceinline__ void read_unit_operands(uint32_t xaddr, uint32_t xsaddr,
-                                                   const uint32_t (&waddr)[4], uint32_t saddr,
-                                                   u32x4_t (&af)[8], f32x4_t (&xs)[4],
-                                                   u32x2_t (&wq)[4], u32x2_t& sc, u32x2_t& bi) {
+  u32x2_t wq[4];
+  uint32_t sv[4], bv[4];
+};
+// Starts the LDS reads of a unit's operands and returns at once: the registers of `o` are
+// written behind the compiler's back until operands_wait(o) has been executed, so nothing
+// may touch `o` in between.  `acc` is threaded through both so that the arithmetic on the
+// previous unit, which ends in `acc`, stays between the two.
+__device__ __forceinline__ void operands_issue(uint32_t xaddr, uint32_t waddr, uint32_t saddr,
+                                               Operands& o, f32x4_t& acc0, f32x4_t& acc1,
+                                               f32x4_t& acc2, f32x4_t& acc3) {
   asm volatile(
       "ds_read_b128 %0, %18\n"
       "ds_read_b128 %1, %18 offset:256\n"
-      "ds_read_b128 %2, %18 offset:2048\n"
-      "ds_read_b128 %3, %18 offset:2304\n"
-      "ds_read_b128 %4, %18 offset:4096\n"
-      "ds_read_b128 %5, %18 offset:4352\n"
-      "ds_read_b128 %6, %18 offset:6144\n"
-      "ds_read_b128 %7, %18 offset:6400\n"
-      "ds_read_b64 %12, %20\n"
-      "ds_read_b64 %13, %21\n"
-      "ds_read_b64 %14, %22\n"
-      "ds_read_b64 %15, %23\n"
-      "ds_read_b64 %16, %24\n"
-      "ds_read_b64 %17, %24 offset:4096\n"
-      "ds_read_b128 %8, %19\n"
-      "ds_read_b128 %9, %19 offset:1024\n"
-      "ds_read_b128 %10, %19 offset:2048\n"
-      "ds_read_b128 %11, %19 offset:3072\n"
-      "s_waitcnt lgkmcnt(0)\n"
-      : "=&v"(af[0]), "=&v"(af[1]), "=&v"(af[2]), "=&v"(af[3]), "=&v"(af[4]), "=&v"(af[5]),
-        "=&v"(af[6]), "=&v"(af[7]), "=&v"(xs[0]), "=&v"(xs[1]), "=&v"(xs[2]), "=&v"(xs[3]),
-        "=&v"(wq[0]), "=&v"(wq[1]), "=&v"(wq[2]), "=&v"(wq[3]), "=&v"(sc), "=&v"(bi)
-      : "v"(xaddr), "v"(xsaddr), "v"(waddr[0]), "v"(waddr[1]), "v"(waddr[2]), "v"(waddr[3]),
-        "v"(saddr)
+      "ds_read_b64 %2, %19\n"
+      "ds_read_b64 %3, %19 offset:2048\n"
+      "ds_read_b64 %4, %19 offset:4096\n"
+      "ds_read_b64 %5, %19 offset:6144\n"
+      "ds_read_u16 %6, %20\n"
+      "ds_read_u16 %10, %20 offset:4096\n"
+      "ds_read_u16 %7, %20 offset:512\n"
+      "ds_read_u16 %11, %20 offset:4608\n"
+      "ds_read_u16 %8, %20 offset:1024\n"
+      "ds_read_u16 %12, %20 offset:5120\n"
+      "ds_read_u16 %9, %20 offset:1536\n"
+      "ds_read_u16 %13, %20 offset:5632\n"
+      : "=&v"(o.f0), "=&v"(o.f1), "=&v"(o.wq[0]), "=&v"(o.wq[1]), "=&v"(o.wq[2]), "=&v"(o.wq[3]),
+        "=&v"(o.sv[0]), "=&v"(o.sv[1]), "=&v"(o.sv[2]), "=&v"(o.sv[3]),
+        "=&v"(o.bv[0]), "=&v"(o.bv[1]), "=&v"(o.bv[2]), "=&v"(o.bv[3]),
+        "+v"(acc0), "+v"(acc1), "+v"(acc2), "+v"(acc3)
+      : "v"(xaddr), "v"(waddr), "v"(saddr)
       : "memory");
+}
+__device__ __forceinline__ void operands_wait(Operands& o, f32x4_t& acc0, f32x4_t& acc1,
+                                              f32x4_t& acc2, f32x4_t& acc3) {
+  asm volatile("s_waitcnt lgkmcnt(0)\n"
+               : "+v"(o.f0), "+v"(o.f1), "+v"(o.wq[0]), "+v"(o.wq[1]), "+v"(o.wq[2]), "+v"(o.wq[3]),
+                 "+v"(o.sv[0]), "+v"(o.sv[1]), "+v"(o.sv[2]), "+v"(o.sv[3]),
+                 "+v"(o.bv[0]), "+v"(o.bv[1]), "+v"(o.bv[2]), "+v"(o.bv[3]),
+                 "+v"(acc0), "+v"(acc1), "+v"(acc2), "+v"(acc3)
+               :
+               : "memory");
+}
+
+// The arithmetic of one unit: acc[j] += (scale, bias)-corrected x . codes^T of tile j.
+template <bool ACT_FP16, bool SB_FP16>
+__device__ __forceinline__ void consume_unit(const Operands& o, f32x4_t (&acc)[4], uint4 ones,
+                                             uint32_t mask, uint32_t magic) {
+  using A = Act<ACT_FP16>;
+  using SB = Act<SB_FP16>;
+  const uint4 a0 = as_uint4(permute_x(o.f0)), a1 = as_uint4(permute_x(o.f1));
+  f32x4_t xs = f32x4_t{0.f, 0.f, 0.f, 0.f};  // row sums of x over this group
+  xs = A::mfma(a0, ones, xs);
+  xs = A::mfma(a1, ones, xs);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    f32x4_t c = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    c = A::mfma(a0, unpack_codes(o.wq[j].x, mask, magic), c);
+    c = A::mfma(a1, unpack_codes(o.wq[j].y, mask, magic), c);
+    const float s = SB::to_f32(o.sv[j]);
+    const float b = SB::to_f32(o.bv[j]);
+    const float bb = __builtin_fmaf(-A::kOffset, s, b);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[j][r] = __builtin_fmaf(bb, xs[r], __builtin_fmaf(s, c[r], acc[j][r]));
+  }
+}
+
+// Cross-wave sum at the end of a row block: every worker hands the three tiles it does
+// not own to their owners through `base` (24 KiB: 8 owners x 3 tiles x 1 KiB), and after
+// a barrier returns the sum of its own tile and the three it receives, in a fixed order.
+__device__ __forceinline__ void reduce_groups_write(uint32_t base, const f32x4_t (&acc)[4], int wave,
+                                                    int lane) {
+  const int g = wave & 3, h = wave >> 2;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (j != g) {
+      const int pos = (g - j - 1) & 3;  // 0..2
+      const uint32_t addr = base + ((4 * h + j) * 3 + pos) * 1024 + lane * 16;
+      asm volatile("ds_write_b128 %0, %1\n" : : "v"(addr), "v"(acc[j]) : "memory");
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+}
+__device__ __forceinline__ f32x4_t reduce_groups_read(uint32_t base, const f32x4_t (&acc)[4], int wave,
+                                                      int lane) {
+  const int g = wave & 3;
+  f32x4_t own = g == 0 ? acc[0] : g == 1 ? acc[1] : g == 2 ? acc[2] : acc[3];
+  f32x4_t v0, v1, v2;
+  const uint32_t addr = base + wave * 3 * 1024 + lane * 16;
+  asm volatile(
+      "ds_read_b128 %0, %3\n"
+      "ds_read_b128 %1, %3 offset:1024\n"
+      "ds_read_b128 %2, %3 offset:2048\n"
+      "s_waitcnt lgkmcnt(0)\n"
+      : "=&v"(v0), "=&v"(v1), "=&v"(v2)
+      : "v"(addr)
+      : "memory");
+#pragma unroll
+  for (int r = 0; r < 4; ++r) own[r] = ((own[r] + v0[r]) + v1[r]) + v2[r];
+  return own;
 }
 
 // Partial accumulator tiles cross XCDs: stored and loaded at agent scope (sc1).
@@ -231,17 +281,21 @@ __device__ __forceinline__ int range_begin(int units, int i, int n) {
 
 #define DFLASH_WAIT_CASE(n) \
   case n:                   \
-    __builtin_amdgcn_s_waitcnt(0x0070 | ((n)&15) | (((n) >> 4) << 14)); \
+    __builtin_amdgcn_s_waitcnt(0x0F70 | ((n)&15) | (((n) >> 4) << 14)); \
     break;
-// Wait until at most n of this wave's loads are outstanding and all its LDS traffic is done.
+// Wait until at most n of this wave's loads are outstanding (loads retire in issue order).
 __device__ __forceinline__ void wait_loads(int n) {
   switch (n) {
     DFLASH_WAIT_CASE(0) DFLASH_WAIT_CASE(1) DFLASH_WAIT_CASE(2) DFLASH_WAIT_CASE(3)
     DFLASH_WAIT_CASE(4) DFLASH_WAIT_CASE(5) DFLASH_WAIT_CASE(6) DFLASH_WAIT_CASE(7)
     DFLASH_WAIT_CASE(8) DFLASH_WAIT_CASE(9) DFLASH_WAIT_CASE(10) DFLASH_WAIT_CASE(11)
     DFLASH_WAIT_CASE(12) DFLASH_WAIT_CASE(13) DFLASH_WAIT_CASE(14) DFLASH_WAIT_CASE(15)
-    DFLASH_WAIT_CASE(16)
-    default: __builtin_amdgcn_s_waitcnt(0x0070); break;
+    DFLASH_WAIT_CASE(16) DFLASH_WAIT_CASE(17) DFLASH_WAIT_CASE(18) DFLASH_WAIT_CASE(19)
+    DFLASH_WAIT_CASE(20) DFLASH_WAIT_CASE(21) DFLASH_WAIT_CASE(22) DFLASH_WAIT_CASE(23)
+    DFLASH_WAIT_CASE(24) DFLASH_WAIT_CASE(25) DFLASH_WAIT_CASE(26) DFLASH_WAIT_CASE(27)
+    DFLASH_WAIT_CASE(28) DFLASH_WAIT_CASE(29) DFLASH_WAIT_CASE(30) DFLASH_WAIT_CASE(31)
+    DFLASH_WAIT_CASE(32)
+    default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
   }
 }
 #undef DFLASH_WAIT_CASE
@@ -249,222 +303,275 @@ __device__ __forceinline__ void wait_loads(int n) {
 template <bool ACT_FP16, bool SB_FP16>
 __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
   using A = Act<ACT_FP16>;
-  using SB = Act<SB_FP16>;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  __shared__ int s_last;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int col = lane & 15;
-  const int kblk = lane >> 4;
-  const int G = p.K / kGS;
-  const size_t row_bytes = (size_t)p.K >> 1;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int grid = gridDim.x;
+  const uint32_t lds0 = lds_address(lds);
 
   const int u0 = range_begin(p.units, blockIdx.x, grid);
   const int u1 = range_begin(p.units, blockIdx.x + 1, grid);
   if (u0 >= u1) return;
+  const int rb0 = u0 / p.stages, st0 = u0 - rb0 * p.stages;
 
-  // ---- producer state ---------------------------------------------------------------
-  //  codes: 16 instructions cover 128 rows x 128 B; instruction q = wave + 8*i holds rows
-  //         8q..8q+7; lane = 8*row_in_8 + slot, and slot holds granule slot ^ sw(row) with
-  //         sw(row) = ((row >> 1) & 3) << 1  (swaps 32-byte pairs, i.e. whole groups)
-  //  x:     wave w moves group w>>1, k-blocks 2*(w&1) and 2*(w&1)+1: lane = 16*(2*kbl + j) + m
-  //         fetches x[m][64g + 16*(2*(w&1) + kbl) + 8j .. +7], 64 contiguous bytes per row
-  //  scales/biases of a chunk: waves 0-3 scales, 4-7 biases, 32 rows per wave, two
-  //         16-byte granules per row
-  const int w_r = lane >> 3;
-  const int w_c = (lane & 7) ^ (((w_r >> 1) & 3) << 1);
-  const char* const xp0 = (const char*)(p.x + (size_t)(lane & 15) * p.K + (wave >> 1) * kGS +
-                                        (2 * (wave & 1) + (lane >> 5)) * 16 + ((lane >> 4) & 1) * 8);
-  const char* wp[2];   // codes of this lane's rows at stage 0 of the row block being issued
-  const char* sbp;     // scales or biases of this lane's row, chunk 0
-  auto set_row_block = [&](int rb) {
-    const int row0 = rb * kRows;
+  // Both kinds of wave walk the same units and pass the same barriers:
+  //   one before the loop (unit u0 has landed),
+  //   one per unit u (unit u+1 has landed; every worker holds unit u in registers, so the
+  //     slot of unit u is free),
+  //   when a row block ends with unit u: one more (the slot of unit u carries the cross-wave
+  //     sum), and two more if other workgroups share the row block (partial tile stored /
+  //     arrival counter bumped).
+
+  if (wave >= kWaves) {
+    // ================================ loader waves ====================================
+    //  codes: 16 instructions cover 128 rows x 128 B; instruction q holds rows 8q..8q+7,
+    //         lane = 8*row_in_8 + slot, and slot holds granule slot ^ sw(row) with
+    //         sw(row) = ((row >> 1) & 3) << 1  (swaps 32-byte pairs, i.e. whole groups);
+    //         loader l issues q = l, l+4, l+8, l+12
+    //  x:     8 instructions; instruction i moves group i>>1, k-blocks 2*(i&1) and 2*(i&1)+1:
+    //         lane = 16*(2*kbl + j) + m fetches x[m][64g + 16*(2*(i&1) + kbl) + 8j .. +7],
+    //         64 contiguous bytes per row; loader l issues i = l, l+4
+    //  scales/biases of a chunk: 4 + 4 instructions of 32 rows, two 16-byte granules per
+    //         row; loader l issues scales and biases of rows 32l..32l+31
+    const int ld = wave - kWaves;
+    const int G = p.K / kGS;
+    const size_t row_bytes = (size_t)p.K >> 1;
+    const int w_r = lane >> 3;
+    const int w_c = (lane & 7) ^ (((w_r >> 1) & 3) << 1);
+    const char* xp[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      int row = row0 + 8 * (wave + kWaves * i) + w_r;
+      const int xi = ld + 4 * i;
+      xp[i] = (const char*)(p.x + (size_t)(lane & 15) * p.K + (xi >> 1) * kGS +
+                            (2 * (xi & 1) + (lane >> 5)) * 16 + ((lane >> 4) & 1) * 8);
+    }
+    const char* wp[4];   // codes of this lane's rows at stage 0 of the row block being issued
+    const char* sbp[2];  // scales, biases of this lane's row, chunk 0
+    auto set_row_block = [&](int rb) __attribute__((always_inline)) {
+      const int row0 = rb * kRows;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int row = row0 + 8 * (ld + 4 * i) + w_r;
+        row = row < p.N ? row : p.N - 1;
+        wp[i] = (const char*)p.w + (size_t)row * row_bytes + w_c * 16;
+      }
+      int row = row0 + 32 * ld + (lane >> 1);
       row = row < p.N ? row : p.N - 1;
-      wp[i] = (const char*)p.w + (size_t)row * row_bytes + w_c * 16;
-    }
-    int row = row0 + 32 * (wave & 3) + (lane >> 1);
-    row = row < p.N ? row : p.N - 1;
-    sbp = (const char*)(((wave & 4) ? p.biases : p.scales) + (size_t)row * G) + (lane & 1) * 16;
-  };
+      sbp[0] = (const char*)(p.scales + (size_t)row * G) + (lane & 1) * 16;
+      sbp[1] = (const char*)(p.biases + (size_t)row * G) + (lane & 1) * 16;
+    };
 
-  int rb_i = u0 / p.stages, st_i = u0 - rb_i * p.stages;  // next unit to issue
-  int issued = u0;
-  int slot_i = 0;     // ring slot of the next unit to issue
-  int sb_slot_i = 0;  // scale/bias slot of the next chunk to issue
-  set_row_block(rb_i);
-  // Issues one unit (x first, so that x of unit u+1 can be awaited without its codes);
-  // returns the number of loads this wave issued for it.
-  auto issue_next = [&]() -> int {
-    char* slot = lds + slot_i * kSlotBytes;
-    int n = 3;
-    load16_to_lds(xp0 + (size_t)st_i * (kUnitK * 2), slot + kXOffset + wave * 1024);
-    if ((st_i % kChunk) == 0 || issued == u0) {
-      load16_to_lds(sbp + (size_t)(st_i / kChunk) * (kChunk * kGroups * 2),
-                    lds + kSbOffset + sb_slot_i * kSbSlotBytes + ((wave & 4) ? kSbArrayBytes : 0) +
-                        (wave & 3) * 1024);
-      if (++sb_slot_i == kSbDepth) sb_slot_i = 0;
-      n = 4;
-    }
-    load16_to_lds(wp[0] + (size_t)st_i * (kUnitK / 2), slot + wave * 1024);
-    load16_to_lds(wp[1] + (size_t)st_i * (kUnitK / 2), slot + (wave + kWaves) * 1024);
-    ++issued;
-    if (++slot_i == kDepth) slot_i = 0;
-    if (++st_i == p.stages) {
-      st_i = 0;
-      ++rb_i;
-      if (issued < u1) set_row_block(rb_i);
-    }
-    return n;
-  };
+    int rb_i = rb0, st_i = st0;  // next unit to issue
+    int issued = u0;
+    int slot_i = 0;     // ring slot of the next unit to issue
+    int sb_slot_i = 0;  // scale/bias slot of the next chunk to issue
+    set_row_block(rb_i);
+    // Issues one unit: 6 loads (2 for x, 4 for codes), plus 2 with the first unit of every
+    // scale/bias chunk and with the first unit of the range.
+    auto issue_next = [&]() __attribute__((always_inline)) {
+      char* slot = lds + slot_i * kSlotBytes;
+      if ((st_i % kChunk) == 0 || issued == u0) {
+        char* sb = lds + kSbOffset + sb_slot_i * kSbSlotBytes + ld * 1024;
+        const size_t off = (size_t)(st_i / kChunk) * (kChunk * kGroups * 2);
+        load16_to_lds(sbp[0] + off, sb);
+        load16_to_lds(sbp[1] + off, sb + kSbArrayBytes);
+        if (++sb_slot_i == kSbDepth) sb_slot_i = 0;
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        load16_to_lds(xp[i] + (size_t)st_i * (kUnitK * 2), slot + kXOffset + (ld + 4 * i) * 1024);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        load16_to_lds_stream(wp[i] + (size_t)st_i * (kUnitK / 2), slot + (ld + 4 * i) * 1024);
+      ++issued;
+      if (++slot_i == kDepth) slot_i = 0;
+      if (++st_i == p.stages) {
+        st_i = 0;
+        ++rb_i;
+        if (issued < u1) set_row_block(rb_i);
+      }
+    };
+    // Loads this loader has issued for units u0..v.  Unit indices are global and the number
+    // of stages is a multiple of kChunk, so a unit starts a chunk iff its index is one.
+    auto loads_through = [&](int v) __attribute__((always_inline)) -> int {
+      return 6 * (v - u0 + 1) + 2 * (1 + (v / kChunk) - (u0 / kChunk));
+    };
+    // Waits until this loader's part of unit v has landed (loads retire in issue order).
+    auto wait_unit = [&](int v) __attribute__((always_inline)) {
+      wait_loads(loads_through(issued - 1) - loads_through(v));
+    };
 
-  // ---- consumer state ---------------------------------------------------------------
+    for (int i = 0; i < kDepth && issued < u1; ++i) issue_next();
+    wait_unit(u0);
+    asm volatile("s_barrier" ::: "memory");
+    int rb_left = p.stages - st0;  // units of the current row block from unit u on
+    int in_rb = 0;                 // units of the current row block this workgroup has done
+#pragma unroll 1
+    for (int u = u0; u < u1; ++u) {
+      const bool rb_ends = rb_left == 1 || u + 1 == u1;
+      if (u + 1 < u1) wait_unit(u + 1);
+      asm volatile("s_barrier" ::: "memory");
+      // the slot of unit u takes unit u+5 - unless a row block ends here: then it first
+      // carries the cross-wave sum and is refilled one unit later
+      const int limit = rb_ends ? u + kDepth - 1 : u + kDepth;
+      while (issued <= limit && issued < u1) issue_next();
+      ++in_rb;
+      --rb_left;
+      if (rb_ends) {
+        asm volatile("s_barrier" ::: "memory");
+        if (in_rb != p.stages) {
+          asm volatile("s_barrier" ::: "memory");
+          asm volatile("s_barrier" ::: "memory");
+        }
+        in_rb = 0;
+        rb_left = p.stages;
+      }
+    }
+    return;
+  }
+
+  // ================================== worker waves ====================================
+  const int col = lane & 15;
+  const int kblk = lane >> 4;
   const uint4 ones = make_uint4(A::kOnes, A::kOnes, A::kOnes, A::kOnes);
   uint32_t mask = 0x000F000Fu, magic = A::kMagic;
   asm volatile("" : "+s"(mask), "+v"(magic));
-  const uint32_t lds0 = lds_address(lds);
-  //   x fragment (g, j) of lane (m = col, kb = kblk) inside a slot: + g*2048 + j*256
-  const uint32_t xoff = kXOffset + (kblk >> 1) * 1024 + (16 * (2 * (kblk & 1)) + col) * 16;
-  const uint32_t wrow = 16 * wave + col;
-  uint32_t woff[4];
-#pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    // group g of this row sits in the 32-byte pair g ^ ((row >> 1) & 3)
-    woff[g] = wrow * 128 + ((g ^ ((wrow >> 1) & 3)) << 5) + (kblk >> 1) * 16 + (kblk & 1) * 8;
-  }
-  int rb = u0 / p.stages, st = u0 - rb * p.stages;  // unit being consumed
-  const int rb_first = rb;
-  int first_in_rb = u0;
-  int slot_c = 0;      // ring slot of the unit being consumed
-  int sb_slot_c = -1;  // scale/bias slot of the chunk being consumed
-  int xs_c = 0;        // which row-sum buffer belongs to the unit being consumed
-  f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int grp = wave & 3;   // quantisation group of the unit this wave works on
+  const int half = wave >> 2; // rows 64*half .. 64*half + 63: tiles j = 0..3
+  //   x fragment j of lane (m = col, kb = kblk) for group grp inside a slot: + j*256
+  const uint32_t xoff =
+      lds0 + kXOffset + grp * 2048 + (kblk >> 1) * 1024 + (16 * (2 * (kblk & 1)) + col) * 16;
+  // codes of row 64*half + 16j + col: group grp sits in the 32-byte pair grp ^ ((row >> 1) & 3),
+  // which does not depend on j; tile j is 2 KiB further
+  const uint32_t wrow = 64 * half + col;
+  const uint32_t woff =
+      lds0 + wrow * 128 + ((grp ^ ((wrow >> 1) & 3)) << 5) + (kblk >> 1) * 16 + (kblk & 1) * 8;
+  // scale of that row: 32 bytes per row and chunk, four 16-bit values per unit; tile j is
+  // 512 bytes further, biases one array further
+  const uint32_t soff = lds0 + kSbOffset + wrow * 32 + grp * 2;
 
-  // waves 0-3: prepare group `wave` of the unit in ring slot s, row sums into buffer b
-  auto prepare = [&](int s, int b) {
-    if (wave < 4) {
-      prepare_group<ACT_FP16>(lds0 + s * kSlotBytes + xoff + wave * 2048,
-                              lds0 + kXsOffset + b * kXsBytes + wave * 1024 + lane * 16, ones);
+  // reading position: the unit whose operands are fetched next
+  int rd_slot = 0;   // byte offset of its ring slot
+  int rd_sb = -kSbSlotBytes;  // byte offset of its scale/bias slot
+  int rd_q = st0 % kChunk;    // its stage within the chunk
+  bool rd_first = true;
+  f32x4_t acc4[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc4[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  Operands op[2];
+
+  auto start_operands = [&](Operands& o) __attribute__((always_inline)) {
+    if (rd_q == 0 || rd_first) {
+      rd_sb += kSbSlotBytes;
+      if (rd_sb == kSbDepth * kSbSlotBytes) rd_sb = 0;
+      rd_first = false;
     }
+    operands_issue(xoff + rd_slot, woff + rd_slot, soff + rd_sb + rd_q * 8, o, acc4[0], acc4[1],
+                   acc4[2], acc4[3]);
+    rd_slot += kSlotBytes;
+    if (rd_slot == kDepth * kSlotBytes) rd_slot = 0;
+    rd_q = (rd_q + 1) & (kChunk - 1);
   };
 
-  // ---- prologue: fill the ring, prepare the first unit ------------------------------
-  // y1..y3: loads this wave issued for the three units after the one being consumed
-  int y1 = 0, y2 = 0, y3 = 0;
-  const int n0 = issue_next();
-  if (issued < u1) y1 = issue_next();
-  if (issued < u1) y2 = issue_next();
-  if (issued < u1) y3 = issue_next();
-  wait_loads(n0 - 1 + y1 + y2 + y3);  // x of the first unit is the oldest load
   asm volatile("s_barrier" ::: "memory");
-  prepare(0, 0);
+  start_operands(op[0]);
+  operands_wait(op[0], acc4[0], acc4[1], acc4[2], acc4[3]);
+
+  int left = u1 - u0;            // units still to consume, the current one included
+  int rb_left = p.stages - st0;  // same, within the current row block
+  int in_rb = 0;                 // units of the current row block this workgroup has done
+  int rb = rb0;
+  int cur_slot = 0;              // byte offset of the current unit's ring slot
 
 #pragma unroll 1
-  for (int u = u0; u < u1; ++u) {
-    // unit u and the x slice of unit u+1 (the oldest load of that unit) must have landed
-    wait_loads(y1 + y2 + y3 - (y1 ? 1 : 0));
-    asm volatile("s_barrier" ::: "memory");  // ... for every wave; unit u-1 is consumed
-    y1 = y2, y2 = y3, y3 = 0;
-    if (issued < u1) y3 = issue_next();  // unit u+4 refills the slot of unit u-1
-    if (u + 1 < u1) prepare(slot_c + 1 == kDepth ? 0 : slot_c + 1, xs_c ^ 1);
-    if ((st % kChunk) == 0 || u == u0) {
-      if (++sb_slot_c == kSbDepth) sb_slot_c = 0;
-    }
-
-    const uint32_t sbase = lds0 + slot_c * kSlotBytes;
-    if (++slot_c == kDepth) slot_c = 0;
-    // four scales of this lane's row for this unit; biases one array further
-    const uint32_t saddr = lds0 + kSbOffset + sb_slot_c * kSbSlotBytes + wrow * 32 + (st % kChunk) * 8;
-    const uint32_t xsaddr = lds0 + kXsOffset + xs_c * kXsBytes + lane * 16;
-    xs_c ^= 1;
-    u32x4_t af[8];
-    f32x4_t xs[4];
-    u32x2_t wq[4], sc, bi;
-    const uint32_t waddr[4] = {sbase + woff[0], sbase + woff[1], sbase + woff[2], sbase + woff[3]};
-    read_unit_operands(sbase + xoff, xsaddr, waddr, saddr, af, xs, wq, sc, bi);
-
+  while (true) {
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      f32x4_t c = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      c = A::mfma(as_uint4(af[2 * g]), unpack_codes(wq[g].x, mask, magic), c);
-      c = A::mfma(as_uint4(af[2 * g + 1]), unpack_codes(wq[g].y, mask, magic), c);
-      const uint32_t sd = (g & 2) ? sc.y : sc.x;
-      const uint32_t bd = (g & 2) ? bi.y : bi.x;
-      const float s = SB::to_f32((g & 1) ? (sd >> 16) : (sd & 0xFFFFu));
-      const float b = SB::to_f32((g & 1) ? (bd >> 16) : (bd & 0xFFFFu));
-      const float bb = __builtin_fmaf(-A::kOffset, s, b);
+    for (int par = 0; par < 2; ++par) {
+      Operands& cur = op[par];
+      Operands& nxt = op[par ^ 1];
+      asm volatile("s_barrier" ::: "memory");
+      if (left > 1) start_operands(nxt);
+      consume_unit<ACT_FP16, SB_FP16>(cur, acc4, ones, mask, magic);
+      if (left > 1) operands_wait(nxt, acc4[0], acc4[1], acc4[2], acc4[3]);
+      --left;
+      ++in_rb;
+      if (--rb_left == 0 || left == 0) {
+        // ---- a row block ends inside my range: emit it -----------------------------------
+        const uint32_t sbase = lds0 + cur_slot;
+        reduce_groups_write(sbase, acc4, wave, lane);
+        asm volatile("s_barrier" ::: "memory");
+        f32x4_t acc = reduce_groups_read(sbase, acc4, wave, lane);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf(bb, xs[g][r], __builtin_fmaf(s, c[r], acc[r]));
-    }
-
-    // ---- advance; emit when this row block ends inside my range -------------------
-    const int cur_rb = rb;
-    const bool rb_ends = (u + 1 == u1) || (st + 1 == p.stages);
-    if (++st == p.stages) {
-      st = 0;
-      ++rb;
-    }
-    if (!rb_ends) continue;
-
-    const int lo = cur_rb * p.stages;
-    const bool complete = (first_in_rb == lo) && (u + 1 == lo + p.stages);
-    const int row0 = cur_rb * kRows;
-    first_in_rb = u + 1;
-    // accumulator r of lane l is output (m = 4*(l/16) + r, n = row0 + 16*wave + l%16)
-    const int n_out = row0 + 16 * wave + col;
-    if (!complete) {
-      // a workgroup shares at most two row blocks with others: the one its range starts in
-      // (slot 0) and the one it ends in (slot 1); tiles are kept in accumulator layout
-      float* part = p.partials + ((size_t)blockIdx.x * 2 + (cur_rb == rb_first ? 0 : 1)) * kPartialFloats;
-      store_partial(part + tid * 4, acc);
-      // The barrier's own wait (vmcnt(0)) retires every thread's store before thread 0
-      // bumps the counter; a release fence here would write back the whole L2.
-      __syncthreads();
-      // contributors: the workgroups whose ranges intersect [lo, lo+stages);
-      // owner(v) = ceil((v+1)*grid/units) - 1 is the workgroup whose range holds unit v
-      const int wg_first = (int)((((unsigned)lo + 1u) * (unsigned)grid + p.units - 1) / (unsigned)p.units) - 1;
-      const int wg_last =
-          (int)((((unsigned)(lo + p.stages)) * (unsigned)grid + p.units - 1) / (unsigned)p.units) - 1;
-      if (tid == 0) {
-        const uint32_t n_contrib = (uint32_t)(wg_last - wg_first + 1);
-        // wrapping increment: the last arrival sees n-1 and leaves 0 behind for the next call
-        const uint32_t prev = atomicInc(&p.counters[cur_rb], n_contrib - 1);
-        s_last = (prev == n_contrib - 1);
-      }
-      __syncthreads();
-      acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      if (!s_last) continue;
-      // only the first contributor can have started before this row block (then the block
-      // is the one its range ends in); every later one starts inside it
-      const int which_first = range_begin(p.units, wg_first, grid) < lo ? 1 : 0;
-      for (int wg = wg_first; wg <= wg_last; wg += 4) {
-        const float* src[4];
+        for (int j = 0; j < 4; ++j) acc4[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        bool emit = true;
+        if (in_rb != p.stages) {
+          // Other workgroups hold the rest of this row block.  A workgroup shares at most two
+          // row blocks: the one its range starts in (slot 0) and the one it ends in (slot 1);
+          // partial tiles are kept in accumulator layout.
+          const int lo = rb * p.stages;
+          float* part = p.partials + ((size_t)blockIdx.x * 2 + (rb == rb0 ? 0 : 1)) * kPartialFloats;
+          // contributors: the workgroups whose ranges intersect [lo, lo+stages);
+          // owner(v) = ceil((v+1)*grid/units) - 1 is the workgroup whose range holds unit v
+          const int wg_first = (int)((((unsigned)lo + 1u) * (unsigned)grid + p.units - 1) / (unsigned)p.units) - 1;
+          const int wg_last =
+              (int)((((unsigned)(lo + p.stages)) * (unsigned)grid + p.units - 1) / (unsigned)p.units) - 1;
+          store_partial(part + tid * 4, acc);
+          // every worker's store has been acknowledged before the barrier, hence before
+          // thread 0 bumps the counter; a release fence here would write back the whole L2
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          // (all workers have their received tiles in registers: the flag may reuse the slot)
+          asm volatile("s_barrier" ::: "memory");
+          if (tid == 0) {
+            const uint32_t n_contrib = (uint32_t)(wg_last - wg_first + 1);
+            // wrapping increment: the last arrival sees n-1 and leaves 0 behind for the next call
+            const uint32_t prev = atomicInc(&p.counters[rb], n_contrib - 1);
+            const uint32_t flag = (prev == n_contrib - 1) ? 1u : 0u;
+            asm volatile("ds_write_b32 %0, %1\n s_waitcnt lgkmcnt(0)" : : "v"(sbase), "v"(flag) : "memory");
+          }
+          asm volatile("s_barrier" ::: "memory");
+          uint32_t last;
+          asm volatile("ds_read_b32 %0, %1\n s_waitcnt lgkmcnt(0)" : "=v"(last) : "v"(sbase) : "memory");
+          emit = __builtin_amdgcn_readfirstlane(last) != 0;
+          if (emit) {
+            // only the first contributor can have started before this row block (then the
+            // block is the one its range ends in); every later one starts inside it
+            const int which_first = range_begin(p.units, wg_first, grid) < lo ? 1 : 0;
+            acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            for (int wg = wg_first; wg <= wg_last; wg += 4) {
+              const float* src[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int w = wg + j <= wg_last ? wg + j : wg_last;  // surplus slots re-read the last tile
-          src[j] = p.partials + ((size_t)w * 2 + (w == wg_first ? which_first : 0)) * kPartialFloats + tid * 4;
-        }
-        f32x4_t v[4];
-        load_partials4(src[0], src[1], src[2], src[3], v);
+              for (int j = 0; j < 4; ++j) {
+                const int w = wg + j <= wg_last ? wg + j : wg_last;  // surplus slots re-read the last tile
+                src[j] = p.partials + ((size_t)w * 2 + (w == wg_first ? which_first : 0)) * kPartialFloats + tid * 4;
+              }
+              f32x4_t v[4];
+              load_partials4(src[0], src[1], src[2], src[3], v);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (wg + j <= wg_last) {
+              for (int j = 0; j < 4; ++j) {
+                if (wg + j <= wg_last) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) acc[r] += v[j][r];
+                  for (int r = 0; r < 4; ++r) acc[r] += v[j][r];
+                }
+              }
+            }
           }
         }
-      }
-    }
-    if (n_out < p.N) {
+        // accumulator r of lane l is output (m = 4*(l/16) + r, n = row0 + 16*wave + l%16)
+        const int n_out = rb * kRows + 16 * wave + col;
+        if (emit && n_out < p.N) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) p.y[(size_t)(4 * kblk + r) * p.N + n_out] = (uint16_t)A::from_f32(acc[r]);
+          for (int r = 0; r < 4; ++r) p.y[(size_t)(4 * kblk + r) * p.N + n_out] = (uint16_t)A::from_f32(acc[r]);
+        }
+        ++rb;
+        in_rb = 0;
+        rb_left = p.stages;
+      }
+      cur_slot += kSlotBytes;
+      if (cur_slot == kDepth * kSlotBytes) cur_slot = 0;
+      if (left == 0) return;
     }
-    acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 }
 
