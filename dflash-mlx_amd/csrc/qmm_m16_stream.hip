@@ -145,34 +145,51 @@ struct Operands {
   u32x2_t wq[4];
   uint32_t sv[4], bv[4];
 };
-// Starts the LDS reads of a unit's operands and returns at once: the registers of `o` are
-// written behind the compiler's back until operands_wait(o) has been executed, so nothing
-// may touch `o` in between.  `acc` is threaded through both so that the arithmetic on the
-// previous unit, which ends in `acc`, stays between the two.
-__device__ __forceinline__ void operands_issue(uint32_t xaddr, uint32_t waddr, uint32_t saddr,
-                                               Operands& o, f32x4_t& acc0, f32x4_t& acc1,
-                                               f32x4_t& acc2, f32x4_t& acc3) {
-  asm volatile(
-      "ds_read_b128 %0, %18\n"
-      "ds_read_b128 %1, %18 offset:256\n"
-      "ds_read_b64 %2, %19\n"
-      "ds_read_b64 %3, %19 offset:2048\n"
-      "ds_read_b64 %4, %19 offset:4096\n"
-      "ds_read_b64 %5, %19 offset:6144\n"
-      "ds_read_u16 %6, %20\n"
-      "ds_read_u16 %10, %20 offset:4096\n"
-      "ds_read_u16 %7, %20 offset:512\n"
-      "ds_read_u16 %11, %20 offset:4608\n"
-      "ds_read_u16 %8, %20 offset:1024\n"
-      "ds_read_u16 %12, %20 offset:5120\n"
-      "ds_read_u16 %9, %20 offset:1536\n"
-      "ds_read_u16 %13, %20 offset:5632\n"
-      : "=&v"(o.f0), "=&v"(o.f1), "=&v"(o.wq[0]), "=&v"(o.wq[1]), "=&v"(o.wq[2]), "=&v"(o.wq[3]),
-        "=&v"(o.sv[0]), "=&v"(o.sv[1]), "=&v"(o.sv[2]), "=&v"(o.sv[3]),
-        "=&v"(o.bv[0]), "=&v"(o.bv[1]), "=&v"(o.bv[2]), "=&v"(o.bv[3]),
-        "+v"(acc0), "+v"(acc1), "+v"(acc2), "+v"(acc3)
-      : "v"(xaddr), "v"(waddr), "v"(saddr)
-      : "memory");
+// The LDS reads of a unit's operands are started in four pieces and return at once: the
+// registers of `o` are written behind the compiler's back until operands_wait(o) has been
+// executed, so nothing may touch `o` in between.  Piece j carries what tile j needs (piece 0
+// also the x fragments).  An accumulator is threaded through every piece and through the
+// wait, which pins piece j behind the arithmetic of tile j-1 of the previous unit's
+// operands: issued in one go, the reads of eight waves queue up in the LDS pipeline and
+// every wave sits in its issue stage instead of doing arithmetic.
+template <int J>
+__device__ __forceinline__ void operands_issue_piece(uint32_t xaddr, uint32_t waddr, uint32_t saddr,
+                                                     Operands& o, f32x4_t& pin) {
+  if (J == 0) {
+    asm volatile(
+        "ds_read_b128 %0, %6\n"
+        "ds_read_b128 %1, %6 offset:256\n"
+        "ds_read_b64 %2, %7\n"
+        "ds_read_u16 %3, %8\n"
+        "ds_read_u16 %4, %8 offset:4096\n"
+        : "=&v"(o.f0), "=&v"(o.f1), "=&v"(o.wq[0]), "=&v"(o.sv[0]), "=&v"(o.bv[0]), "+v"(pin)
+        : "v"(xaddr), "v"(waddr), "v"(saddr)
+        : "memory");
+  } else if (J == 1) {
+    asm volatile(
+        "ds_read_b64 %0, %4 offset:2048\n"
+        "ds_read_u16 %1, %5 offset:512\n"
+        "ds_read_u16 %2, %5 offset:4608\n"
+        : "=&v"(o.wq[1]), "=&v"(o.sv[1]), "=&v"(o.bv[1]), "+v"(pin)
+        : "v"(waddr), "v"(saddr)
+        : "memory");
+  } else if (J == 2) {
+    asm volatile(
+        "ds_read_b64 %0, %4 offset:4096\n"
+        "ds_read_u16 %1, %5 offset:1024\n"
+        "ds_read_u16 %2, %5 offset:5120\n"
+        : "=&v"(o.wq[2]), "=&v"(o.sv[2]), "=&v"(o.bv[2]), "+v"(pin)
+        : "v"(waddr), "v"(saddr)
+        : "memory");
+  } else {
+    asm volatile(
+        "ds_read_b64 %0, %4 offset:6144\n"
+        "ds_read_u16 %1, %5 offset:1536\n"
+        "ds_read_u16 %2, %5 offset:5632\n"
+        : "=&v"(o.wq[3]), "=&v"(o.sv[3]), "=&v"(o.bv[3]), "+v"(pin)
+        : "v"(waddr), "v"(saddr)
+        : "memory");
+  }
 }
 __device__ __forceinline__ void operands_wait(Operands& o, f32x4_t& acc0, f32x4_t& acc1,
                                               f32x4_t& acc2, f32x4_t& acc3) {
@@ -185,26 +202,36 @@ __device__ __forceinline__ void operands_wait(Operands& o, f32x4_t& acc0, f32x4_
                : "memory");
 }
 
-// The arithmetic of one unit: acc[j] += (scale, bias)-corrected x . codes^T of tile j.
+// The arithmetic of one unit: acc[j] += (scale, bias)-corrected x . codes^T of tile j, from
+// the operands in `cur`.  With `fetch` set, the reads of the next unit's operands into `nxt`
+// are started along the way (nothing else may touch `nxt` before operands_wait).
 template <bool ACT_FP16, bool SB_FP16>
-__device__ __forceinline__ void consume_unit(const Operands& o, f32x4_t (&acc)[4], uint4 ones,
-                                             uint32_t mask, uint32_t magic) {
+__device__ __forceinline__ void consume_unit(const Operands& cur, Operands& nxt, bool fetch,
+                                             uint32_t xaddr, uint32_t waddr, uint32_t saddr,
+                                             f32x4_t (&acc)[4], uint4 ones, uint32_t mask,
+                                             uint32_t magic) {
   using A = Act<ACT_FP16>;
   using SB = Act<SB_FP16>;
-  const uint4 a0 = as_uint4(permute_x(o.f0)), a1 = as_uint4(permute_x(o.f1));
+  if (fetch) operands_issue_piece<0>(xaddr, waddr, saddr, nxt, acc[3]);
+  const uint4 a0 = as_uint4(permute_x(cur.f0)), a1 = as_uint4(permute_x(cur.f1));
   f32x4_t xs = f32x4_t{0.f, 0.f, 0.f, 0.f};  // row sums of x over this group
   xs = A::mfma(a0, ones, xs);
   xs = A::mfma(a1, ones, xs);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     f32x4_t c = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    c = A::mfma(a0, unpack_codes(o.wq[j].x, mask, magic), c);
-    c = A::mfma(a1, unpack_codes(o.wq[j].y, mask, magic), c);
-    const float s = SB::to_f32(o.sv[j]);
-    const float b = SB::to_f32(o.bv[j]);
+    c = A::mfma(a0, unpack_codes(cur.wq[j].x, mask, magic), c);
+    c = A::mfma(a1, unpack_codes(cur.wq[j].y, mask, magic), c);
+    const float s = SB::to_f32(cur.sv[j]);
+    const float b = SB::to_f32(cur.bv[j]);
     const float bb = __builtin_fmaf(-A::kOffset, s, b);
 #pragma unroll
     for (int r = 0; r < 4; ++r) acc[j][r] = __builtin_fmaf(bb, xs[r], __builtin_fmaf(s, c[r], acc[j][r]));
+    if (fetch) {
+      if (j == 0) operands_issue_piece<1>(xaddr, waddr, saddr, nxt, acc[0]);
+      if (j == 1) operands_issue_piece<2>(xaddr, waddr, saddr, nxt, acc[1]);
+      if (j == 2) operands_issue_piece<3>(xaddr, waddr, saddr, nxt, acc[2]);
+    }
   }
 }
 
@@ -462,21 +489,28 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
   for (int j = 0; j < 4; ++j) acc4[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   Operands op[2];
 
-  auto start_operands = [&](Operands& o) __attribute__((always_inline)) {
+  // addresses of the next unit's operands, and the step to the unit after it
+  uint32_t rd_x, rd_w, rd_s;
+  auto next_addresses = [&]() __attribute__((always_inline)) {
     if (rd_q == 0 || rd_first) {
       rd_sb += kSbSlotBytes;
       if (rd_sb == kSbDepth * kSbSlotBytes) rd_sb = 0;
       rd_first = false;
     }
-    operands_issue(xoff + rd_slot, woff + rd_slot, soff + rd_sb + rd_q * 8, o, acc4[0], acc4[1],
-                   acc4[2], acc4[3]);
+    rd_x = xoff + rd_slot;
+    rd_w = woff + rd_slot;
+    rd_s = soff + rd_sb + rd_q * 8;
     rd_slot += kSlotBytes;
     if (rd_slot == kDepth * kSlotBytes) rd_slot = 0;
     rd_q = (rd_q + 1) & (kChunk - 1);
   };
 
   asm volatile("s_barrier" ::: "memory");
-  start_operands(op[0]);
+  next_addresses();
+  operands_issue_piece<0>(rd_x, rd_w, rd_s, op[0], acc4[0]);
+  operands_issue_piece<1>(rd_x, rd_w, rd_s, op[0], acc4[0]);
+  operands_issue_piece<2>(rd_x, rd_w, rd_s, op[0], acc4[0]);
+  operands_issue_piece<3>(rd_x, rd_w, rd_s, op[0], acc4[0]);
   operands_wait(op[0], acc4[0], acc4[1], acc4[2], acc4[3]);
 
   int left = u1 - u0;            // units still to consume, the current one included
@@ -492,9 +526,10 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       Operands& cur = op[par];
       Operands& nxt = op[par ^ 1];
       asm volatile("s_barrier" ::: "memory");
-      if (left > 1) start_operands(nxt);
-      consume_unit<ACT_FP16, SB_FP16>(cur, acc4, ones, mask, magic);
-      if (left > 1) operands_wait(nxt, acc4[0], acc4[1], acc4[2], acc4[3]);
+      const bool fetch = left > 1;
+      if (fetch) next_addresses();
+      consume_unit<ACT_FP16, SB_FP16>(cur, nxt, fetch, rd_x, rd_w, rd_s, acc4, ones, mask, magic);
+      if (fetch) operands_wait(nxt, acc4[0], acc4[1], acc4[2], acc4[3]);
       --left;
       ++in_rb;
       if (--rb_left == 0 || left == 0) {
