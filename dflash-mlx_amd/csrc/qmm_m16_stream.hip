@@ -3,39 +3,42 @@
 // y[16,N] = x[16,K] . (s*q + b)^T for group_size 64, K % 1024 == 0, N % 16 == 0 -
 // the shapes of the projections in the dense verify stacks.  Same arithmetic as
 // qmm_m16.hip (MFMA 16x16x32 on raw codes, scale/bias applied per (column, group) to
-// the fp32 accumulators); what differs is how bytes move:
+// the fp32 accumulators); what differs is how bytes move and who moves them:
 //
 //  * The weight matrix is cut into units of 128 rows x 256 k (16 KiB of codes plus the
 //    8 KiB slice of x they multiply; scales/biases come per chunk of four units).  Units
 //    are numbered row-block-major and divided EVENLY among a persistent grid of one
-//    512-thread workgroup per CU: every CU streams the same number of bytes (+-1 unit)
-//    whatever N and K are, fills its load pipeline once, and there is no tail of
-//    half-empty rounds.
-//  * Units go global -> LDS with 16-byte direct loads (no VGPR staging); each wave
-//    instruction moves 128-byte row segments of 8 rows.  A 5-deep ring keeps four units
-//    (96 KiB per CU) in flight while the fifth is consumed - HBM latency times bandwidth
-//    is ~100 KiB per CU on this part.  Granules are XOR-swizzled inside a row so that the
-//    MFMA-shaped reads spread evenly over the LDS banks.
-//  * Within a unit, wave w works on ONE quantisation group (w & 3) for 64 rows (four MFMA
+//    workgroup per CU: every CU streams the same number of bytes (+-1 unit) whatever N and
+//    K are, fills its load pipeline once, and there is no tail of half-empty rounds.
+//  * A workgroup is 8 worker waves plus 4 loader waves.  Loaders do nothing but move units
+//    global -> LDS with 16-byte direct loads (no VGPR staging; each instruction moves
+//    128-byte row segments of 8 rows) into a ring of slots, a few units ahead of the
+//    workers.  An instruction that finds the CU's load queue full sits in its issue stage;
+//    in a loader that costs nothing, in a worker it would stop the arithmetic.  Granules
+//    are XOR-swizzled inside a row so that MFMA-shaped reads spread over the LDS banks.
+//  * Within a unit, worker w handles ONE quantisation group (w & 3) for 64 rows (four MFMA
 //    tiles, rows 64*(w >> 2) ..): the x fragments and the row sums of x (an MFMA against
-//    ones, already in accumulator layout) are then shared by its four tiles, which keeps
-//    the LDS read traffic per unit at a quarter of what "one tile, all groups" costs.  The
-//    four waves that cover the same rows add their accumulators through LDS only when a
-//    row block ends; after that wave w holds tile w and writes it out.
-//  * A workgroup whose range covers all of K for a row block writes y directly.
-//    Row blocks shared between workgroups go through fp32 partial tiles in the
-//    workspace; the last contributor to arrive (wrapping agent-scope counter)
-//    adds them in contributor order and rounds once - deterministic, no spinning.
-//    Partials are written through to / read from the level all XCDs share (sc1), so
-//    that no L2 write-back fence is ever issued.
+//    ones, already in accumulator layout) are shared by its four tiles.  The operands of
+//    the next unit are read from LDS into a second register set while the current unit is
+//    worked on, a few reads between one tile and the next.  The four workers that cover
+//    the same rows add their accumulators through LDS only when a row block ends; after
+//    that worker w holds tile w.
+//  * A workgroup whose range covers all of K for a row block writes y directly.  Row
+//    blocks shared between workgroups go through fp32 partial tiles in the workspace; a
+//    workgroup announces its tiles once, after its last unit (wrapping agent-scope
+//    counter per row block), and the last contributor to arrive adds them in contributor
+//    order and rounds once - deterministic, no spinning.  Partials are written through to
+//    / read from the level all XCDs share (sc1): no L2 write-back fence is ever issued.
 //
 // The compiler orders every LDS access it can see behind ALL outstanding direct-to-LDS
 // loads (s_waitcnt vmcnt(0)), and __syncthreads() carries a fence with the same effect;
-// either would drain the ring on every unit.  The main loop therefore touches LDS only
-// through hand-written instruction blocks and synchronises with a bare s_barrier plus
-// an explicit vmcnt wait (loads retire in issue order and every wave issues the same
-// number of them per unit: one for x, two for codes, plus one with each scale/bias chunk).
-// The row-block epilogue (a few times per workgroup) uses ordinary code.
+// either would drain the ring on every unit.  The kernel therefore touches LDS only
+// through hand-written instruction blocks and synchronises with bare s_barriers; a loader
+// waits for "my part of unit v has landed" with an explicit vmcnt (loads retire in issue
+// order, and the number a loader issues per unit is a closed form of the unit index).
+// Every instruction a wave issues costs it at least four cycles, scalar bookkeeping
+// included, so the per-unit paths are kept short: ring positions advance by addition,
+// and the loaders and the workers run separate loops that meet only at the barriers.
 #include "dflash_common.h"
 
 namespace dflash {
@@ -49,6 +52,10 @@ constexpr int kUnitK = 256;  // k per unit (four groups of 64)
 constexpr int kGS = 64;
 constexpr int kGroups = kUnitK / kGS;
 constexpr int kDepth = 5;                      // ring slots of (codes + x)
+// Units a loader keeps issued beyond the one being consumed.  A CU holds about 64 KiB of
+// loads in flight (what HBM latency times its share of the bandwidth comes to); a loader
+// that tries to issue more only sits in its issue stage and is late for the next barrier.
+constexpr int kAhead = 3;
 constexpr int kWBytes = kRows * (kUnitK / 2);  // 16 KiB: 128 B per row
 constexpr int kXBytes = 16 * kUnitK * 2;       // 8 KiB
 constexpr int kXOffset = kWBytes;
@@ -348,8 +355,9 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
   //   one per unit u (unit u+1 has landed; every worker holds unit u in registers, so the
   //     slot of unit u is free),
   //   when a row block ends with unit u: one more (the slot of unit u carries the cross-wave
-  //     sum), and two more if other workgroups share the row block (partial tile stored /
-  //     arrival counter bumped).
+  //     sum),
+  //   after the last unit, if a row block was shared with other workgroups: two more (partial
+  //     tiles stored / arrival counters bumped).
 
   if (wave >= kWaves) {
     // ================================ loader waves ====================================
@@ -430,31 +438,34 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       wait_loads(loads_through(issued - 1) - loads_through(v));
     };
 
-    for (int i = 0; i < kDepth && issued < u1; ++i) issue_next();
+    for (int i = 0; i < kAhead && issued < u1; ++i) issue_next();
     wait_unit(u0);
     asm volatile("s_barrier" ::: "memory");
     int rb_left = p.stages - st0;  // units of the current row block from unit u on
     int in_rb = 0;                 // units of the current row block this workgroup has done
+    bool any_shared = false;       // a row block ended that other workgroups share
 #pragma unroll 1
     for (int u = u0; u < u1; ++u) {
       const bool rb_ends = rb_left == 1 || u + 1 == u1;
       if (u + 1 < u1) wait_unit(u + 1);
       asm volatile("s_barrier" ::: "memory");
-      // the slot of unit u takes unit u+5 - unless a row block ends here: then it first
-      // carries the cross-wave sum and is refilled one unit later
-      const int limit = rb_ends ? u + kDepth - 1 : u + kDepth;
+      // keep kAhead units issued beyond unit u; their slots are free: the ring has kDepth > kAhead
+      // slots, and the slot of unit u itself (which may carry a cross-wave sum below) is only
+      // refilled kDepth - kAhead units later
+      const int limit = u + kAhead;
       while (issued <= limit && issued < u1) issue_next();
       ++in_rb;
       --rb_left;
       if (rb_ends) {
         asm volatile("s_barrier" ::: "memory");
-        if (in_rb != p.stages) {
-          asm volatile("s_barrier" ::: "memory");
-          asm volatile("s_barrier" ::: "memory");
-        }
+        if (in_rb != p.stages) any_shared = true;
         in_rb = 0;
         rb_left = p.stages;
       }
+    }
+    if (any_shared) {
+      asm volatile("s_barrier" ::: "memory");
+      asm volatile("s_barrier" ::: "memory");
     }
     return;
   }
@@ -518,6 +529,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
   int in_rb = 0;                 // units of the current row block this workgroup has done
   int rb = rb0;
   int cur_slot = 0;              // byte offset of the current unit's ring slot
+  int shared_rb[2] = {-1, -1};   // row blocks whose partial tiles I have stored
 
 #pragma unroll 1
   while (true) {
@@ -533,71 +545,30 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       --left;
       ++in_rb;
       if (--rb_left == 0 || left == 0) {
-        // ---- a row block ends inside my range: emit it -----------------------------------
+        // ---- a row block ends inside my range ---------------------------------------------
         const uint32_t sbase = lds0 + cur_slot;
         reduce_groups_write(sbase, acc4, wave, lane);
         asm volatile("s_barrier" ::: "memory");
-        f32x4_t acc = reduce_groups_read(sbase, acc4, wave, lane);
+        const f32x4_t acc = reduce_groups_read(sbase, acc4, wave, lane);
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc4[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-        bool emit = true;
-        if (in_rb != p.stages) {
+        if (in_rb == p.stages) {
+          // the whole row block was mine: accumulator r of lane l is output
+          // (m = 4*(l/16) + r, n = row0 + 16*wave + l%16)
+          const int n_out = rb * kRows + 16 * wave + col;
+          if (n_out < p.N) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              p.y[(size_t)(4 * kblk + r) * p.N + n_out] = (uint16_t)A::from_f32(acc[r]);
+          }
+        } else {
           // Other workgroups hold the rest of this row block.  A workgroup shares at most two
-          // row blocks: the one its range starts in (slot 0) and the one it ends in (slot 1);
-          // partial tiles are kept in accumulator layout.
-          const int lo = rb * p.stages;
-          float* part = p.partials + ((size_t)blockIdx.x * 2 + (rb == rb0 ? 0 : 1)) * kPartialFloats;
-          // contributors: the workgroups whose ranges intersect [lo, lo+stages);
-          // owner(v) = ceil((v+1)*grid/units) - 1 is the workgroup whose range holds unit v
-          const int wg_first = (int)((((unsigned)lo + 1u) * (unsigned)grid + p.units - 1) / (unsigned)p.units) - 1;
-          const int wg_last =
-              (int)((((unsigned)(lo + p.stages)) * (unsigned)grid + p.units - 1) / (unsigned)p.units) - 1;
-          store_partial(part + tid * 4, acc);
-          // every worker's store has been acknowledged before the barrier, hence before
-          // thread 0 bumps the counter; a release fence here would write back the whole L2
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-          // (all workers have their received tiles in registers: the flag may reuse the slot)
-          asm volatile("s_barrier" ::: "memory");
-          if (tid == 0) {
-            const uint32_t n_contrib = (uint32_t)(wg_last - wg_first + 1);
-            // wrapping increment: the last arrival sees n-1 and leaves 0 behind for the next call
-            const uint32_t prev = atomicInc(&p.counters[rb], n_contrib - 1);
-            const uint32_t flag = (prev == n_contrib - 1) ? 1u : 0u;
-            asm volatile("ds_write_b32 %0, %1\n s_waitcnt lgkmcnt(0)" : : "v"(sbase), "v"(flag) : "memory");
-          }
-          asm volatile("s_barrier" ::: "memory");
-          uint32_t last;
-          asm volatile("ds_read_b32 %0, %1\n s_waitcnt lgkmcnt(0)" : "=v"(last) : "v"(sbase) : "memory");
-          emit = __builtin_amdgcn_readfirstlane(last) != 0;
-          if (emit) {
-            // only the first contributor can have started before this row block (then the
-            // block is the one its range ends in); every later one starts inside it
-            const int which_first = range_begin(p.units, wg_first, grid) < lo ? 1 : 0;
-            acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            for (int wg = wg_first; wg <= wg_last; wg += 4) {
-              const float* src[4];
-#pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                const int w = wg + j <= wg_last ? wg + j : wg_last;  // surplus slots re-read the last tile
-                src[j] = p.partials + ((size_t)w * 2 + (w == wg_first ? which_first : 0)) * kPartialFloats + tid * 4;
-              }
-              f32x4_t v[4];
-              load_partials4(src[0], src[1], src[2], src[3], v);
-#pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                if (wg + j <= wg_last) {
-#pragma unroll
-                  for (int r = 0; r < 4; ++r) acc[r] += v[j][r];
-                }
-              }
-            }
-          }
-        }
-        // accumulator r of lane l is output (m = 4*(l/16) + r, n = row0 + 16*wave + l%16)
-        const int n_out = rb * kRows + 16 * wave + col;
-        if (emit && n_out < p.N) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r) p.y[(size_t)(4 * kblk + r) * p.N + n_out] = (uint16_t)A::from_f32(acc[r]);
+          // row blocks: the one its range starts in (partial slot 0) and the one it ends in
+          // (slot 1); partial tiles are kept in accumulator layout.  The store is not awaited
+          // here: arrival is announced once, after the last unit.
+          const int which = rb == rb0 ? 0 : 1;
+          store_partial(p.partials + ((size_t)blockIdx.x * 2 + which) * kPartialFloats + tid * 4, acc);
+          shared_rb[which] = rb;
         }
         ++rb;
         in_rb = 0;
@@ -605,7 +576,78 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       }
       cur_slot += kSlotBytes;
       if (cur_slot == kDepth * kSlotBytes) cur_slot = 0;
-      if (left == 0) return;
+      if (left == 0) goto arrive;
+    }
+  }
+arrive:
+  if (shared_rb[0] < 0 && shared_rb[1] < 0) return;
+  // ---- arrival at the shared row blocks ---------------------------------------------------
+  // Every worker's partial stores have been acknowledged before the barrier, hence before
+  // thread 0 bumps the counters; a release fence here would write back the whole L2.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  asm volatile("s_barrier" ::: "memory");
+  int wg_lo[2], wg_hi[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    // contributors of a row block: the workgroups whose ranges intersect [lo, lo+stages);
+    // owner(v) = ceil((v+1)*grid/units) - 1 is the workgroup whose range holds unit v
+    const int lo = shared_rb[i] * p.stages;
+    wg_lo[i] = (int)((((unsigned)lo + 1u) * (unsigned)grid + p.units - 1) / (unsigned)p.units) - 1;
+    wg_hi[i] = (int)((((unsigned)(lo + p.stages)) * (unsigned)grid + p.units - 1) / (unsigned)p.units) - 1;
+  }
+  if (tid == 0) {
+    uint32_t prev[2] = {0u, 0u}, flag[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      // wrapping increment: the last arrival sees n-1 and leaves 0 behind for the next call
+      if (shared_rb[i] >= 0) prev[i] = atomicInc(&p.counters[shared_rb[i]], (uint32_t)(wg_hi[i] - wg_lo[i]));
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      flag[i] = (shared_rb[i] >= 0 && prev[i] == (uint32_t)(wg_hi[i] - wg_lo[i])) ? 1u : 0u;
+    asm volatile("ds_write_b32 %0, %1\n ds_write_b32 %0, %2 offset:4\n s_waitcnt lgkmcnt(0)"
+                 :
+                 : "v"(lds0), "v"(flag[0]), "v"(flag[1])
+                 : "memory");
+  }
+  asm volatile("s_barrier" ::: "memory");
+  uint32_t last0, last1;
+  asm volatile("ds_read_b32 %0, %2\n ds_read_b32 %1, %2 offset:4\n s_waitcnt lgkmcnt(0)"
+               : "=&v"(last0), "=&v"(last1)
+               : "v"(lds0)
+               : "memory");
+  const bool is_last[2] = {__builtin_amdgcn_readfirstlane(last0) != 0,
+                           __builtin_amdgcn_readfirstlane(last1) != 0};
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    if (!is_last[i]) continue;
+    // The last contributor to arrive adds the partial tiles in contributor order.  Only the
+    // first contributor can have started before this row block (then the block is the one
+    // its range ends in, slot 1); every later one starts inside it (slot 0).
+    const int lo = shared_rb[i] * p.stages;
+    const int which_first = range_begin(p.units, wg_lo[i], grid) < lo ? 1 : 0;
+    f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int wg = wg_lo[i]; wg <= wg_hi[i]; wg += 4) {
+      const float* src[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int w = wg + j <= wg_hi[i] ? wg + j : wg_hi[i];  // surplus slots re-read the last tile
+        src[j] = p.partials + ((size_t)w * 2 + (w == wg_lo[i] ? which_first : 0)) * kPartialFloats + tid * 4;
+      }
+      f32x4_t v[4];
+      load_partials4(src[0], src[1], src[2], src[3], v);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (wg + j <= wg_hi[i]) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[r] += v[j][r];
+        }
+      }
+    }
+    const int n_out = shared_rb[i] * kRows + 16 * wave + col;
+    if (n_out < p.N) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) p.y[(size_t)(4 * kblk + r) * p.N + n_out] = (uint16_t)A::from_f32(acc[r]);
     }
   }
 }
