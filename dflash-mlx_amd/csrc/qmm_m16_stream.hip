@@ -281,17 +281,21 @@ __device__ __forceinline__ f32x4_t reduce_groups_read(uint32_t base, const f32x4
 __device__ __forceinline__ void store_partial(float* p, f32x4_t v) {
   asm volatile("global_store_dwordx4 %0, %1, off sc1\n" : : "v"(p), "v"(v) : "memory");
 }
-// four tiles at once, so that their latencies overlap
-__device__ __forceinline__ void load_partials4(const float* p0, const float* p1, const float* p2,
-                                               const float* p3, f32x4_t (&v)[4]) {
+// eight tiles at once, so that their latencies overlap
+__device__ __forceinline__ void load_partials8(const float* const (&p)[8], f32x4_t (&v)[8]) {
   asm volatile(
-      "global_load_dwordx4 %0, %4, off sc1\n"
-      "global_load_dwordx4 %1, %5, off sc1\n"
-      "global_load_dwordx4 %2, %6, off sc1\n"
-      "global_load_dwordx4 %3, %7, off sc1\n"
+      "global_load_dwordx4 %0, %8, off sc1\n"
+      "global_load_dwordx4 %1, %9, off sc1\n"
+      "global_load_dwordx4 %2, %10, off sc1\n"
+      "global_load_dwordx4 %3, %11, off sc1\n"
+      "global_load_dwordx4 %4, %12, off sc1\n"
+      "global_load_dwordx4 %5, %13, off sc1\n"
+      "global_load_dwordx4 %6, %14, off sc1\n"
+      "global_load_dwordx4 %7, %15, off sc1\n"
       "s_waitcnt vmcnt(0)\n"
-      : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3])
-      : "v"(p0), "v"(p1), "v"(p2), "v"(p3)
+      : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]),
+        "=&v"(v[7])
+      : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7])
       : "memory");
 }
 
@@ -627,17 +631,17 @@ arrive:
     const int lo = shared_rb[i] * p.stages;
     const int which_first = range_begin(p.units, wg_lo[i], grid) < lo ? 1 : 0;
     f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    for (int wg = wg_lo[i]; wg <= wg_hi[i]; wg += 4) {
-      const float* src[4];
+    for (int wg = wg_lo[i]; wg <= wg_hi[i]; wg += 8) {
+      const float* src[8];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < 8; ++j) {
         const int w = wg + j <= wg_hi[i] ? wg + j : wg_hi[i];  // surplus slots re-read the last tile
         src[j] = p.partials + ((size_t)w * 2 + (w == wg_lo[i] ? which_first : 0)) * kPartialFloats + tid * 4;
       }
-      f32x4_t v[4];
-      load_partials4(src[0], src[1], src[2], src[3], v);
+      f32x4_t v[8];
+      load_partials8(src, v);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < 8; ++j) {
         if (wg + j <= wg_hi[i]) {
 #pragma unroll
           for (int r = 0; r < 4; ++r) acc[r] += v[j][r];

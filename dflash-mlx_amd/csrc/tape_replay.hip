@@ -131,11 +131,44 @@ __global__ __launch_bounds__(kThreads) void replay_f32_128(ReplayArgs a) {
   const f32x4_t* in = reinterpret_cast<const f32x4_t*>(a.state_in) + (size_t)blockIdx.x * (128 * 32);
   f32x4_t* out = reinterpret_cast<f32x4_t*>(a.state_out) + (size_t)blockIdx.x * (128 * 32);
 
+  // The tape is asked for first and the state right behind it: loads return in issue order,
+  // so the tape is in LDS and the gates are folded while the 64 KiB of state are still on
+  // their way, instead of the state waiting in registers for the tape.
+  float td[8], tk[8], tg[8];
+  float tg1 = 1.f;
+  {
+    const int hk = hv / (a.Hv / a.Hk);
+    const size_t slotT = (size_t)slot * a.T;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = tid + kThreads * j, t = i >> 7, d = i & 127;  // step, element
+      const bool on = t < n && (a.mask == nullptr || a.mask[slotT + t] != 0);
+      td[j] = 0.f, tk[j] = 0.f, tg[j] = 1.f;
+      if (on) {
+        td[j] = load_as_f32(a.tape, ((slotT + t) * a.Hv + hv) * 128 + d, a.tape_dtype);
+        tk[j] = load_as_f32(a.k, ((slotT + t) * a.Hk + hk) * 128 + d, a.k_dtype);
+        if (a.g_per_dk) tg[j] = load_as_f32(a.g, ((slotT + t) * a.Hv + hv) * 128 + d, a.g_dtype);
+      }
+    }
+    if (!a.g_per_dk && tid < Tl) {
+      if (tid < n && (a.mask == nullptr || a.mask[slotT + tid] != 0))
+        tg1 = load_as_f32(a.g, (slotT + tid) * a.Hv + hv, a.g_dtype);
+    }
+  }
+
   f32x4_t st[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) st[i] = __builtin_nontemporal_load(&in[(row0 + 8 * i) * 32 + c4]);
 
-  stage_tape(a, s, slot, hv, n, Tl, Tl);
+  // same tables as stage_tape(): masked and missing steps are (delta = 0, k = 0, g = 1)
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int i = tid + kThreads * j, t = i >> 7, d = i & 127;
+    s.sA[(size_t)d * Tl + t] = td[j];
+    s.sK[i] = tk[j];
+    if (a.g_per_dk) s.sG[i] = tg[j];
+  }
+  if (!a.g_per_dk && tid < Tl) s.sG[tid] = tg1;
   __syncthreads();
   fold_gates(a, s, n);
   __syncthreads();
