@@ -1,0 +1,83 @@
+"""Static check of the streaming qmm kernel's machine code.
+
+The kernel starts LDS reads whose destination registers are written after the issuing
+instruction block has ended, and waits for them in a later block; the compiler does not
+know that.  This test compiles the kernel to gfx950 assembly and scans it: between an LDS
+read and the next wait for lgkmcnt(0), no instruction may name a register the read is still
+writing (a register copy or spill placed there by the compiler would read garbage).
+"""
+import os
+import re
+import shutil
+import subprocess
+import tempfile
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SRC = os.path.join(ROOT, "dflash-mlx_amd", "csrc", "qmm_m16_stream.hip")
+
+
+def _regs(text):
+    out = set()
+    for m in re.finditer(r"\bv\[(\d+):(\d+)\]|\bv(\d+)\b", text):
+        if m.group(1):
+            out.update(range(int(m.group(1)), int(m.group(2)) + 1))
+        else:
+            out.add(int(m.group(3)))
+    return out
+
+
+def scan(asm_text):
+    """Returns (number of LDS reads seen, list of offending lines)."""
+    pending, bad, reads = set(), [], 0
+    for no, line in enumerate(asm_text.split("\n"), 1):
+        t = line.split(";")[0].strip()
+        if not t or t.startswith(".") or t.endswith(":"):
+            continue
+        if t.startswith("ds_read") or t.startswith("ds_bpermute"):
+            ops = t.split(None, 1)[1].split(",")
+            if _regs(",".join(ops[1:])) & pending:
+                bad.append((no, t))
+            pending |= _regs(ops[0])
+            reads += 1
+            continue
+        if t.startswith("s_waitcnt") and "lgkmcnt(0)" in t:
+            pending = set()
+            continue
+        if t.startswith("s_endpgm"):
+            pending = set()
+            continue
+        if _regs(t) & pending:
+            bad.append((no, t))
+    return reads, bad
+
+
+def test_scanner_flags_a_premature_use():
+    ok = "ds_read_b128 v[4:7], v1\nv_add_f32 v9, v8, v8\ns_waitcnt lgkmcnt(0)\nv_add_f32 v9, v4, v8\n"
+    assert scan(ok) == (1, [])
+    early = "ds_read_b128 v[4:7], v1\nv_mov_b32 v9, v5\ns_waitcnt lgkmcnt(0)\n"
+    reads, bad = scan(early)
+    assert reads == 1 and len(bad) == 1 and "v_mov_b32" in bad[0][1]
+    partial = "ds_read_b64 v[4:5], v1\ns_waitcnt lgkmcnt(1)\nv_mov_b32 v9, v4\n"
+    assert len(scan(partial)[1]) == 1
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not available")
+def test_no_instruction_touches_registers_of_reads_in_flight():
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "stream.s")
+        cmd = ["hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
+               "-Xclang", "-packed-fp32-ops", "-I", os.path.join(ROOT, "include"),
+               "-I", os.path.dirname(SRC), "--cuda-device-only", "-S", "-o", out, SRC]
+        subprocess.run(cmd, check=True, capture_output=True, timeout=600)
+        text = open(out).read()
+    kernels = re.findall(r"^(_ZN6dflash6stream17qmm_stream_kernel\w+):", text, flags=re.M)
+    assert len(kernels) == 4, kernels
+    for name in kernels:
+        body = text[text.index(name + ":"):]
+        body = body[:body.index(".Lfunc_end")]
+        reads, bad = scan(body)
+        assert reads >= 40, (name, reads)   # the operand reads are there at all
+        assert not bad, (name, bad[:5])
+        assert "scratch_" not in body, name  # nothing spilled
