@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
@@ -24,6 +24,7 @@ EXPORTED_SYMBOLS = (
     "dflash_last_error",
     "dflash_qmm_m16_workspace_bytes",
     "dflash_qmm_m16",
+    "dflash_qmm_m16_gather_workspace_bytes",
     "dflash_qmm_m16_gather",
     "dflash_tape_replay",
     "dflash_conv_state_rebuild",
@@ -49,8 +50,12 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.dflash_qmm_m16.argtypes = (
         [c.c_void_p] * 6 + [c.c_size_t] + [c.c_int] * 8 + [c.c_void_p]
     )
+    lib.dflash_qmm_m16_gather_workspace_bytes.restype = c.c_size_t
+    lib.dflash_qmm_m16_gather_workspace_bytes.argtypes = [c.c_int] * 5
     lib.dflash_qmm_m16_gather.restype = c.c_int
-    lib.dflash_qmm_m16_gather.argtypes = [c.c_void_p] * 6 + [c.c_int] * 7 + [c.c_void_p]
+    lib.dflash_qmm_m16_gather.argtypes = (
+        [c.c_void_p] * 7 + [c.c_size_t] + [c.c_int] * 7 + [c.c_void_p]
+    )
     lib.dflash_tape_replay.restype = c.c_int
     lib.dflash_tape_replay.argtypes = (
         [c.c_void_p] * 6 + [c.c_int] + [c.c_void_p] + [c.c_int] * 12 + [c.c_void_p]

@@ -402,6 +402,11 @@ int qmm_stream_grid();
 int qmm_stream_launch(const void* x, const uint32_t* w, const void* scales, const void* biases,
                       void* y, void* workspace, size_t workspace_bytes, int K, int N,
                       int act_dtype, int sb_dtype, hipStream_t stream);
+bool qmm_stream_gather_eligible(int P, int K, int N, int E, int group_size);
+int qmm_stream_gather_launch(const void* x, const int32_t* expert_ids, const uint32_t* w,
+                             const void* scales, const void* biases, void* y, void* workspace,
+                             size_t workspace_bytes, int P, int K, int N, int E, int act_dtype,
+                             int sb_dtype, hipStream_t stream);
 }  // namespace dflash
 
 extern "C" size_t dflash_qmm_m16_workspace_bytes(int K, int N, int group_size, int variant,
@@ -475,9 +480,16 @@ extern "C" int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* sc
   }
 }
 
+extern "C" size_t dflash_qmm_m16_gather_workspace_bytes(int P, int K, int N, int E,
+                                                        int group_size) {
+  if (!dflash::qmm_stream_gather_eligible(P, K, N, E, group_size)) return 0;
+  return dflash::qmm_stream_workspace_bytes(N, dflash::qmm_stream_grid());
+}
+
 extern "C" int dflash_qmm_m16_gather(const void* x, const int32_t* expert_ids, const uint32_t* w_q,
-                                     const void* scales, const void* biases, void* y, int P, int K,
-                                     int N, int E, int group_size, int act_dtype, int sb_dtype,
+                                     const void* scales, const void* biases, void* y,
+                                     void* workspace, size_t workspace_bytes, int P, int K, int N,
+                                     int E, int group_size, int act_dtype, int sb_dtype,
                                      void* stream) {
   using namespace dflash;
   DFLASH_REQUIRE(x && expert_ids && w_q && scales && biases && y, DFLASH_ERR_ARG,
@@ -499,6 +511,12 @@ extern "C" int dflash_qmm_m16_gather(const void* x, const int32_t* expert_ids, c
                  DFLASH_ERR_ARG, "dflash_qmm_m16_gather: x and w_q must be 16-byte aligned");
   if (P == 0) return DFLASH_OK;
   hipStream_t s = (hipStream_t)stream;
+  // With a workspace, shapes the streaming kernel covers go through it; everything else,
+  // and callers without a workspace, through the one-workgroup-per-(columns, expert) kernel.
+  if (workspace != nullptr && qmm_stream_gather_eligible(P, K, N, E, group_size)) {
+    return qmm_stream_gather_launch(x, expert_ids, w_q, scales, biases, y, workspace, workspace_bytes,
+                                    P, K, N, E, act_dtype, sb_dtype, s);
+  }
   switch (group_size) {
     case 32:
       return launch_gather_gs<32>(act_dtype, sb_dtype, x, expert_ids, w_q, scales, biases, y, P, K, N, E, s);

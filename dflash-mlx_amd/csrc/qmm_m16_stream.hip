@@ -1,7 +1,10 @@
 // Streaming M=16 int4 qmm for gfx950: persistent workgroups, LDS-staged weights.
 //
-// y[16,N] = x[16,K] . (s*q + b)^T for group_size 64, K % 1024 == 0, N % 16 == 0 -
-// the shapes of the projections in the dense verify stacks.  Same arithmetic as
+// y[16,N] = x[16,K] . (s*q + b)^T for group_size 64, K % 512 == 0, N % 16 == 0 - the
+// shapes of the projections in the dense verify stacks - and its gathered form for MoE
+// layers, y[p] = x[p] . (s*q + b)^T of expert ids[p] for up to 256 rows: rows that share an
+// expert are taken 16 at a time as the M dimension, and the weights of the experts that
+// have rows are streamed like one tall matrix.  Same arithmetic as
 // qmm_m16.hip (MFMA 16x16x32 on raw codes, scale/bias applied per (column, group) to
 // the fp32 accumulators); what differs is how bytes move and who moves them:
 //
@@ -60,16 +63,26 @@ constexpr int kWBytes = kRows * (kUnitK / 2);  // 16 KiB: 128 B per row
 constexpr int kXBytes = 16 * kUnitK * 2;       // 8 KiB
 constexpr int kXOffset = kWBytes;
 constexpr int kSlotBytes = kWBytes + kXBytes;  // 24 KiB
-// Scales and biases are staged per chunk of kChunk units (32 bytes per row and array):
-// fetching them unit by unit would cost two 8-byte requests per row and unit, twice the
-// number of memory requests the codes themselves need.
-constexpr int kChunk = 4;
+// Scales and biases are staged per chunk of CHUNK units (CHUNK = 4: 32 bytes per row and
+// array; CHUNK = 2, for K that is a multiple of 512 only: 16 bytes): fetching them unit by
+// unit would cost two 8-byte requests per row and unit, twice the number of memory requests
+// the codes themselves need.
 constexpr int kSbDepth = 3;
-constexpr int kSbArrayBytes = kRows * kChunk * kGroups * 2;  // 4 KiB
-constexpr int kSbSlotBytes = 2 * kSbArrayBytes;              // scales then biases
+constexpr int kSbArrayBytes = kRows * 4 * kGroups * 2;  // 4 KiB, sized for CHUNK = 4
+constexpr int kSbSlotBytes = 2 * kSbArrayBytes;         // scales then biases
 constexpr int kSbOffset = kDepth * kSlotBytes;
 constexpr int kLdsBytes = kSbOffset + kSbDepth * kSbSlotBytes;  // 144 KiB
 constexpr int kPartialFloats = 16 * kRows;
+// Gathered (per-expert) form: tables built in LDS by every workgroup at kernel start.
+//   an "entry" is up to 16 rows of x that go through the same expert's weights
+constexpr int kMaxEntries = 256;  // hence at most 256 rows of x
+constexpr int kMaxExperts = 1024;
+constexpr int kTabOffset = kLdsBytes;
+constexpr int kTabCount = 0;                        // u32 [kMaxExperts]: rows << 16 | first entry
+constexpr int kTabEntry = kTabCount + 4 * kMaxExperts;   // u32 [kMaxEntries]: rows << 16 | expert
+constexpr int kTabRows = kTabEntry + 4 * kMaxEntries;    // u16 [kMaxEntries][16]: row of x, y
+constexpr int kTabTotal = kTabRows + 2 * 16 * kMaxEntries;  // u32: number of entries
+constexpr int kLdsBytesGather = kTabOffset + kTabTotal + 64;  // 157.1 KiB
 
 template <bool FP16>
 struct Act;
@@ -159,7 +172,8 @@ struct Operands {
 // wait, which pins piece j behind the arithmetic of tile j-1 of the previous unit's
 // operands: issued in one go, the reads of eight waves queue up in the LDS pipeline and
 // every wave sits in its issue stage instead of doing arithmetic.
-template <int J>
+// SBROW: bytes of scales per row and chunk in LDS (8 * CHUNK); tile j is 16 rows further.
+template <int J, int SBROW>
 __device__ __forceinline__ void operands_issue_piece(uint32_t xaddr, uint32_t waddr, uint32_t saddr,
                                                      Operands& o, f32x4_t& pin) {
   if (J == 0) {
@@ -172,29 +186,13 @@ __device__ __forceinline__ void operands_issue_piece(uint32_t xaddr, uint32_t wa
         : "=&v"(o.f0), "=&v"(o.f1), "=&v"(o.wq[0]), "=&v"(o.sv[0]), "=&v"(o.bv[0]), "+v"(pin)
         : "v"(xaddr), "v"(waddr), "v"(saddr)
         : "memory");
-  } else if (J == 1) {
-    asm volatile(
-        "ds_read_b64 %0, %4 offset:2048\n"
-        "ds_read_u16 %1, %5 offset:512\n"
-        "ds_read_u16 %2, %5 offset:4608\n"
-        : "=&v"(o.wq[1]), "=&v"(o.sv[1]), "=&v"(o.bv[1]), "+v"(pin)
-        : "v"(waddr), "v"(saddr)
-        : "memory");
-  } else if (J == 2) {
-    asm volatile(
-        "ds_read_b64 %0, %4 offset:4096\n"
-        "ds_read_u16 %1, %5 offset:1024\n"
-        "ds_read_u16 %2, %5 offset:5120\n"
-        : "=&v"(o.wq[2]), "=&v"(o.sv[2]), "=&v"(o.bv[2]), "+v"(pin)
-        : "v"(waddr), "v"(saddr)
-        : "memory");
   } else {
     asm volatile(
-        "ds_read_b64 %0, %4 offset:6144\n"
-        "ds_read_u16 %1, %5 offset:1536\n"
-        "ds_read_u16 %2, %5 offset:5632\n"
-        : "=&v"(o.wq[3]), "=&v"(o.sv[3]), "=&v"(o.bv[3]), "+v"(pin)
-        : "v"(waddr), "v"(saddr)
+        "ds_read_b64 %0, %4 offset:%6\n"
+        "ds_read_u16 %1, %5 offset:%7\n"
+        "ds_read_u16 %2, %5 offset:%8\n"
+        : "=&v"(o.wq[J]), "=&v"(o.sv[J]), "=&v"(o.bv[J]), "+v"(pin)
+        : "v"(waddr), "v"(saddr), "n"(2048 * J), "n"(16 * SBROW * J), "n"(4096 + 16 * SBROW * J)
         : "memory");
   }
 }
@@ -212,14 +210,14 @@ __device__ __forceinline__ void operands_wait(Operands& o, f32x4_t& acc0, f32x4_
 // The arithmetic of one unit: acc[j] += (scale, bias)-corrected x . codes^T of tile j, from
 // the operands in `cur`.  With `fetch` set, the reads of the next unit's operands into `nxt`
 // are started along the way (nothing else may touch `nxt` before operands_wait).
-template <bool ACT_FP16, bool SB_FP16>
+template <bool ACT_FP16, bool SB_FP16, int SBROW>
 __device__ __forceinline__ void consume_unit(const Operands& cur, Operands& nxt, bool fetch,
                                              uint32_t xaddr, uint32_t waddr, uint32_t saddr,
                                              f32x4_t (&acc)[4], uint4 ones, uint32_t mask,
                                              uint32_t magic) {
   using A = Act<ACT_FP16>;
   using SB = Act<SB_FP16>;
-  if (fetch) operands_issue_piece<0>(xaddr, waddr, saddr, nxt, acc[3]);
+  if (fetch) operands_issue_piece<0, SBROW>(xaddr, waddr, saddr, nxt, acc[3]);
   const uint4 a0 = as_uint4(permute_x(cur.f0)), a1 = as_uint4(permute_x(cur.f1));
   f32x4_t xs = f32x4_t{0.f, 0.f, 0.f, 0.f};  // row sums of x over this group
   xs = A::mfma(a0, ones, xs);
@@ -235,9 +233,9 @@ __device__ __forceinline__ void consume_unit(const Operands& cur, Operands& nxt,
 #pragma unroll
     for (int r = 0; r < 4; ++r) acc[j][r] = __builtin_fmaf(bb, xs[r], __builtin_fmaf(s, c[r], acc[j][r]));
     if (fetch) {
-      if (j == 0) operands_issue_piece<1>(xaddr, waddr, saddr, nxt, acc[0]);
-      if (j == 1) operands_issue_piece<2>(xaddr, waddr, saddr, nxt, acc[1]);
-      if (j == 2) operands_issue_piece<3>(xaddr, waddr, saddr, nxt, acc[2]);
+      if (j == 0) operands_issue_piece<1, SBROW>(xaddr, waddr, saddr, nxt, acc[0]);
+      if (j == 1) operands_issue_piece<2, SBROW>(xaddr, waddr, saddr, nxt, acc[1]);
+      if (j == 2) operands_issue_piece<3, SBROW>(xaddr, waddr, saddr, nxt, acc[2]);
     }
   }
 }
@@ -306,10 +304,14 @@ struct Params {
   const uint16_t* biases;
   uint16_t* y;
   float* partials;     // [2 * grid][wave][lane][4] fp32
-  uint32_t* counters;  // [row blocks]
+  uint32_t* counters;  // [row blocks of all entries]
   int K, N;
   int stages;          // K / 256
-  int units;           // row blocks * stages
+  int units;           // row blocks * stages (dense form; the gathered form counts its own)
+  // gathered form: x, y [P, .], row p goes through the weights of expert expert_ids[p];
+  // w, scales, biases hold E matrices of [N, .] back to back
+  const int32_t* expert_ids;
+  int P, E;
 };
 
 // Unit range of workgroup i out of n: [units*i/n, units*(i+1)/n)  (units*n < 2^31).
@@ -338,21 +340,123 @@ __device__ __forceinline__ void wait_loads(int n) {
 }
 #undef DFLASH_WAIT_CASE
 
-template <bool ACT_FP16, bool SB_FP16>
+// Reads of the row tables by waves that have direct-to-LDS loads in flight: written out by
+// hand for the same reason as the operand reads (the compiler would wait for all loads).
+__device__ __forceinline__ uint32_t lds_read_u32(uint32_t addr) {
+  uint32_t v;
+  asm volatile("ds_read_b32 %0, %1\n s_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
+  return v;
+}
+__device__ __forceinline__ uint32_t lds_read_u16(uint32_t addr) {
+  uint32_t v;
+  asm volatile("ds_read_u16 %0, %1\n s_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
+  return v;
+}
+__device__ __forceinline__ u32x2_t lds_read_u64(uint32_t addr) {
+  u32x2_t v;
+  asm volatile("ds_read_b64 %0, %1\n s_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
+  return v;
+}
+
+// CHUNK: units per scale/bias chunk (4, or 2 when K is a multiple of 512 only).
+// GATHER: per-expert form.  Rows of x that share an expert are taken 16 at a time as one
+// "entry"; an entry is a matrix problem of its own, [rows, K] x [N, K]^T, and the unit
+// space is that of all entries back to back: virtual row block = entry * RB + row block.
+template <bool ACT_FP16, bool SB_FP16, int CHUNK, bool GATHER>
 __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
   using A = Act<ACT_FP16>;
+  constexpr int SBROW = 8 * CHUNK;              // bytes of scales per row and chunk
+  constexpr int kChunkLoads = CHUNK == 4 ? 2 : 1;  // loads per loader and chunk
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int grid = gridDim.x;
   const uint32_t lds0 = lds_address(lds);
+  const int RB = (p.N + kRows - 1) / kRows;  // row blocks of one matrix
 
-  const int u0 = range_begin(p.units, blockIdx.x, grid);
-  const int u1 = range_begin(p.units, blockIdx.x + 1, grid);
-  if (u0 >= u1) return;
-  const int rb0 = u0 / p.stages, st0 = u0 - rb0 * p.stages;
+  int units = p.units;
+  if (GATHER) {
+    // ---- entry tables (ordinary code: no direct-to-LDS load has been issued yet) ----------
+    uint32_t* t_count = reinterpret_cast<uint32_t*>(lds + kTabOffset + kTabCount);
+    uint32_t* t_entry = reinterpret_cast<uint32_t*>(lds + kTabOffset + kTabEntry);
+    uint16_t* t_rows = reinterpret_cast<uint16_t*>(lds + kTabOffset + kTabRows);
+    uint32_t* t_total = reinterpret_cast<uint32_t*>(lds + kTabOffset + kTabTotal);
+    // Every workgroup builds the same tables: a row's place among the rows of its expert is
+    // its rank by row index, not the order in which threads happen to get there (partial
+    // tiles of one row block come from several workgroups and must agree on the rows).
+    for (int e = tid; e < p.E; e += kThreads) t_count[e] = 0;
+    int my_e = -1;
+    if (tid < p.P) {
+      const int e = p.expert_ids[tid];
+      if (e >= 0 && e < p.E) my_e = e;
+      t_entry[tid] = (uint32_t)my_e;  // the ids, until the entries are written below
+    }
+    __syncthreads();
+    int my_pos = 0;
+    if (my_e >= 0) {
+      atomicAdd(&t_count[my_e], 1u);
+      for (int j = 0; j < tid; ++j) my_pos += (t_entry[j] == (uint32_t)my_e) ? 1 : 0;
+    }
+    __syncthreads();
+    if (wave == 0) {
+      // exclusive scan of ceil(rows / 16) over the experts: first entry of each expert
+      int carry = 0;
+      for (int base = 0; base < p.E; base += 64) {
+        const int e = base + lane;
+        const int rows = e < p.E ? (int)t_count[e] : 0;
+        const int n = (rows + 15) >> 4;
+        int incl = n;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const int up = __shfl_up(incl, d, 64);
+          if (lane >= d) incl += up;
+        }
+        if (e < p.E) t_count[e] = ((uint32_t)rows << 16) | (uint32_t)(carry + incl - n);
+        carry += __shfl(incl, 63, 64);
+      }
+      if (lane == 0) *t_total = (uint32_t)carry;
+    }
+    __syncthreads();
+    if (my_e >= 0) {
+      const uint32_t c = t_count[my_e];
+      const int rows = (int)(c >> 16), first = (int)(c & 0xFFFFu);
+      const int ent = first + (my_pos >> 4), m = my_pos & 15;
+      t_rows[ent * 16 + m] = (uint16_t)tid;
+      if (m == 0) {
+        const int left_rows = rows - (my_pos & ~15);
+        t_entry[ent] = ((uint32_t)(left_rows < 16 ? left_rows : 16) << 16) | (uint32_t)my_e;
+      }
+    }
+    __syncthreads();
+    units = (int)*t_total * RB * p.stages;
+  }
+
+  // Workgroups beyond the number of units leave; the others divide the units among
+  // themselves, so every one of them has work and every contributor of a row block arrives.
+  const int grid = (int)gridDim.x < units ? (int)gridDim.x : units;
+  if ((int)blockIdx.x >= grid) return;
+  const int u0 = range_begin(units, blockIdx.x, grid);
+  const int u1 = range_begin(units, blockIdx.x + 1, grid);
+  const int rb0 = u0 / p.stages, st0 = u0 - rb0 * p.stages;  // (virtual) row block, stage
+
+  // Where a virtual row block lives: entry, row block inside the matrix, expert, rows.
+  struct Where {
+    int entry, rb, expert, rows;
+  };
+  auto locate = [&](int vrb) __attribute__((always_inline)) -> Where {
+    Where wh;
+    if (GATHER) {
+      wh.entry = vrb / RB;
+      wh.rb = vrb - wh.entry * RB;
+      const uint32_t e = lds_read_u32(lds0 + kTabOffset + kTabEntry + 4 * wh.entry);
+      wh.expert = (int)(e & 0xFFFFu);
+      wh.rows = (int)(e >> 16);
+    } else {
+      wh.entry = 0, wh.rb = vrb, wh.expert = 0, wh.rows = 16;
+    }
+    return wh;
+  };
 
   // Both kinds of wave walk the same units and pass the same barriers:
   //   one before the loop (unit u0 has landed),
@@ -372,34 +476,54 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
     //  x:     8 instructions; instruction i moves group i>>1, k-blocks 2*(i&1) and 2*(i&1)+1:
     //         lane = 16*(2*kbl + j) + m fetches x[m][64g + 16*(2*(i&1) + kbl) + 8j .. +7],
     //         64 contiguous bytes per row; loader l issues i = l, l+4
-    //  scales/biases of a chunk: 4 + 4 instructions of 32 rows, two 16-byte granules per
-    //         row; loader l issues scales and biases of rows 32l..32l+31
+    //  scales/biases of a chunk, CHUNK = 4: 4 + 4 instructions of 32 rows, two 16-byte
+    //         granules per row; loader l issues scales and biases of rows 32l..32l+31
+    //         CHUNK = 2: 2 + 2 instructions of 64 rows, one granule per row; loaders 0, 1
+    //         issue the scales of rows 0..63, 64..127, loaders 2, 3 the biases
     const int ld = wave - kWaves;
     const int G = p.K / kGS;
     const size_t row_bytes = (size_t)p.K >> 1;
     const int w_r = lane >> 3;
     const int w_c = (lane & 7) ^ (((w_r >> 1) & 3) << 1);
-    const char* xp[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int xi = ld + 4 * i;
-      xp[i] = (const char*)(p.x + (size_t)(lane & 15) * p.K + (xi >> 1) * kGS +
-                            (2 * (xi & 1) + (lane >> 5)) * 16 + ((lane >> 4) & 1) * 8);
-    }
+    const char* xp[2];   // x of this lane's row at stage 0
     const char* wp[4];   // codes of this lane's rows at stage 0 of the row block being issued
-    const char* sbp[2];  // scales, biases of this lane's row, chunk 0
-    auto set_row_block = [&](int rb) __attribute__((always_inline)) {
-      const int row0 = rb * kRows;
+    const char* sbp[2];  // scales / biases of this lane's row, chunk 0 (CHUNK = 2: [0] only)
+    auto set_row_block = [&](int vrb) __attribute__((always_inline)) {
+      const Where wh = locate(vrb);
+      const int row0 = wh.rb * kRows;
+      const uint32_t* wmat = p.w + (size_t)wh.expert * p.N * (row_bytes >> 2);
+      const uint16_t* smat = p.scales + (size_t)wh.expert * p.N * G;
+      const uint16_t* bmat = p.biases + (size_t)wh.expert * p.N * G;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         int row = row0 + 8 * (ld + 4 * i) + w_r;
         row = row < p.N ? row : p.N - 1;
-        wp[i] = (const char*)p.w + (size_t)row * row_bytes + w_c * 16;
+        wp[i] = (const char*)wmat + (size_t)row * row_bytes + w_c * 16;
       }
-      int row = row0 + 32 * ld + (lane >> 1);
-      row = row < p.N ? row : p.N - 1;
-      sbp[0] = (const char*)(p.scales + (size_t)row * G) + (lane & 1) * 16;
-      sbp[1] = (const char*)(p.biases + (size_t)row * G) + (lane & 1) * 16;
+      if (CHUNK == 4) {
+        int row = row0 + 32 * ld + (lane >> 1);
+        row = row < p.N ? row : p.N - 1;
+        sbp[0] = (const char*)(smat + (size_t)row * G) + (lane & 1) * 16;
+        sbp[1] = (const char*)(bmat + (size_t)row * G) + (lane & 1) * 16;
+      } else {
+        int row = row0 + 64 * (ld & 1) + lane;
+        row = row < p.N ? row : p.N - 1;
+        sbp[0] = (const char*)(((ld & 2) ? bmat : smat) + (size_t)row * G);
+        sbp[1] = sbp[0];
+      }
+      // rows of x: the entry's rows in the order of its table; surplus rows of the MFMA tile
+      // repeat the entry's first row (their results are never stored)
+      int xrow = lane & 15;
+      if (GATHER) {
+        const int m = xrow < wh.rows ? xrow : 0;
+        xrow = (int)lds_read_u16(lds0 + kTabOffset + kTabRows + 2 * (wh.entry * 16 + m));
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int xi = ld + 4 * i;
+        xp[i] = (const char*)(p.x + (size_t)xrow * p.K + (xi >> 1) * kGS +
+                              (2 * (xi & 1) + (lane >> 5)) * 16 + ((lane >> 4) & 1) * 8);
+      }
     };
 
     int rb_i = rb0, st_i = st0;  // next unit to issue
@@ -407,15 +531,19 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
     int slot_i = 0;     // ring slot of the next unit to issue
     int sb_slot_i = 0;  // scale/bias slot of the next chunk to issue
     set_row_block(rb_i);
-    // Issues one unit: 6 loads (2 for x, 4 for codes), plus 2 with the first unit of every
-    // scale/bias chunk and with the first unit of the range.
+    // Issues one unit: 6 loads (2 for x, 4 for codes), plus kChunkLoads with the first unit
+    // of every scale/bias chunk and with the first unit of the range.
     auto issue_next = [&]() __attribute__((always_inline)) {
       char* slot = lds + slot_i * kSlotBytes;
-      if ((st_i % kChunk) == 0 || issued == u0) {
-        char* sb = lds + kSbOffset + sb_slot_i * kSbSlotBytes + ld * 1024;
-        const size_t off = (size_t)(st_i / kChunk) * (kChunk * kGroups * 2);
-        load16_to_lds(sbp[0] + off, sb);
-        load16_to_lds(sbp[1] + off, sb + kSbArrayBytes);
+      if ((st_i % CHUNK) == 0 || issued == u0) {
+        char* sb = lds + kSbOffset + sb_slot_i * kSbSlotBytes;
+        const size_t off = (size_t)(st_i / CHUNK) * (CHUNK * kGroups * 2);
+        if (CHUNK == 4) {
+          load16_to_lds(sbp[0] + off, sb + ld * 1024);
+          load16_to_lds(sbp[1] + off, sb + kSbArrayBytes + ld * 1024);
+        } else {
+          load16_to_lds(sbp[0] + off, sb + (ld >> 1) * kSbArrayBytes + (ld & 1) * 1024);
+        }
         if (++sb_slot_i == kSbDepth) sb_slot_i = 0;
       }
 #pragma unroll
@@ -433,9 +561,9 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       }
     };
     // Loads this loader has issued for units u0..v.  Unit indices are global and the number
-    // of stages is a multiple of kChunk, so a unit starts a chunk iff its index is one.
+    // of stages is a multiple of CHUNK, so a unit starts a chunk iff its index is one.
     auto loads_through = [&](int v) __attribute__((always_inline)) -> int {
-      return 6 * (v - u0 + 1) + 2 * (1 + (v / kChunk) - (u0 / kChunk));
+      return 6 * (v - u0 + 1) + kChunkLoads * (1 + (v / CHUNK) - (u0 / CHUNK));
     };
     // Waits until this loader's part of unit v has landed (loads retire in issue order).
     auto wait_unit = [&](int v) __attribute__((always_inline)) {
@@ -490,14 +618,14 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
   const uint32_t wrow = 64 * half + col;
   const uint32_t woff =
       lds0 + wrow * 128 + ((grp ^ ((wrow >> 1) & 3)) << 5) + (kblk >> 1) * 16 + (kblk & 1) * 8;
-  // scale of that row: 32 bytes per row and chunk, four 16-bit values per unit; tile j is
-  // 512 bytes further, biases one array further
-  const uint32_t soff = lds0 + kSbOffset + wrow * 32 + grp * 2;
+  // scale of that row: SBROW bytes per row and chunk, four 16-bit values per unit; tile j is
+  // 16 rows further, biases one array further
+  const uint32_t soff = lds0 + kSbOffset + wrow * SBROW + grp * 2;
 
   // reading position: the unit whose operands are fetched next
   int rd_slot = 0;   // byte offset of its ring slot
   int rd_sb = -kSbSlotBytes;  // byte offset of its scale/bias slot
-  int rd_q = st0 % kChunk;    // its stage within the chunk
+  int rd_q = st0 % CHUNK;     // its stage within the chunk
   bool rd_first = true;
   f32x4_t acc4[4];
 #pragma unroll
@@ -517,15 +645,34 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
     rd_s = soff + rd_sb + rd_q * 8;
     rd_slot += kSlotBytes;
     if (rd_slot == kDepth * kSlotBytes) rd_slot = 0;
-    rd_q = (rd_q + 1) & (kChunk - 1);
+    rd_q = (rd_q + 1) & (CHUNK - 1);
+  };
+
+  // Output of a finished tile: accumulator r of lane l is (m = 4*(l/16) + r, n = 16*wave + l%16)
+  // of the row block; in the gathered form m is a position in the entry's row table.
+  auto emit = [&](int vrb, const f32x4_t& acc) __attribute__((always_inline)) {
+    const Where wh = locate(vrb);
+    const int n_out = wh.rb * kRows + 16 * wave + col;
+    if (n_out >= p.N) return;
+    if (GATHER) {
+      const u32x2_t rr = lds_read_u64(lds0 + kTabOffset + kTabRows + 2 * (wh.entry * 16 + 4 * kblk));
+      const uint32_t rows4[4] = {rr.x & 0xFFFFu, rr.x >> 16, rr.y & 0xFFFFu, rr.y >> 16};
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (4 * kblk + r < wh.rows) p.y[(size_t)rows4[r] * p.N + n_out] = (uint16_t)A::from_f32(acc[r]);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) p.y[(size_t)(4 * kblk + r) * p.N + n_out] = (uint16_t)A::from_f32(acc[r]);
+    }
   };
 
   asm volatile("s_barrier" ::: "memory");
   next_addresses();
-  operands_issue_piece<0>(rd_x, rd_w, rd_s, op[0], acc4[0]);
-  operands_issue_piece<1>(rd_x, rd_w, rd_s, op[0], acc4[0]);
-  operands_issue_piece<2>(rd_x, rd_w, rd_s, op[0], acc4[0]);
-  operands_issue_piece<3>(rd_x, rd_w, rd_s, op[0], acc4[0]);
+  operands_issue_piece<0, SBROW>(rd_x, rd_w, rd_s, op[0], acc4[0]);
+  operands_issue_piece<1, SBROW>(rd_x, rd_w, rd_s, op[0], acc4[0]);
+  operands_issue_piece<2, SBROW>(rd_x, rd_w, rd_s, op[0], acc4[0]);
+  operands_issue_piece<3, SBROW>(rd_x, rd_w, rd_s, op[0], acc4[0]);
   operands_wait(op[0], acc4[0], acc4[1], acc4[2], acc4[3]);
 
   int left = u1 - u0;            // units still to consume, the current one included
@@ -544,7 +691,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       asm volatile("s_barrier" ::: "memory");
       const bool fetch = left > 1;
       if (fetch) next_addresses();
-      consume_unit<ACT_FP16, SB_FP16>(cur, nxt, fetch, rd_x, rd_w, rd_s, acc4, ones, mask, magic);
+      consume_unit<ACT_FP16, SB_FP16, SBROW>(cur, nxt, fetch, rd_x, rd_w, rd_s, acc4, ones, mask, magic);
       if (fetch) operands_wait(nxt, acc4[0], acc4[1], acc4[2], acc4[3]);
       --left;
       ++in_rb;
@@ -557,14 +704,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc4[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         if (in_rb == p.stages) {
-          // the whole row block was mine: accumulator r of lane l is output
-          // (m = 4*(l/16) + r, n = row0 + 16*wave + l%16)
-          const int n_out = rb * kRows + 16 * wave + col;
-          if (n_out < p.N) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-              p.y[(size_t)(4 * kblk + r) * p.N + n_out] = (uint16_t)A::from_f32(acc[r]);
-          }
+          emit(rb, acc);  // the whole row block was mine
         } else {
           // Other workgroups hold the rest of this row block.  A workgroup shares at most two
           // row blocks: the one its range starts in (partial slot 0) and the one it ends in
@@ -596,8 +736,8 @@ arrive:
     // contributors of a row block: the workgroups whose ranges intersect [lo, lo+stages);
     // owner(v) = ceil((v+1)*grid/units) - 1 is the workgroup whose range holds unit v
     const int lo = shared_rb[i] * p.stages;
-    wg_lo[i] = (int)((((unsigned)lo + 1u) * (unsigned)grid + p.units - 1) / (unsigned)p.units) - 1;
-    wg_hi[i] = (int)((((unsigned)(lo + p.stages)) * (unsigned)grid + p.units - 1) / (unsigned)p.units) - 1;
+    wg_lo[i] = (int)((((unsigned)lo + 1u) * (unsigned)grid + units - 1) / (unsigned)units) - 1;
+    wg_hi[i] = (int)((((unsigned)(lo + p.stages)) * (unsigned)grid + units - 1) / (unsigned)units) - 1;
   }
   if (tid == 0) {
     uint32_t prev[2] = {0u, 0u}, flag[2];
@@ -629,7 +769,7 @@ arrive:
     // first contributor can have started before this row block (then the block is the one
     // its range ends in, slot 1); every later one starts inside it (slot 0).
     const int lo = shared_rb[i] * p.stages;
-    const int which_first = range_begin(p.units, wg_lo[i], grid) < lo ? 1 : 0;
+    const int which_first = range_begin(units, wg_lo[i], grid) < lo ? 1 : 0;
     f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
     for (int wg = wg_lo[i]; wg <= wg_hi[i]; wg += 8) {
       const float* src[8];
@@ -648,11 +788,7 @@ arrive:
         }
       }
     }
-    const int n_out = shared_rb[i] * kRows + 16 * wave + col;
-    if (n_out < p.N) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) p.y[(size_t)(4 * kblk + r) * p.N + n_out] = (uint16_t)A::from_f32(acc[r]);
-    }
+    emit(shared_rb[i], acc);
   }
 }
 
@@ -677,11 +813,20 @@ int qmm_stream_grid() {
 }
 
 bool qmm_stream_eligible(int K, int N, int group_size) {
-  // whole scale/bias chunks: K must be a multiple of kChunk units
-  if (group_size != 64 || K <= 0 || K % (stream::kUnitK * stream::kChunk) != 0 || N <= 0 || N % 16 != 0) return false;
+  // whole scale/bias chunks: K must be a multiple of two units
+  if (group_size != 64 || K <= 0 || K % (stream::kUnitK * 2) != 0 || N <= 0 || N % 16 != 0) return false;
   const long long row_blocks = (N + stream::kRows - 1) / stream::kRows;
   const long long units = row_blocks * (K / stream::kUnitK);
   return units * 1024 < (1ll << 31) && row_blocks <= (64 * 1024) / 4;
+}
+
+bool qmm_stream_gather_eligible(int P, int K, int N, int E, int group_size) {
+  if (!qmm_stream_eligible(K, N, group_size)) return false;
+  const long long row_blocks = (N + stream::kRows - 1) / stream::kRows;
+  // every row could be an entry of its own
+  return P > 0 && P <= stream::kMaxEntries && E > 0 && E <= stream::kMaxExperts &&
+         row_blocks * stream::kMaxEntries <= (64 * 1024) / 4 &&
+         row_blocks * stream::kMaxEntries * (K / stream::kUnitK) * 1024 < (1ll << 31);
 }
 
 size_t qmm_stream_workspace_bytes(int N, int grid) {
@@ -689,11 +834,46 @@ size_t qmm_stream_workspace_bytes(int N, int grid) {
   return (size_t)64 * 1024 + (size_t)grid * 2 * stream::kPartialFloats * sizeof(float);
 }
 
+namespace {
+template <bool GATHER>
+const void* stream_kernel_for(bool a16, bool s16, bool chunk4) {
+  using namespace stream;
+#define DFLASH_STREAM_PICK(A16, S16)                                                      \
+  if (a16 == A16 && s16 == S16)                                                           \
+    return chunk4 ? (const void*)qmm_stream_kernel<A16, S16, 4, GATHER>                   \
+                  : (const void*)qmm_stream_kernel<A16, S16, 2, GATHER>;
+  DFLASH_STREAM_PICK(false, false)
+  DFLASH_STREAM_PICK(false, true)
+  DFLASH_STREAM_PICK(true, false)
+  DFLASH_STREAM_PICK(true, true)
+#undef DFLASH_STREAM_PICK
+  return nullptr;
+}
+
+int launch_stream(stream::Params& p, bool gather, int grid, int act_dtype, int sb_dtype,
+                  hipStream_t stream) {
+  using namespace stream;
+  const bool a16 = act_dtype == DFLASH_FP16, s16 = sb_dtype == DFLASH_FP16;
+  const bool chunk4 = p.K % (kUnitK * 4) == 0;
+  const void* fn = gather ? stream_kernel_for<true>(a16, s16, chunk4) : stream_kernel_for<false>(a16, s16, chunk4);
+  const int lds_bytes = gather ? kLdsBytesGather : kLdsBytes;
+  static bool attr_set[16] = {};
+  const int idx = (gather ? 8 : 0) + (chunk4 ? 4 : 0) + (a16 ? 2 : 0) + (s16 ? 1 : 0);
+  if (!attr_set[idx]) {
+    DFLASH_HIP_OK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
+    attr_set[idx] = true;
+  }
+  void* args[] = {&p};
+  DFLASH_HIP_OK(hipLaunchKernel(fn, dim3(grid), dim3(kThreads), args, lds_bytes, stream));
+  return DFLASH_OK;
+}
+}  // namespace
+
 int qmm_stream_launch(const void* x, const uint32_t* w, const void* scales, const void* biases,
                       void* y, void* workspace, size_t workspace_bytes, int K, int N,
                       int act_dtype, int sb_dtype, hipStream_t stream) {
   using namespace stream;
-  Params p;
+  Params p{};
   p.x = (const uint16_t*)x;
   p.w = w;
   p.scales = (const uint16_t*)scales;
@@ -711,22 +891,36 @@ int qmm_stream_launch(const void* x, const uint32_t* w, const void* scales, cons
                  workspace ? workspace_bytes : (size_t)0);
   p.counters = (uint32_t*)workspace;
   p.partials = (float*)((char*)workspace + 64 * 1024);
+  return launch_stream(p, false, grid, act_dtype, sb_dtype, stream);
+}
 
-  static bool attr_set[4] = {false, false, false, false};
-  const bool a16 = act_dtype == DFLASH_FP16, s16 = sb_dtype == DFLASH_FP16;
-  const int idx = (a16 ? 2 : 0) + (s16 ? 1 : 0);
-  const void* fn = nullptr;
-  if (!a16 && !s16) fn = (const void*)qmm_stream_kernel<false, false>;
-  if (!a16 && s16) fn = (const void*)qmm_stream_kernel<false, true>;
-  if (a16 && !s16) fn = (const void*)qmm_stream_kernel<true, false>;
-  if (a16 && s16) fn = (const void*)qmm_stream_kernel<true, true>;
-  if (!attr_set[idx]) {
-    DFLASH_HIP_OK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));
-    attr_set[idx] = true;
-  }
-  void* args[] = {&p};
-  DFLASH_HIP_OK(hipLaunchKernel(fn, dim3(grid), dim3(kThreads), args, kLdsBytes, stream));
-  return DFLASH_OK;
+int qmm_stream_gather_launch(const void* x, const int32_t* expert_ids, const uint32_t* w,
+                             const void* scales, const void* biases, void* y, void* workspace,
+                             size_t workspace_bytes, int P, int K, int N, int E, int act_dtype,
+                             int sb_dtype, hipStream_t stream) {
+  using namespace stream;
+  Params p{};
+  p.x = (const uint16_t*)x;
+  p.w = w;
+  p.scales = (const uint16_t*)scales;
+  p.biases = (const uint16_t*)biases;
+  p.y = (uint16_t*)y;
+  p.K = K;
+  p.N = N;
+  p.stages = K / kUnitK;
+  p.units = 0;  // counted on the device from the routing
+  p.expert_ids = expert_ids;
+  p.P = P;
+  p.E = E;
+  // the number of entries is not known here: a full grid, workgroups without units leave
+  const int grid = qmm_stream_grid();
+  const size_t need = qmm_stream_workspace_bytes(N, grid);
+  DFLASH_REQUIRE(workspace && workspace_bytes >= need, DFLASH_ERR_WORKSPACE,
+                 "dflash_qmm_m16_gather: workspace of %zu bytes needed, %zu given", need,
+                 workspace ? workspace_bytes : (size_t)0);
+  p.counters = (uint32_t*)workspace;
+  p.partials = (float*)((char*)workspace + 64 * 1024);
+  return launch_stream(p, true, grid, act_dtype, sb_dtype, stream);
 }
 
 }  // namespace dflash

@@ -170,8 +170,15 @@ def gather_qmm(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: t
         raise ValueError("one expert id per row of x is required")
     y = torch.empty((P, N), dtype=x2.dtype, device=x2.device)
     stream = torch.cuda.current_stream(x2.device).cuda_stream
+    # DFLASH_QMM_KERNEL=tile keeps the streaming kernel out of the gathered form as well
+    need = 0 if _kernel_select() == _native.QMM_KERNEL_TILE else \
+        lib.dflash_qmm_m16_gather_workspace_bytes(P, K, N, E, group_size)
+    ws_ptr, ws_bytes = None, 0
+    if need:
+        ws = _workspace(x2.device, stream, need)
+        ws_ptr, ws_bytes = ws.data_ptr(), ws.numel() * ws.element_size()
     rc = lib.dflash_qmm_m16_gather(x2.data_ptr(), ids.data_ptr(), w_q.data_ptr(), scales.data_ptr(),
-                                   biases.data_ptr(), y.data_ptr(), P, K, N, E, group_size,
-                                   _DTYPE_CODE[x2.dtype], _DTYPE_CODE[scales.dtype], stream)
+                                   biases.data_ptr(), y.data_ptr(), ws_ptr, ws_bytes, P, K, N, E,
+                                   group_size, _DTYPE_CODE[x2.dtype], _DTYPE_CODE[scales.dtype], stream)
     _native.check(rc, "dflash_qmm_m16_gather")
     return y.reshape(*x.shape[:-1], N)

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 2
+#define DFLASH_ABI_VERSION 3
 
 enum {
   DFLASH_OK = 0,
@@ -45,7 +45,7 @@ enum { DFLASH_QMM_MMA2BIG = 0, DFLASH_QMM_MMA2BIG_PIPE = 1 };
  * Which device kernel serves a qmm call.  TILE: one workgroup per 32 output columns and
  * per K slice, K cut into k_parts slices for the pipe variant.  STREAM: persistent
  * workgroups that divide the weight matrix evenly and stream it through LDS; needs
- * group_size 64 and K % 1024 == 0, and decides the K split itself (variant and k_parts
+ * group_size 64 and K % 512 == 0, and decides the K split itself (variant and k_parts
  * then only name the caller's dispatch decision).  AUTO: STREAM where it applies.
  */
 enum { DFLASH_QMM_KERNEL_AUTO = 0, DFLASH_QMM_KERNEL_TILE = 1, DFLASH_QMM_KERNEL_STREAM = 2 };
@@ -91,12 +91,23 @@ int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* scales, const
  *
  *   x [P, K] act_dtype      expert_ids [P] int32 in [0, E)
  *   w_q [E, N, K/8] uint32  scales, biases [E, N, K/group_size] sb_dtype     y [P, N] act_dtype
+ *   workspace               optional (may be NULL): >= dflash_qmm_m16_gather_workspace_bytes(...)
+ *                           bytes, same rules as the workspace of dflash_qmm_m16 (zero-filled
+ *                           once, reusable, shareable with it).  With a workspace, calls with
+ *                           group_size 64, K % 512 == 0, P <= 256 and E <= 1024 are served by
+ *                           the streaming kernel: the weights of the experts that have rows
+ *                           are streamed through LDS by persistent workgroups, as for the
+ *                           dense form.  Without one, or for other shapes, one workgroup per
+ *                           (32 columns, expert) reads its weights directly.
  * Requirements: P <= 2048, group_size in {32,64,128}, N % 16 == 0, K % group_size == 0.
- * Rows whose expert id is outside [0, E) are left unwritten.
+ * Rows whose expert id is outside [0, E) are left unwritten.  Deterministic.
  */
+size_t dflash_qmm_m16_gather_workspace_bytes(int P, int K, int N, int E, int group_size);
+
 int dflash_qmm_m16_gather(const void* x, const int32_t* expert_ids, const uint32_t* w_q,
-                          const void* scales, const void* biases, void* y, int P, int K, int N,
-                          int E, int group_size, int act_dtype, int sb_dtype, void* stream);
+                          const void* scales, const void* biases, void* y, void* workspace,
+                          size_t workspace_bytes, int P, int K, int N, int E, int group_size,
+                          int act_dtype, int sb_dtype, void* stream);
 
 /*
  * GatedDeltaNet tape replay: for every slot s and value head hv apply the first

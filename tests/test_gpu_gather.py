@@ -13,6 +13,14 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+@pytest.fixture(autouse=True, params=["auto", "tile"])
+def kernel_mode(request, monkeypatch):
+    """Every test runs once with the streaming kernel where it applies (auto: group 64,
+    K % 512 == 0, at most 256 rows) and once with the per-(columns, expert) kernel forced."""
+    monkeypatch.setenv("DFLASH_QMM_KERNEL", request.param)
+    return request.param
+
+
 def _check(case, y):
     xf = case.x.float().numpy()
     exact = O.qmm_gather_exact(xf, case.expert_ids.numpy(), case.w.numpy().view(np.uint32),
@@ -48,12 +56,69 @@ def test_more_than_sixteen_rows_per_expert_and_unused_experts(native_lib):
     assert torch.equal(one[0], y[7])
 
 
+@pytest.mark.parametrize("K,N,E,rows", [
+    (1024, 272, 5, (37, 0, 0, 40, 23)),      # > 16 rows per expert, ragged last row block, CHUNK 4
+    (1536, 128, 7, (1, 16, 17, 0, 33, 15, 2)),  # K a multiple of 512 only: CHUNK 2
+    (512, 640, 3, (250, 1, 5)),              # 256 rows, nearly all on one expert
+    (2048, 16, 300, None),                   # one row block of 16 columns, many experts
+])
+def test_streamed_shapes_and_row_tables(native_lib, K, N, E, rows):
+    g = torch.Generator().manual_seed(K + N)
+    if rows is None:
+        ids = torch.randint(0, E, (200,), generator=g, dtype=torch.int32)
+    else:
+        ids = torch.cat([torch.full((n,), e, dtype=torch.int32) for e, n in enumerate(rows)])
+        ids = ids[torch.randperm(ids.numel(), generator=g)]
+    case = make_moe_case(K, N, 5 + K, experts=E, tokens=ids.numel(), top_k=1)
+    case.expert_ids = ids
+    d = case.to(DEV)
+    y = gather_qmm(d.x, d.w, d.scales, d.biases, d.expert_ids, group_size=64)
+    _check(case, y)
+    assert torch.equal(y, gather_qmm(d.x, d.w, d.scales, d.biases, d.expert_ids, group_size=64))
+    # a row's result does not depend on which other rows share the call
+    j = ids.numel() // 2
+    one = gather_qmm(d.x[j:j + 1], d.w, d.scales, d.biases, d.expert_ids[j:j + 1], group_size=64)
+    assert torch.equal(one[0], y[j])
+
+
+def test_rows_with_invalid_expert_ids_are_left_alone(native_lib, kernel_mode):
+    """Straight through the C ABI, so that y can be pre-filled."""
+    import ctypes
+    L = native_lib
+    K, N, E, P = 1024, 256, 4, 24
+    case = make_moe_case(K, N, 31, experts=E, tokens=P, top_k=1)
+    ids = case.expert_ids.clone()
+    ids[3], ids[10], ids[23] = -1, E, 1 << 20
+    case.expert_ids = ids
+    d = case.to(DEV)
+    y = torch.full((P, N), 7.0, dtype=torch.bfloat16, device=DEV)
+    need = 0 if kernel_mode == "tile" else L.dflash_qmm_m16_gather_workspace_bytes(P, K, N, E, 64)
+    assert (need > 0) == (kernel_mode == "auto")
+    ws = torch.zeros(max(need, 16), dtype=torch.uint8, device=DEV)
+    for _ in range(2):  # the workspace is handed back reusable
+        rc = L.dflash_qmm_m16_gather(d.x.data_ptr(), d.expert_ids.data_ptr(), d.w.data_ptr(),
+                                     d.scales.data_ptr(), d.biases.data_ptr(), y.data_ptr(),
+                                     ws.data_ptr() if need else None, need, P, K, N, E, 64, 0, 0, None)
+        assert rc == 0, L.dflash_last_error()
+        torch.cuda.synchronize()
+    bad = [3, 10, 23]
+    assert torch.all(y[bad] == 7.0)
+    good = [i for i in range(P) if i not in bad]
+    sub = make_moe_case(K, N, 31, experts=E, tokens=P, top_k=1)
+    exact = O.qmm_gather_exact(sub.x.float().numpy()[good], ids.numpy()[good], sub.w.numpy().view(np.uint32),
+                               sub.scales.float().numpy(), sub.biases.float().numpy(), 64)
+    got = y[good].float().cpu().numpy()
+    assert np.linalg.norm(got - exact) / np.linalg.norm(exact) <= 5e-3
+    assert L.dflash_qmm_m16_gather_workspace_bytes(4096, K, N, E, 64) == 0   # too many rows to stream
+    assert L.dflash_qmm_m16_gather_workspace_bytes(P, K, N, E, 32) == 0      # group size
+
+
 def test_argument_checks(native_lib):
     L = native_lib
-    assert L.dflash_qmm_m16_gather(None, None, None, None, None, None, 1, 64, 32, 2, 64, 0, 0, None) == -1
+    assert L.dflash_qmm_m16_gather(None, None, None, None, None, None, None, 0, 1, 64, 32, 2, 64, 0, 0, None) == -1
     import ctypes
     one = ctypes.c_void_p(256)
-    assert L.dflash_qmm_m16_gather(one, one, one, one, one, one, 4096, 64, 32, 2, 64, 0, 0, None) == -2
+    assert L.dflash_qmm_m16_gather(one, one, one, one, one, one, None, 0, 4096, 64, 32, 2, 64, 0, 0, None) == -2
     assert b"at most" in L.dflash_last_error()
     with pytest.raises(nat.NativeLibraryError):
         c = make_moe_case(64, 32, 1, experts=2, tokens=2, top_k=1)

@@ -71,7 +71,8 @@ def test_config0_single_call(verify_env, native_lib, c_oracle):
     assert np.max(np.abs(y - O.round_bf16(exact.astype(np.float32)))) <= 2 ** -7 * np.max(np.abs(exact))
 
 
-@pytest.mark.parametrize("K,N", [(5120, 17408), (17408, 5120), (5120, 7168), (4096, 12288)])
+@pytest.mark.parametrize("K,N", [(5120, 17408), (17408, 5120), (5120, 7168), (4096, 12288),
+                                 (512, 2048), (1536, 272)])  # the last two: K a multiple of 512 only
 def test_real_projection_shapes(verify_env, native_lib, c_oracle, K, N):
     """27B / 9B projection shapes at full size, both dispatch branches."""
     case = make_qmm_case(K, N, seed_for(3, K % 97))

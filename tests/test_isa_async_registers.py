@@ -29,26 +29,40 @@ def _regs(text):
 
 
 def scan(asm_text):
-    """Returns (number of LDS reads seen, list of offending lines)."""
-    pending, bad, reads = set(), [], 0
+    """Returns (number of LDS reads seen, list of offending lines).
+
+    LDS operations complete in issue order, so after `s_waitcnt lgkmcnt(n)` only the n most
+    recent ones can still be outstanding; scalar memory operations share the counter and are
+    counted as if they were LDS operations, which errs on the side of flagging."""
+    pending, bad, reads = [], [], 0   # pending: destination registers per outstanding operation
     for no, line in enumerate(asm_text.split("\n"), 1):
         t = line.split(";")[0].strip()
         if not t or t.startswith(".") or t.endswith(":"):
             continue
-        if t.startswith("ds_read") or t.startswith("ds_bpermute"):
-            ops = t.split(None, 1)[1].split(",")
-            if _regs(",".join(ops[1:])) & pending:
+        busy = set().union(*pending) if pending else set()
+        op = t.split(None, 1)[0]
+        if op.startswith("ds_"):
+            ops = t.split(None, 1)[1].split(",") if " " in t else []
+            returns = op.startswith("ds_read") or op.startswith("ds_bpermute") or "_rtn" in op
+            srcs = ops[1:] if returns else ops
+            if _regs(",".join(srcs)) & busy:
                 bad.append((no, t))
-            pending |= _regs(ops[0])
-            reads += 1
+            pending.append(_regs(ops[0]) if returns else set())
+            reads += 1 if op.startswith("ds_read") else 0
             continue
-        if t.startswith("s_waitcnt") and "lgkmcnt(0)" in t:
-            pending = set()
+        if op.startswith(("s_load", "s_buffer_load", "s_memtime", "s_memrealtime")):
+            pending.append(set())
             continue
-        if t.startswith("s_endpgm"):
-            pending = set()
+        if op == "s_waitcnt":
+            m = re.search(r"lgkmcnt\((\d+)\)", t)
+            if m:
+                n = int(m.group(1))
+                pending = pending[-n:] if n > 0 else []
             continue
-        if _regs(t) & pending:
+        if op == "s_endpgm":
+            pending = []
+            continue
+        if _regs(t) & busy:
             bad.append((no, t))
     return reads, bad
 
@@ -61,6 +75,10 @@ def test_scanner_flags_a_premature_use():
     assert reads == 1 and len(bad) == 1 and "v_mov_b32" in bad[0][1]
     partial = "ds_read_b64 v[4:5], v1\ns_waitcnt lgkmcnt(1)\nv_mov_b32 v9, v4\n"
     assert len(scan(partial)[1]) == 1
+    in_order = "ds_read_b32 v4, v1\nds_read_b32 v5, v1\ns_waitcnt lgkmcnt(1)\nv_mov_b32 v9, v4\n"
+    assert scan(in_order) == (2, [])
+    too_early = "ds_read_b32 v4, v1\nds_read_b32 v5, v1\ns_waitcnt lgkmcnt(1)\nv_mov_b32 v9, v5\n"
+    assert len(scan(too_early)[1]) == 1
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not available")
@@ -73,7 +91,7 @@ def test_no_instruction_touches_registers_of_reads_in_flight():
         subprocess.run(cmd, check=True, capture_output=True, timeout=600)
         text = open(out).read()
     kernels = re.findall(r"^(_ZN6dflash6stream17qmm_stream_kernel\w+):", text, flags=re.M)
-    assert len(kernels) == 4, kernels
+    assert len(kernels) == 16, kernels  # activation x scale dtype x chunk size x dense|gathered
     for name in kernels:
         body = text[text.index(name + ":"):]
         body = body[:body.index(".Lfunc_end")]
