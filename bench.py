@@ -256,6 +256,51 @@ def bench_replay(device: str, steps: int, warmup: int):
                 steps=T, kv_trim_host_ns_16_layers=trim_ns)
 
 
+def bench_gdn_forward(device: str, steps: int, warmup: int):
+    """The producer of the tape: GatedDeltaNet forward over a block of 16 tokens with the
+    innovation tape recorded, 48 layers x 32 value heads (16 key heads) of 128 x 128 fp32
+    state in one launch, bf16 q/k/v.  Algorithmic bytes per value head: the state once in and
+    once out, v, y (bf16) and the tape (fp32) once, its share of q and k, g and beta."""
+    import torch
+
+    from dflash_mlx_amd.kernels import gated_delta_kernel_with_tape
+
+    L, Hk, Hv, T, D = 48, 16, 32, 16, 128
+    gen = torch.Generator(device=device).manual_seed(0xDF1A + 2500)
+    sets = []
+    for _ in range(4):   # four state sets (400 MB): the Infinity Cache cannot hold them
+        q = torch.randn((L, T, Hk, D), generator=gen, device=device)
+        k = torch.randn((L, T, Hk, D), generator=gen, device=device)
+        q = (q / q.norm(dim=-1, keepdim=True) * D ** -0.5).to(torch.bfloat16)
+        k = (k / k.norm(dim=-1, keepdim=True)).to(torch.bfloat16)
+        v = torch.randn((L, T, Hv, D), generator=gen, device=device).to(torch.bfloat16)
+        g = torch.exp(-torch.nn.functional.softplus(torch.randn((L, T, Hv), generator=gen, device=device)))
+        beta = torch.sigmoid(torch.randn((L, T, Hv), generator=gen, device=device)).to(torch.bfloat16)
+        state = torch.randn((L, Hv, D, D), generator=gen, device=device) * 0.1
+        sets.append((q, k, v, g, beta, state))
+
+    def one_pass(i):
+        return gated_delta_kernel_with_tape(*sets[i % 4])
+
+    for i in range(max(warmup, 4)):
+        one_pass(i)
+    n = max(steps * 10, 40)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for i in range(n):
+        one_pass(i)
+    stop.record()
+    torch.cuda.synchronize()
+    us = start.elapsed_time(stop) / n * 1e3
+    per_head = 2 * D * D * 4 + T * (D * 2 + D * 2 + D * 4 + (Hk * 2 * D * 2) // Hv + 4 + 2)
+    total = per_head * L * Hv
+    del sets
+    torch.cuda.empty_cache()
+    return dict(us_per_forward=us, us_per_layer=us / L, gbps=total / us / 1e3,
+                frac_hbm=total / (us * 1e-6) / HBM_PEAK, bytes=total, layers=L, heads=Hv, steps=T)
+
+
 def bench_cpu_baseline(stack: str, budget_s: float = 12.0):
     """The oracle's C port of the reference kernel arithmetic (bf16-rounded dequantised
     weights, fp32 accumulation) on the host cores: whole layers of the same stack, one
@@ -340,6 +385,9 @@ def main() -> int:
         log(f"[bench] moe: {mo['ms_per_step']:.3f} ms/step, {mo['weight_gbps']:.0f} GB/s")
         rp = bench_replay(device, args.steps, args.warmup)
         extra["gdn_tape_replay"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in rp.items()}
+        fw = bench_gdn_forward(device, args.steps, args.warmup)
+        log(f"forward with tape: {fw['us_per_layer']:.3f} us/layer, {fw['gbps']:.0f} GB/s")
+        extra["gdn_forward_with_tape"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in fw.items()}
         log(f"[bench] replay: {rp['us_per_layer']:.3f} us/layer, {rp['gbps']:.0f} GB/s")
 
     achieved = main_res["bytes_per_launch"] / (main_res["avg_launch_us"] * 1e-6) / 1e9

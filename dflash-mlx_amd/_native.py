@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
@@ -27,6 +27,7 @@ EXPORTED_SYMBOLS = (
     "dflash_qmm_m16_gather_workspace_bytes",
     "dflash_qmm_m16_gather",
     "dflash_tape_replay",
+    "dflash_gdn_forward_tape",
     "dflash_conv_state_rebuild",
 )
 
@@ -56,6 +57,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.dflash_qmm_m16_gather.argtypes = (
         [c.c_void_p] * 7 + [c.c_size_t] + [c.c_int] * 7 + [c.c_void_p]
     )
+    lib.dflash_gdn_forward_tape.restype = c.c_int
+    lib.dflash_gdn_forward_tape.argtypes = [c.c_void_p] * 10 + [c.c_int] * 11 + [c.c_void_p]
     lib.dflash_tape_replay.restype = c.c_int
     lib.dflash_tape_replay.argtypes = (
         [c.c_void_p] * 6 + [c.c_int] + [c.c_void_p] + [c.c_int] * 12 + [c.c_void_p]

@@ -1,0 +1,359 @@
+// GatedDeltaNet forward over a block of T tokens that also records the innovation tape,
+// for gfx950 (MI355X).
+//
+// Counterpart of the reference's `gated_delta_tape{,_vec}{,_mask}` Metal kernels
+// (dflash_mlx/kernels.py:12-127; array-op form :131-173; dispatcher :176-224): for every
+// (batch slot, value head), with the state S[Dv][Dk] (Dk contiguous) and for t = 0..T-1,
+//     S      <- g_t * S                      (g_t a scalar per head, or one value per dk)
+//     kv     =  S k_t                        (a value per dv)
+//     delta  =  (v_t - kv) * beta_t
+//     S      <- S + delta (x) k_t
+//     y_t    =  S q_t
+//     tape_t =  delta                        (fp32)
+// and S rounded through the state dtype after every step (kernels.py:96-98; a no-op for an
+// fp32 state).  A step whose mask byte is zero leaves S alone and gives y_t = tape_t = 0.
+// The tape, with k and g, is what dflash_tape_replay needs to rebuild the state after any
+// prefix of the block.
+//
+// Like the replay, the operation moves the state once in and once out and little else, but
+// it is sequential in t, needs two reductions over dk per step, and at 16 steps its
+// arithmetic costs about as much as its memory traffic.  Layout for 128 x 128 heads: one
+// workgroup of 4 waves per (slot, head); a lane owns 4 rows x 16 columns of S (rows
+// 32*wave + 4*(lane/8) + i; columns 4*(lane%8) + 32*c + {0..3}, c = 0..3), so that
+//  * a row of S is spread over 8 neighbouring lanes: a reduction over dk is three DPP steps,
+//    every lane ends up with the sums and nothing goes through LDS;
+//  * every wave load or store of S is eight runs of 128 contiguous bytes;
+//  * y_t = (g S) q + (k . q) delta, so one pass over S yields both sums of a step and one
+//    reduction round serves both;
+//  * with one gate per head and an fp32 state the decay is not applied to S at all: the
+//    kernel keeps S / c with c = prod g, scales the two sums and delta instead, and
+//    multiplies c back in once at the end (renormalising if c gets very small).
+// q, k, v, g, beta of the block are staged once in LDS as fp32.
+#include "dflash_common.h"
+
+namespace dflash {
+namespace {
+
+constexpr int kThreads = 256;
+
+struct GdnArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* g;
+  const void* beta;
+  const void* state_in;
+  void* state_out;
+  void* y;
+  float* tape;
+  const uint8_t* mask;
+  int T, Hk, Hv, Dk, Dv;
+  int in_dtype, g_dtype, beta_dtype, state_dtype, g_per_dk;
+};
+
+__device__ __forceinline__ void store_from_f32(void* p, size_t i, float v, int dt) {
+  if (dt == DFLASH_BF16) {
+    ((uint16_t*)p)[i] = (uint16_t)f32_to_bf16_bits(v);
+  } else if (dt == DFLASH_FP16) {
+    ((uint16_t*)p)[i] = (uint16_t)f32_to_f16_bits(v);
+  } else {
+    ((float*)p)[i] = v;
+  }
+}
+
+// v + (v of the lane the DPP control names): butterfly steps inside a row of 16 lanes -
+// quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror (lanes of an aligned group of 8),
+// row_mirror (the two groups of 8).
+template <int CTRL>
+__device__ __forceinline__ float add_dpp(float v) {
+  const int o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true);
+  return v + __int_as_float(o);
+}
+__device__ __forceinline__ float sum_over_8(float v) {
+  v = add_dpp<0xB1>(v);
+  v = add_dpp<0x4E>(v);
+  v = add_dpp<0x141>(v);
+  return v;
+}
+__device__ __forceinline__ float sum_over_16(float v) { return add_dpp<0x140>(sum_over_8(v)); }
+
+__device__ __forceinline__ float dot4(const f32x4_t& s, const float4& k) {
+  return s.x * k.x + s.y * k.y + s.z * k.z + s.w * k.w;
+}
+
+// ---------------------------------------------------------------------------
+// Dk = Dv = 128.  LDS (floats): sQ[T][128] | sK[T][128] | sV[T][128] | sG[T][128 or 1] |
+// sBeta[T] | sKQ[T].  FOLD: keep S / prod(g) instead of applying the decay (one gate per
+// head, fp32 state only).
+// ---------------------------------------------------------------------------
+template <bool VECG, bool FOLD>
+__global__ __launch_bounds__(kThreads) void gdn_forward_128(GdnArgs a) {
+  static_assert(!(VECG && FOLD), "the folded decay needs one gate per head");
+  extern __shared__ float smem[];
+  const int T = a.T;
+  float* sQ = smem;
+  float* sK = sQ + T * 128;
+  float* sV = sK + T * 128;
+  float* sG = sV + T * 128;
+  float* sBeta = sG + T * (VECG ? 128 : 1);
+  float* sKQ = sBeta + T;
+
+  const int slot = blockIdx.x / a.Hv, hv = blockIdx.x % a.Hv;
+  const int hk = hv / (a.Hv / a.Hk);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c3 = lane & 7;
+  const int row0 = 32 * wave + 4 * (lane >> 3);  // this lane's rows: row0 .. row0 + 3
+  const size_t slotT = (size_t)slot * T;
+  const bool f32_state = FOLD || a.state_dtype == DFLASH_FP32;
+
+  // ---- state in: float4 columns c3 + 8c (c = 0..3) of 4 rows --------------------------------
+  const size_t sbase = (size_t)blockIdx.x * 128 * 128;
+  f32x4_t st[4][4];
+  if (f32_state) {
+    const f32x4_t* in = reinterpret_cast<const f32x4_t*>((const float*)a.state_in + sbase);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) st[i][c] = __builtin_nontemporal_load(&in[(row0 + i) * 32 + c3 + 8 * c]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          st[i][c][e] = load_as_f32(a.state_in, sbase + (size_t)(row0 + i) * 128 + 4 * (c3 + 8 * c) + e,
+                                    a.state_dtype);
+  }
+
+  // ---- stage the block ---------------------------------------------------------------------
+  for (int i = tid; i < T * 128; i += kThreads) {
+    const int t = i >> 7, d = i & 127;
+    sQ[i] = load_as_f32(a.q, ((slotT + t) * a.Hk + hk) * 128 + d, a.in_dtype);
+    sK[i] = load_as_f32(a.k, ((slotT + t) * a.Hk + hk) * 128 + d, a.in_dtype);
+    sV[i] = load_as_f32(a.v, ((slotT + t) * a.Hv + hv) * 128 + d, a.in_dtype);
+    if (VECG) sG[i] = load_as_f32(a.g, ((slotT + t) * a.Hv + hv) * 128 + d, a.g_dtype);
+  }
+  for (int t = tid; t < T; t += kThreads) {
+    if (!VECG) sG[t] = load_as_f32(a.g, (slotT + t) * a.Hv + hv, a.g_dtype);
+    sBeta[t] = load_as_f32(a.beta, (slotT + t) * a.Hv + hv, a.beta_dtype);
+  }
+  __syncthreads();
+  // k_t . q_t: 16 lanes per step, 8 products each
+  for (int t = tid >> 4; t < T; t += kThreads / 16) {
+    const int c16 = tid & 15;
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) s += sK[t * 128 + 8 * c16 + c] * sQ[t * 128 + 8 * c16 + c];
+    s = sum_over_16(s);
+    if (c16 == 0) sKQ[t] = s;
+  }
+  __syncthreads();
+
+  float cum = 1.f;  // FOLD: the registers hold S / cum
+  const size_t obase = (size_t)slot * T * a.Hv * 128 + (size_t)hv * 128;  // + t * Hv * 128 + dv
+  for (int t = 0; t < T; ++t) {
+    float delta[4], yv[4];
+    const bool on = a.mask == nullptr || a.mask[slotT + t] != 0;
+    if (on) {
+      float4 kk[4], qq[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        kk[c] = reinterpret_cast<const float4*>(sK + t * 128)[c3 + 8 * c];
+        qq[c] = reinterpret_cast<const float4*>(sQ + t * 128)[c3 + 8 * c];
+      }
+      const float4 v4 = *reinterpret_cast<const float4*>(sV + t * 128 + row0);
+      const float vv[4] = {v4.x, v4.y, v4.z, v4.w};
+      const float beta = sBeta[t], kq = sKQ[t];
+      if (FOLD) {
+        cum *= sG[t];
+        if (cum < 1e-12f) {  // same for the whole workgroup: put the scale back into S
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) st[i][c] *= cum;
+          cum = 1.f;
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          f32x4_t g4;
+          if (VECG) {
+            const float4 g = reinterpret_cast<const float4*>(sG + t * 128)[c3 + 8 * c];
+            g4 = f32x4_t{g.x, g.y, g.z, g.w};
+          } else {
+            const float g = sG[t];
+            g4 = f32x4_t{g, g, g, g};
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) st[i][c] *= g4;
+        }
+      }
+      float pk[4], pq[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        pk[i] = (dot4(st[i][0], kk[0]) + dot4(st[i][1], kk[1])) + (dot4(st[i][2], kk[2]) + dot4(st[i][3], kk[3]));
+        pq[i] = (dot4(st[i][0], qq[0]) + dot4(st[i][1], qq[1])) + (dot4(st[i][2], qq[2]) + dot4(st[i][3], qq[3]));
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        pk[i] = sum_over_8(pk[i]);
+        pq[i] = sum_over_8(pq[i]);
+      }
+      const float rcum = FOLD ? 1.f / cum : 1.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (FOLD) {
+          pk[i] *= cum;
+          pq[i] *= cum;
+        }
+        delta[i] = (vv[i] - pk[i]) * beta;
+        yv[i] = pq[i] + kq * delta[i];
+        const float d = FOLD ? delta[i] * rcum : delta[i];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          st[i][c].x += kk[c].x * d;
+          st[i][c].y += kk[c].y * d;
+          st[i][c].z += kk[c].z * d;
+          st[i][c].w += kk[c].w * d;
+        }
+      }
+      if (!f32_state) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) st[i][c][e] = round_through(st[i][c][e], a.state_dtype);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) delta[i] = 0.f, yv[i] = 0.f;
+    }
+    // lane c3 = i of each group of 8 lanes writes the outputs of row row0 + i
+    float d_out = delta[0], y_out = yv[0];
+#pragma unroll
+    for (int i = 1; i < 4; ++i) {
+      d_out = c3 == i ? delta[i] : d_out;
+      y_out = c3 == i ? yv[i] : y_out;
+    }
+    if (c3 < 4) {
+      const size_t o = obase + (size_t)t * a.Hv * 128 + row0 + c3;
+      a.tape[o] = d_out;
+      store_from_f32(a.y, o, y_out, a.in_dtype);
+    }
+  }
+
+  // ---- state out ----------------------------------------------------------------------------
+  if (f32_state) {
+    f32x4_t* out = reinterpret_cast<f32x4_t*>((float*)a.state_out + sbase);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        if (FOLD) st[i][c] *= cum;
+        __builtin_nontemporal_store(st[i][c], &out[(row0 + i) * 32 + c3 + 8 * c]);
+      }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          store_from_f32(a.state_out, sbase + (size_t)(row0 + i) * 128 + 4 * (c3 + 8 * c) + e, st[i][c][e],
+                         a.state_dtype);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Any Dk, Dv: one workgroup per (slot, head), a thread walks whole rows of S, which lives in
+// state_out between steps (so it is rounded through the state dtype after every step by
+// construction).  Slow and simple; the 128 x 128 kernel above is the one that is measured.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void gdn_forward_generic(GdnArgs a) {
+  const int slot = blockIdx.x / a.Hv, hv = blockIdx.x % a.Hv;
+  const int hk = hv / (a.Hv / a.Hk);
+  const size_t slotT = (size_t)slot * a.T;
+  const size_t sbase = (size_t)blockIdx.x * a.Dv * a.Dk;
+  for (int dv = threadIdx.x; dv < a.Dv; dv += kThreads) {
+    const size_t row = sbase + (size_t)dv * a.Dk;
+    for (int dk = 0; dk < a.Dk; ++dk)
+      store_from_f32(a.state_out, row + dk, load_as_f32(a.state_in, row + dk, a.state_dtype), a.state_dtype);
+    for (int t = 0; t < a.T; ++t) {
+      const size_t o = ((slotT + t) * a.Hv + hv) * a.Dv + dv;
+      float delta = 0.f, y = 0.f;
+      if (a.mask == nullptr || a.mask[slotT + t] != 0) {
+        const size_t kq0 = ((slotT + t) * a.Hk + hk) * a.Dk;
+        const size_t g0 = a.g_per_dk ? ((slotT + t) * a.Hv + hv) * a.Dk : (slotT + t) * a.Hv + hv;
+        float kv = 0.f;
+        for (int dk = 0; dk < a.Dk; ++dk) {
+          const float g = load_as_f32(a.g, a.g_per_dk ? g0 + dk : g0, a.g_dtype);
+          kv += load_as_f32(a.state_out, row + dk, a.state_dtype) * g * load_as_f32(a.k, kq0 + dk, a.in_dtype);
+        }
+        delta = (load_as_f32(a.v, o, a.in_dtype) - kv) * load_as_f32(a.beta, (slotT + t) * a.Hv + hv, a.beta_dtype);
+        for (int dk = 0; dk < a.Dk; ++dk) {
+          const float g = load_as_f32(a.g, a.g_per_dk ? g0 + dk : g0, a.g_dtype);
+          const float s = load_as_f32(a.state_out, row + dk, a.state_dtype) * g +
+                          load_as_f32(a.k, kq0 + dk, a.in_dtype) * delta;
+          y += s * load_as_f32(a.q, kq0 + dk, a.in_dtype);
+          store_from_f32(a.state_out, row + dk, s, a.state_dtype);
+        }
+      }
+      a.tape[o] = delta;
+      store_from_f32(a.y, o, y, a.in_dtype);
+    }
+  }
+}
+
+}  // namespace
+}  // namespace dflash
+
+extern "C" int dflash_gdn_forward_tape(const void* q, const void* k, const void* v, const void* g,
+                                       const void* beta, const void* state_in, void* state_out,
+                                       void* y, float* tape, const uint8_t* mask, int slots, int T,
+                                       int Hk, int Hv, int Dk, int Dv, int in_dtype, int g_dtype,
+                                       int beta_dtype, int state_dtype, int g_per_dk, void* stream) {
+  using namespace dflash;
+  DFLASH_REQUIRE(q && k && v && g && beta && state_in && state_out && y && tape, DFLASH_ERR_ARG,
+                 "dflash_gdn_forward_tape: null operand");
+  DFLASH_REQUIRE(state_in != state_out, DFLASH_ERR_ARG,
+                 "dflash_gdn_forward_tape: state_out must not alias state_in");
+  auto ok = [](int dt) { return dt == DFLASH_BF16 || dt == DFLASH_FP16 || dt == DFLASH_FP32; };
+  DFLASH_REQUIRE(ok(in_dtype) && ok(g_dtype) && ok(beta_dtype) && ok(state_dtype), DFLASH_ERR_ARG,
+                 "dflash_gdn_forward_tape: unknown dtype code");
+  DFLASH_REQUIRE(slots >= 0 && T >= 0 && Hk > 0 && Hv > 0 && Dk > 0 && Dv > 0, DFLASH_ERR_SHAPE,
+                 "dflash_gdn_forward_tape: non-positive dimension");
+  DFLASH_REQUIRE(Hv % Hk == 0, DFLASH_ERR_SHAPE,
+                 "dflash_gdn_forward_tape: cannot align K heads %d to V heads %d", Hk, Hv);
+  DFLASH_REQUIRE((long long)slots * Hv < (1ll << 31), DFLASH_ERR_SHAPE,
+                 "dflash_gdn_forward_tape: too many (slot, head) pairs");
+  if (slots == 0) return DFLASH_OK;
+
+  GdnArgs a;
+  a.q = q; a.k = k; a.v = v; a.g = g; a.beta = beta; a.state_in = state_in; a.state_out = state_out;
+  a.y = y; a.tape = tape; a.mask = mask;
+  a.T = T; a.Hk = Hk; a.Hv = Hv; a.Dk = Dk; a.Dv = Dv;
+  a.in_dtype = in_dtype; a.g_dtype = g_dtype; a.beta_dtype = beta_dtype; a.state_dtype = state_dtype;
+  a.g_per_dk = g_per_dk ? 1 : 0;
+
+  const dim3 grid((unsigned)(slots * Hv)), block(kThreads);
+  hipStream_t s = (hipStream_t)stream;
+  const size_t smem = ((size_t)T * 128 * 3 + (size_t)T * (g_per_dk ? 128 : 1) + 2 * (size_t)T) * sizeof(float);
+  const bool fast = Dk == 128 && Dv == 128 && T >= 1 && smem <= 64 * 1024 &&
+                    (state_dtype != DFLASH_FP32 ||
+                     (((uintptr_t)state_in % 16) == 0 && ((uintptr_t)state_out % 16) == 0));
+  if (fast) {
+    if (g_per_dk) {
+      hipLaunchKernelGGL((gdn_forward_128<true, false>), grid, block, smem, s, a);
+    } else if (state_dtype == DFLASH_FP32) {
+      hipLaunchKernelGGL((gdn_forward_128<false, true>), grid, block, smem, s, a);
+    } else {
+      hipLaunchKernelGGL((gdn_forward_128<false, false>), grid, block, smem, s, a);
+    }
+  } else {
+    hipLaunchKernelGGL(gdn_forward_generic, grid, block, 0, s, a);
+  }
+  DFLASH_HIP_OK(hipGetLastError());
+  return DFLASH_OK;
+}

@@ -1,10 +1,11 @@
-"""GatedDeltaNet tape replay (host side).
+"""GatedDeltaNet forward-with-tape and tape replay (host side).
 
-Mirror of the replay half of dflash_mlx/kernels.py: ``tape_replay_kernel``
-(:361-407) dispatches to the gfx950 kernel behind ``dflash_tape_replay``
-(include/dflash_mi355.h); ``_tape_replay_ops`` (:328-358) is the same recurrence
-in array ops, which the reference takes when the kernel does not cover a shape
-(:374-375) and which this module takes for the same shapes and for host tensors.
+Mirror of the GatedDeltaNet half of dflash_mlx/kernels.py: ``gated_delta_kernel_with_tape``
+(:176-224) and ``tape_replay_kernel`` (:361-407) dispatch to the gfx950 kernels behind
+``dflash_gdn_forward_tape`` and ``dflash_tape_replay`` (include/dflash_mi355.h); the
+``_..._ops`` functions (:131-173, :328-358) are the same recurrences in array ops, which
+the reference takes when its kernels do not cover a shape (:187-188, :374-375) and which
+this module takes for the same shapes and for host tensors.
 
 Layouts: tape [B,T,Hv,Dv]; k [B,T,Hk,Dk]; g [B,T,Hv] or [B,T,Hv,Dk];
 state [B,Hv,Dv,Dk]; mask [B,T] bool.
@@ -21,32 +22,97 @@ from . import _native
 _DTYPE_CODE = {torch.bfloat16: _native.BF16, torch.float16: _native.FP16, torch.float32: _native.FP32}
 
 
+def _expand_heads(x: torch.Tensor, hv: int, what: str) -> torch.Tensor:
+    hk = int(x.shape[2])
+    if hv % hk != 0:
+        raise ValueError(f"Cannot align K heads {hk} to {what} heads {hv}")
+    return x if hk == hv else torch.repeat_interleave(x, hv // hk, dim=2)
+
+
+def _gate_per_step(g: torch.Tensor) -> torch.Tensor:
+    """g as [B, T, Hv, 1, Dk or 1], broadcastable against a state [B, Hv, Dv, Dk]."""
+    if g.ndim == 4:
+        return g.unsqueeze(-2)
+    if g.ndim == 3:
+        return g[..., None, None]
+    raise ValueError(f"Unsupported gating shape {tuple(g.shape)}")
+
+
 def _tape_replay_ops(tape: torch.Tensor, k: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
                      mask: Optional[torch.Tensor] = None) -> torch.Tensor:
-    _, _, hk, _ = k.shape
-    hv = tape.shape[2]
-    if hv % hk != 0:
-        raise ValueError(f"Cannot align K heads {hk} to tape heads {hv}")
-    repeat_factor = hv // hk
-    if repeat_factor > 1:
-        k = torch.repeat_interleave(k, repeat_factor, dim=2)
-
+    """The replay recurrence in array ops (what the reference does without its kernel,
+    dflash_mlx/kernels.py:328-358): S <- g_t S + delta_t (x) k_t for every unmasked step."""
+    kk = _expand_heads(k, int(tape.shape[2]), "tape")
+    gate = _gate_per_step(g)
+    keep = None if mask is None else mask.to(torch.bool)
     for t in range(int(tape.shape[1])):
-        prev_state = state
-        if g.ndim == 4:
-            decay = g[:, t, :, None, :]
-        elif g.ndim == 3:
-            decay = g[:, t, :, None, None]
-        else:
-            raise ValueError(f"Unsupported gating shape {tuple(g.shape)}")
-        delta = tape[:, t, :, :, None]
-        k_t = k[:, t, :, None, :]
-        state = state * decay
-        state = state + delta * k_t
-        if mask is not None:
-            step_mask = mask[:, t][:, None, None, None]
-            state = torch.where(step_mask, state, prev_state)
+        stepped = state * gate[:, t] + tape[:, t].unsqueeze(-1) * kk[:, t].unsqueeze(-2)
+        state = stepped if keep is None else torch.where(keep[:, t].view(-1, 1, 1, 1), stepped, state)
     return state
+
+
+def _gated_delta_ops_with_tape(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor,
+                               beta: torch.Tensor, state: torch.Tensor,
+                               mask: Optional[torch.Tensor] = None):
+    """The forward recurrence in array ops (dflash_mlx/kernels.py:131-173): returns
+    (y [B,T,Hv,Dv], state, tape [B,T,Hv,Dv] fp32)."""
+    hv = int(v.shape[2])
+    qq, kk = _expand_heads(q, hv, "V"), _expand_heads(k, hv, "V")
+    gate = _gate_per_step(g)
+    keep = None if mask is None else mask.to(torch.bool)
+    ys, tape = [], []
+    for t in range(int(k.shape[1])):
+        decayed = state * gate[:, t]
+        innovation = (v[:, t] - (decayed * kk[:, t].unsqueeze(-2)).sum(-1)) * beta[:, t].unsqueeze(-1)
+        stepped = decayed + innovation.unsqueeze(-1) * kk[:, t].unsqueeze(-2)
+        y_t = (stepped * qq[:, t].unsqueeze(-2)).sum(-1)
+        if keep is not None:
+            on = keep[:, t]
+            stepped = torch.where(on.view(-1, 1, 1, 1), stepped, state)
+            innovation = torch.where(on.view(-1, 1, 1), innovation, torch.zeros_like(innovation))
+            y_t = torch.where(on.view(-1, 1, 1), y_t, torch.zeros_like(y_t))
+        state = stepped
+        ys.append(y_t)
+        tape.append(innovation.to(torch.float32))
+    return torch.stack(ys, dim=1), state, torch.stack(tape, dim=1)
+
+
+def gated_delta_kernel_with_tape(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor,
+                                 beta: torch.Tensor, state: torch.Tensor,
+                                 mask: Optional[torch.Tensor] = None):
+    """GatedDeltaNet forward over a block that records the innovation tape (mirror of
+    dflash_mlx/kernels.py:176-224): ``(y, state_out, tape)`` with y in q's dtype, the state in
+    its own dtype and an fp32 tape.  Device tensors with Dk a multiple of 32 go to the gfx950
+    kernel behind ``dflash_gdn_forward_tape``; host tensors and other shapes take the array
+    ops, as the reference does without its kernel."""
+    B, T, hk, dk = (int(d) for d in k.shape)
+    hv, dv = int(v.shape[2]), int(v.shape[3])
+    if g.ndim not in (3, 4):
+        raise ValueError(f"Unsupported gating shape {tuple(g.shape)}")
+    if hv % hk != 0:
+        raise ValueError(f"Cannot align K heads {hk} to V heads {hv}")
+    dtypes_ok = (q.dtype == k.dtype == v.dtype and
+                 all(t.dtype in _DTYPE_CODE for t in (q, g, beta, state)))
+    if not state.is_cuda or dk < 32 or dk % 32 != 0 or not dtypes_ok or T == 0:
+        return _gated_delta_ops_with_tape(q, k, v, g, beta, state, mask)
+    lib = _native.lib()
+    q_c, k_c, v_c, g_c, beta_c = (t.contiguous() for t in (q, k, v, g, beta))
+    state_c = state.contiguous()
+    y = torch.empty((B, T, hv, dv), dtype=q.dtype, device=q.device)
+    tape = torch.empty((B, T, hv, dv), dtype=torch.float32, device=q.device)
+    state_out = torch.empty_like(state_c)
+    mask_ptr = None
+    if mask is not None:
+        mask = mask.to(torch.uint8).contiguous()
+        mask_ptr = mask.data_ptr()
+    rc = lib.dflash_gdn_forward_tape(
+        q_c.data_ptr(), k_c.data_ptr(), v_c.data_ptr(), g_c.data_ptr(), beta_c.data_ptr(),
+        state_c.data_ptr(), state_out.data_ptr(), y.data_ptr(), tape.data_ptr(), mask_ptr,
+        B, T, hk, hv, dk, dv, _DTYPE_CODE[q.dtype], _DTYPE_CODE[g.dtype], _DTYPE_CODE[beta.dtype],
+        _DTYPE_CODE[state.dtype], 1 if g.ndim == 4 else 0,
+        torch.cuda.current_stream(q.device).cuda_stream)
+    _native.check(rc, "dflash_gdn_forward_tape")
+    return y, state_out, tape
 
 
 def _exact_order() -> bool:

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 3
+#define DFLASH_ABI_VERSION 4
 
 enum {
   DFLASH_OK = 0,
@@ -138,6 +138,33 @@ int dflash_tape_replay(const void* tape, const void* k, const void* g, const voi
                        const uint8_t* mask, int slots, int T, int Hk, int Hv, int Dk, int Dv,
                        int state_dtype, int tape_dtype, int k_dtype, int g_dtype, int g_per_dk,
                        int exact_order, void* stream);
+
+/*
+ * GatedDeltaNet forward over a block of T tokens that records the innovation tape - the
+ * producer of what dflash_tape_replay consumes.  For every slot s and value head hv, with
+ * hk = hv / (Hv / Hk), for t = 0 .. T-1 (steps whose mask byte is zero leave S alone and give
+ * y_t = tape_t = 0):
+ *     S <- g_t * S;  delta = (v_t - S k_t) * beta_t;  S <- S + delta (x) k_t;  y_t = S q_t;
+ *     tape_t = delta;  S rounded through state_dtype.
+ * Replaces the `gated_delta_tape{,_vec}{,_mask}` launch of dflash_mlx/kernels.py:207-224
+ * (kernel body :29-106).
+ *
+ *   q, k      [slots, T, Hk, Dk]   in_dtype (bf16 / fp16 / fp32)
+ *   v         [slots, T, Hv, Dv]   in_dtype
+ *   g         [slots, T, Hv] (g_per_dk = 0) or [slots, T, Hv, Dk] (g_per_dk = 1), g_dtype
+ *   beta      [slots, T, Hv]       beta_dtype
+ *   state_in  [slots, Hv, Dv, Dk]  state_dtype, Dk contiguous; state_out same, no aliasing
+ *   y         [slots, T, Hv, Dv]   in_dtype (output)
+ *   tape      [slots, T, Hv, Dv]   fp32 (output)
+ *   mask      [slots, T] uint8 or NULL
+ * 128 x 128 heads with T*(3*128 + (g_per_dk ? 128 : 1) + 2)*4 bytes <= 64 KiB of LDS take the
+ * register-resident kernel; every other shape a simple one that keeps S in state_out.
+ */
+int dflash_gdn_forward_tape(const void* q, const void* k, const void* v, const void* g,
+                            const void* beta, const void* state_in, void* state_out, void* y,
+                            float* tape, const uint8_t* mask, int slots, int T, int Hk, int Hv,
+                            int Dk, int Dv, int in_dtype, int g_dtype, int beta_dtype,
+                            int state_dtype, int g_per_dk, void* stream);
 
 /*
  * Conv-window rebuild of a GatedDeltaNet layer after a partial acceptance: output

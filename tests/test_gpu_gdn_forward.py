@@ -1,0 +1,141 @@
+"""Parity of the gfx950 GatedDeltaNet forward-with-tape kernel against the CPU oracle
+(fp64 restatement of dflash_mlx/kernels.py:131-173), and its contract with the replay:
+the tape it records, replayed for any prefix, gives the state the forward had there.
+
+Bars: fp32 state and fp32 tape rel-L2 <= 2e-5; y (rounded to the input dtype) within one
+rounding of the input dtype of the exact value; low-precision states compared against the
+oracle run with the same per-step rounding."""
+import numpy as np
+import pytest
+import torch
+
+from dflash_mlx_amd.kernels import (_gated_delta_ops_with_tape, gated_delta_kernel_with_tape,
+                                    tape_replay_kernel)
+from oracle import dflash_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _case(B=2, T=16, Hk=4, Hv=8, Dk=128, Dv=128, seed=0, g_per_dk=False, dtype=torch.bfloat16,
+          state_dtype=torch.float32):
+    g = torch.Generator().manual_seed(0xDF1A + seed)
+    q = torch.randn((B, T, Hk, Dk), generator=g)
+    k = torch.randn((B, T, Hk, Dk), generator=g)
+    q = (q / q.norm(dim=-1, keepdim=True) * Dk ** -0.5).to(dtype)
+    k = (k / k.norm(dim=-1, keepdim=True)).to(dtype)
+    v = torch.randn((B, T, Hv, Dv), generator=g).to(dtype)
+    gshape = (B, T, Hv, Dk) if g_per_dk else (B, T, Hv)
+    gate = torch.exp(-torch.nn.functional.softplus(torch.randn(gshape, generator=g)))
+    beta = torch.sigmoid(torch.randn((B, T, Hv), generator=g)).to(dtype)
+    state = (torch.randn((B, Hv, Dv, Dk), generator=g) * 0.1).to(state_dtype)
+    return q, k, v, gate, beta, state
+
+
+def _f64(t):
+    return t.detach().cpu().to(torch.float64).numpy()
+
+
+def _rel(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+def _run(args, mask=None):
+    dev = [t.to(DEV) for t in args]
+    y, s, tape = gated_delta_kernel_with_tape(*dev, mask=None if mask is None else mask.to(DEV))
+    torch.cuda.synchronize()
+    return y, s, tape
+
+
+@pytest.mark.parametrize("g_per_dk", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_against_fp64_oracle(native_lib, g_per_dk, dtype):
+    args = _case(seed=1 + int(g_per_dk), g_per_dk=g_per_dk, dtype=dtype)
+    y, s, tape = _run(args)
+    assert y.dtype == dtype and s.dtype == torch.float32 and tape.dtype == torch.float32
+    yo, so, to = O.gated_delta_ops_with_tape(*[_f64(t) for t in args])
+    assert _rel(_f64(s), so) <= 2e-5
+    assert _rel(_f64(tape), to) <= 2e-5
+    eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -20}[dtype]
+    assert np.all(np.abs(_f64(y) - yo) <= eps * np.abs(yo) + 2e-5 * np.abs(yo).max())
+
+
+def test_config2_shape_all_heads(native_lib):
+    """32 value heads of 128 x 128 with 16 key heads, 16 steps: the GDN layer shape of config[2]."""
+    args = _case(B=3, Hk=16, Hv=32, seed=7)
+    y, s, tape = _run(args)
+    yo, so, to = O.gated_delta_ops_with_tape(*[_f64(t) for t in args])
+    assert _rel(_f64(s), so) <= 2e-5 and _rel(_f64(tape), to) <= 2e-5 and _rel(_f64(y), yo) <= 4e-3
+
+
+def test_mask_skips_steps(native_lib):
+    args = _case(seed=3)
+    mask = torch.tensor([[1, 1, 0, 1, 0, 0, 1, 1, 1, 0, 1, 1, 1, 1, 0, 1],
+                         [0, 0, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 0]], dtype=torch.bool)
+    y, s, tape = _run(args, mask)
+    yo, so, to = O.gated_delta_ops_with_tape(*[_f64(t) for t in args], mask=mask.numpy())
+    assert _rel(_f64(s), so) <= 2e-5 and _rel(_f64(tape), to) <= 2e-5
+    off = ~mask
+    assert torch.all(tape.cpu()[off] == 0) and torch.all(y.cpu()[off] == 0)
+
+
+def test_recorded_tape_replays_to_every_prefix_state(native_lib):
+    """The contract between the two kernels (dflash_mlx/recurrent_rollback_cache.py:160-167)."""
+    q, k, v, gate, beta, state = _case(seed=5)
+    y, s_full, tape = _run((q, k, v, gate, beta, state))
+    kd, gd, sd = k.to(DEV), gate.to(DEV), state.to(DEV)
+    for a in (0, 1, 7, 16):
+        prefix = [t[:, :a] for t in (q, k, v, gate, beta)]
+        if a == 0:
+            want = sd
+        else:
+            _, want, _ = _run(prefix + [state])
+        got = tape_replay_kernel(tape[:, :a], kd[:, :a], gd[:, :a], sd) if a else sd
+        assert _rel(_f64(got), _f64(want)) <= 2e-5
+    assert _rel(_f64(tape_replay_kernel(tape, kd, gd, sd)), _f64(s_full)) <= 2e-5
+
+
+@pytest.mark.parametrize("state_dtype", [torch.bfloat16, torch.float16])
+def test_low_precision_state_is_rounded_after_every_step(native_lib, state_dtype):
+    """kernels.py:96-98: the state goes through its storage type after every step."""
+    args = _case(B=1, Hk=2, Hv=2, seed=9, state_dtype=state_dtype)
+    y, s, tape = _run(args)
+    assert s.dtype == state_dtype
+    # the same recurrence on the host, fp32 arithmetic, rounding through the state dtype per step
+    q, k, v, gate, beta, state = args
+    S = state.float()
+    tapes = []
+    for t in range(q.shape[1]):
+        _, S, tp = _gated_delta_ops_with_tape(q[:, t:t + 1].float(), k[:, t:t + 1].float(), v[:, t:t + 1].float(),
+                                              gate[:, t:t + 1], beta[:, t:t + 1].float(), S)
+        S = S.to(state_dtype).float()
+        tapes.append(tp)
+    assert _rel(_f64(s), _f64(S)) <= 2e-3            # one unit of the state dtype here and there
+    assert _rel(_f64(tape), _f64(torch.cat(tapes, dim=1))) <= 2e-3
+
+
+@pytest.mark.parametrize("shape", [dict(Dk=64, Dv=64), dict(Dk=96, Dv=32, Hk=2, Hv=2), dict(Dk=128, Dv=64),
+                                   dict(T=3), dict(T=40, Hk=1, Hv=2, B=1)])
+def test_other_shapes(native_lib, shape):
+    args = _case(seed=11, **shape)
+    y, s, tape = _run(args)
+    yo, so, to = O.gated_delta_ops_with_tape(*[_f64(t) for t in args])
+    assert _rel(_f64(s), so) <= 2e-5 and _rel(_f64(tape), to) <= 2e-5 and _rel(_f64(y), yo) <= 4e-3
+
+
+def test_errors_and_host_tensors(native_lib):
+    q, k, v, gate, beta, state = _case(B=1, T=2, Hk=3, Hv=4, Dk=32, Dv=8)
+    with pytest.raises(ValueError, match="Cannot align"):
+        gated_delta_kernel_with_tape(q, k, v, gate, beta, state)
+    q, k, v, gate, beta, state = _case(B=1, T=2, Hk=2, Hv=4, Dk=32, Dv=8)
+    with pytest.raises(ValueError, match="Unsupported gating shape"):
+        gated_delta_kernel_with_tape(q, k, v, gate[..., 0], beta, state)
+    # host tensors: the array ops, as in the reference without its kernel
+    y, s, tape = gated_delta_kernel_with_tape(q.float(), k.float(), v.float(), gate, beta.float(), state)
+    yo, so, to = O.gated_delta_ops_with_tape(*[_f64(t) for t in (q, k, v, gate, beta, state)])
+    assert _rel(_f64(s), so) <= 1e-5 and _rel(_f64(tape), to) <= 1e-5 and _rel(_f64(y), yo) <= 1e-5
+    # the C entry point refuses aliasing and null pointers
+    L = native_lib
+    assert L.dflash_gdn_forward_tape(None, None, None, None, None, None, None, None, None, None,
+                                     1, 1, 1, 1, 32, 8, 0, 2, 0, 2, 0, None) == -1

@@ -293,3 +293,32 @@ def test_rollback_cache_state_machine_on_host():
     with pytest.raises(ValueError):
         from dflash_mlx_amd.kernels import _tape_replay_ops
         _tape_replay_ops(t(tape)[:, :, :3], t(k), t(g)[:, :, :3], t(S0)[:, :3])
+
+
+@pytest.mark.parametrize("g_per_dk", [False, True])
+def test_array_op_forms_match_the_oracle(g_per_dk):
+    """The torch array-op forms of forward-with-tape and replay (what host tensors and
+    uncovered shapes take) against the NumPy oracle, with a mask and Hk < Hv."""
+    from dflash_mlx_amd.kernels import (_gated_delta_ops_with_tape, _tape_replay_ops,
+                                        gated_delta_kernel_with_tape)
+    rng = np.random.default_rng(31 + int(g_per_dk))
+    B, T, Hk, Hv, Dk, Dv = 2, 7, 2, 6, 8, 5
+    q = rng.standard_normal((B, T, Hk, Dk)); k = rng.standard_normal((B, T, Hk, Dk))
+    v = rng.standard_normal((B, T, Hv, Dv))
+    g = rng.uniform(0.2, 1, (B, T, Hv, Dk) if g_per_dk else (B, T, Hv))
+    beta = rng.uniform(0, 1, (B, T, Hv)); S0 = rng.standard_normal((B, Hv, Dv, Dk)) * 0.1
+    mask = rng.uniform(size=(B, T)) > 0.3
+    t = torch.from_numpy
+    for m in (None, mask):
+        yo, so, to = O.gated_delta_ops_with_tape(q, k, v, g, beta, S0, mask=m)
+        tm = None if m is None else t(m)
+        y, s, tape = _gated_delta_ops_with_tape(t(q), t(k), t(v), t(g), t(beta), t(S0), tm)
+        np.testing.assert_allclose(y.numpy(), yo, rtol=1e-12, atol=1e-13)
+        np.testing.assert_allclose(s.numpy(), so, rtol=1e-12, atol=1e-13)
+        np.testing.assert_allclose(tape.numpy(), to, rtol=1e-6, atol=1e-7)   # the tape is fp32
+        y2, s2, _ = gated_delta_kernel_with_tape(t(q), t(k), t(v), t(g), t(beta), t(S0), tm)  # host tensors
+        assert torch.equal(y2, y) and torch.equal(s2, s)
+        ro = O.tape_replay_ops(to, k, g, S0, mask=m)
+        r = _tape_replay_ops(t(to), t(k), t(g), t(S0), tm)
+        np.testing.assert_allclose(r.numpy(), ro, rtol=1e-12, atol=1e-13)
+        np.testing.assert_allclose(r.numpy(), so, rtol=1e-9, atol=1e-10)     # replay of the full tape
