@@ -139,3 +139,31 @@ def test_errors_and_host_tensors(native_lib):
     L = native_lib
     assert L.dflash_gdn_forward_tape(None, None, None, None, None, None, None, None, None, None,
                                      1, 1, 1, 1, 32, 8, 0, 2, 0, 2, 0, None) == -1
+
+
+@pytest.mark.parametrize("accepted", [0, 5, 14])
+def test_speculative_cycle_through_the_rollback_cache(native_lib, accepted):
+    """One verify cycle of a GatedDeltaNet layer on the device (runtime.py:411-442, 878-907):
+    arm, run the block with the tape recorded, roll back to `accepted` drafted tokens - the
+    cache must hold what a run over only the committed accepted+1 tokens leaves."""
+    from dflash_mlx_amd.recurrent_rollback_cache import RecurrentRollbackCache
+    q, k, v, gate, beta, state = [t.to(DEV) for t in _case(B=1, Hk=4, Hv=8, seed=21)]
+    C = 64
+    gen = torch.Generator().manual_seed(5)
+    conv0 = torch.randn((1, 3, C), generator=gen).to(torch.bfloat16).to(DEV)
+    qkv = torch.randn((1, 16, C), generator=gen).to(torch.bfloat16).to(DEV)
+    cache = RecurrentRollbackCache(size=2, conv_kernel_size=4)
+    cache[0], cache[1] = conv0, state
+    cache.arm_rollback()
+    y, s_block, tape = gated_delta_kernel_with_tape(q, k, v, gate, beta, cache[1])
+    cache.record_tape(tape=tape, k=k, g=gate, qkv=qkv)
+    cache[0], cache[1] = qkv[:, -3:].clone(), s_block          # what the layer leaves after 16 tokens
+    cache.rollback(accepted)
+    torch.cuda.synchronize()
+    n = accepted + 1
+    y_n, s_n, _ = gated_delta_kernel_with_tape(q[:, :n], k[:, :n], v[:, :n], gate[:, :n], beta[:, :n], state)
+    assert _rel(_f64(cache[1]), _f64(s_n)) <= 2e-5
+    assert torch.equal(y[:, :n], y_n)                             # outputs of the kept tokens are the block's
+    want_conv = torch.cat([conv0, qkv], dim=1)[:, n:n + 3]
+    assert torch.equal(cache[0], want_conv)
+    assert not cache._armed and cache._tape is None
