@@ -30,6 +30,7 @@
 //    multiplies c back in once at the end (renormalising if c gets very small).
 // q, k, v, g, beta of the block are staged once in LDS as fp32.
 #include "dflash_common.h"
+#include <cstdlib>
 
 namespace dflash {
 namespace {
@@ -267,6 +268,326 @@ __global__ __launch_bounds__(kThreads) void gdn_forward_128(GdnArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// Dk = Dv = 128, T <= 16, one gate per head, fp32 state: the block in closed form.
+// With c_t = prod_{u<=t} g_u (masked steps: g = 1, beta = 0) the recurrence unrolls to
+//     kv_t    = c_t (S0 k_t) + sum_{s<t}  (c_t/c_s) (k_s.k_t) delta_s
+//     delta_t = beta_t (v_t - kv_t)
+//     y_t     = c_t (S0 q_t) + sum_{s<=t} (c_t/c_s) (k_s.q_t) delta_s
+//     S_T     = c_T S0 + sum_s (c_T/c_s) delta_s (x) k_s
+// In matrix form, with U = S0 K^T, W = S0 Q^T (Dv x T), L[t][s] = beta_t (c_t/c_s)(k_s.k_t) for
+// s < t and Lq[t][s] = (c_t/c_s)(k_s.q_t) for s <= t:
+//     Delta = R (I + L)^-T with R[dv][t] = beta_t (v_t[dv] - c_t U[dv][t]),
+//     Y = c W + Delta Lq^T,     S_T^T = c_T S0^T + K^T diag(c_T/c_s) Delta^T.
+// Every product runs on the fp32 matrix cores (v_mfma_f32_16x16x4_f32); the only serial part
+// is the inverse of the T x T unit triangular matrix, once per head.  The arithmetic per
+// state element drops from ~5 T vector operations to ~1.5 T matrix-core operations, which
+// leaves the kernel bound by the state traffic.
+//
+// MFMA 16x16x4 lanes: A lane l holds A[i = l % 16][k = l / 16], B lane l holds B[k = l / 16]
+// [j = l % 16], accumulator register r of lane l is C[4 (l / 16) + r][l % 16].
+// Lane (li = lane % 16, kq = lane / 16) of wave w keeps S rows 32w + 16a + li (a = 0, 1),
+// columns 16c + 4kq + e (c = 0..7, e = 0..3).  As the A operand of S0 K^T, component e of
+// chunk c pairs with k_t[16c + 4kq + e] on the B side: the columns are only summed in another
+// order.  As the accumulator of the transposed update (rows = Dk, columns = Dv) the same
+// registers are C[16c + 4kq + e][row li], so the new state lands where the old one was.
+// ---------------------------------------------------------------------------
+constexpr int kKPad = 132;  // row pitch of K and Q in LDS, in floats
+constexpr int kRPad = 17;   // row pitch of R
+constexpr int kOffK = 0;
+constexpr int kOffQ = kOffK + 16 * kKPad;  // Q, then Delta[t][dv]
+constexpr int kOffV = kOffQ + 16 * kKPad;
+constexpr int kOffR = kOffV + 16 * 128;
+constexpr int kOffRat = kOffR + 128 * kRPad;  // c_t / c_s, 0 above the diagonal
+constexpr int kOffL = kOffRat + 256;
+constexpr int kOffLq = kOffL + 256;
+constexpr int kOffM = kOffLq + 256;  // (I + L)^-1
+constexpr int kOffC = kOffM + 256;
+constexpr int kOffBeta = kOffC + 16;   // 0 for masked and missing steps
+constexpr int kOffGate = kOffBeta + 16;  // 1 for masked and missing steps
+constexpr int kChunkLdsFloats = kOffGate + 16;
+
+struct Raw8 {
+  uint4 lo, hi;
+};
+// Eight consecutive elements from element i (a multiple of 8) of a 16-byte aligned array.
+__device__ __forceinline__ Raw8 load8_raw(const void* p, size_t i, int dt) {
+  Raw8 r;
+  r.hi = uint4{0u, 0u, 0u, 0u};
+  if (dt == DFLASH_FP32) {
+    const uint4* src = reinterpret_cast<const uint4*>((const float*)p + i);
+    r.lo = src[0];
+    r.hi = src[1];
+  } else {
+    r.lo = *reinterpret_cast<const uint4*>((const uint16_t*)p + i);
+  }
+  return r;
+}
+__device__ __forceinline__ void raw8_to_lds(const Raw8& r, int dt, float* dst) {
+  const uint32_t w[8] = {r.lo.x, r.lo.y, r.lo.z, r.lo.w, r.hi.x, r.hi.y, r.hi.z, r.hi.w};
+  float o[8];
+  if (dt == DFLASH_FP32) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = __uint_as_float(w[j]);
+  } else if (dt == DFLASH_BF16) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      o[2 * j] = __uint_as_float(w[j] << 16);
+      o[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      o[2 * j] = f16_bits_to_f32(w[j] & 0xffffu);
+      o[2 * j + 1] = f16_bits_to_f32(w[j] >> 16);
+    }
+  }
+  reinterpret_cast<float4*>(dst)[0] = float4{o[0], o[1], o[2], o[3]};
+  reinterpret_cast<float4*>(dst)[1] = float4{o[4], o[5], o[6], o[7]};
+}
+// Four consecutive elements at element i (a multiple of 4) of a 16-byte aligned array.
+__device__ __forceinline__ void store4_from_f32(void* p, size_t i, f32x4_t v, int dt) {
+  if (dt == DFLASH_FP32) {
+    *reinterpret_cast<f32x4_t*>((float*)p + i) = v;
+  } else if (dt == DFLASH_BF16) {
+    *reinterpret_cast<uint2*>((uint16_t*)p + i) = uint2{f32_to_bf16_bits(v.x) | (f32_to_bf16_bits(v.y) << 16),
+                                                        f32_to_bf16_bits(v.z) | (f32_to_bf16_bits(v.w) << 16)};
+  } else {
+    *reinterpret_cast<uint2*>((uint16_t*)p + i) = uint2{f32_to_f16_bits(v.x) | (f32_to_f16_bits(v.y) << 16),
+                                                        f32_to_f16_bits(v.z) | (f32_to_f16_bits(v.w) << 16)};
+  }
+}
+__device__ __forceinline__ f32x4_t mfma4(float x, float y, f32x4_t acc) {
+  return __builtin_amdgcn_mfma_f32_16x16x4f32(x, y, acc, 0, 0, 0);
+}
+
+// The matrix-core layout puts 4 lanes (kq) on a row of S per 16-byte access: 64 contiguous
+// bytes per row, which the memory system moves at about half the rate of full 128-byte lines
+// (stores above all).  Memory is therefore accessed with 8 lanes per row - register (t2, c) of
+// lane (li, kq) is row 16 t2 + 8 (c & 1) + li % 8, 16-byte column 8 (c / 2) + 4 (li / 8) + kq -
+// and swap_row_bit() exchanges lane bit 3 with the low bit of c between the two layouts:
+// the odd register of lanes li < 8 trades places with the even register of lanes li >= 8
+// (DPP row_ror:8 reads lane li ^ 8; the bank mask picks the half row that is written).
+__device__ __forceinline__ int memory_index(int wave, int li, int kq, int t2, int c) {
+  return (32 * wave + 16 * t2 + 8 * (c & 1) + (li & 7)) * 32 + 8 * (c >> 1) + 4 * (li >> 3) + kq;
+}
+__device__ __forceinline__ void swap_row_bit(f32x4_t& even, f32x4_t& odd) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int x = __float_as_int(even[e]), y = __float_as_int(odd[e]);
+    even[e] = __int_as_float(__builtin_amdgcn_update_dpp(x, y, 0x128, 0xF, 0xC, false));
+    odd[e] = __int_as_float(__builtin_amdgcn_update_dpp(y, x, 0x128, 0xF, 0x3, false));
+  }
+}
+
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void gdn_forward_chunk_128(GdnArgs a) {
+  extern __shared__ __align__(16) float smem[];
+  float* sK = smem + kOffK;
+  float* sQ = smem + kOffQ;
+  float* sD = smem + kOffQ;
+  float* sV = smem + kOffV;
+  float* sR = smem + kOffR;
+  float* sRat = smem + kOffRat;
+  float* sL = smem + kOffL;
+  float* sLq = smem + kOffLq;
+  float* sM = smem + kOffM;
+  float* sC = smem + kOffC;
+  float* sBeta = smem + kOffBeta;
+  float* sGate = smem + kOffGate;
+
+  const int T = a.T;
+  const int slot = blockIdx.x / a.Hv, hv = blockIdx.x % a.Hv;
+  const int hk = hv / (a.Hv / a.Hk);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int li = lane & 15, kq = lane >> 4;
+  const size_t slotT = (size_t)slot * T;
+  const size_t sbase = (size_t)blockIdx.x * 128 * 128;
+
+  // ---- the block's operands first, the state behind them ------------------------------------
+  Raw8 rk, rq, rv;
+  rk.lo = rk.hi = rq.lo = rq.hi = rv.lo = rv.hi = uint4{0u, 0u, 0u, 0u};
+  {
+    const int t = tid >> 4, seg = tid & 15;
+    if (t < T) {
+      const size_t kq_at = ((slotT + t) * a.Hk + hk) * 128 + 8 * seg;
+      const size_t v_at = ((slotT + t) * a.Hv + hv) * 128 + 8 * seg;
+      rk = load8_raw(a.k, kq_at, a.in_dtype);
+      rq = load8_raw(a.q, kq_at, a.in_dtype);
+      rv = load8_raw(a.v, v_at, a.in_dtype);
+    }
+  }
+  float gate = 1.f, beta = 0.f;
+  if (tid < T && (a.mask == nullptr || a.mask[slotT + tid] != 0)) {
+    gate = load_as_f32(a.g, (slotT + tid) * a.Hv + hv, a.g_dtype);
+    beta = load_as_f32(a.beta, (slotT + tid) * a.Hv + hv, a.beta_dtype);
+  }
+  f32x4_t st[2][8];
+  {
+    const f32x4_t* in = reinterpret_cast<const f32x4_t*>((const float*)a.state_in + sbase);
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int c = 0; c < 8; ++c)
+        st[t2][c] = __builtin_nontemporal_load(&in[memory_index(wave, li, kq, t2, c)]);
+  }
+  {
+    const int t = tid >> 4, seg = tid & 15;
+    raw8_to_lds(rk, a.in_dtype, sK + t * kKPad + 8 * seg);
+    raw8_to_lds(rq, a.in_dtype, sQ + t * kKPad + 8 * seg);
+    raw8_to_lds(rv, a.in_dtype, sV + t * 128 + 8 * seg);
+  }
+  if (tid < 16) {
+    sGate[tid] = gate;
+    sBeta[tid] = beta;
+  }
+  __syncthreads();
+  {  // c_t / c_s = prod_{s < u <= t} g_u for s <= t, and c_t itself
+    const int t = tid >> 4, sx = tid & 15;
+    float r = 0.f;
+    if (sx <= t) {
+      r = 1.f;
+      for (int u = sx + 1; u <= t; ++u) r *= sGate[u];
+    }
+    sRat[tid] = r;
+    if (sx == 0) sC[t] = r * sGate[0];
+  }
+  __syncthreads();
+
+  // ---- U = S0 K^T, W = S0 Q^T (every wave, its 32 rows); K K^T (wave 1), K Q^T (wave 2) -------
+#pragma unroll
+  for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+    for (int m = 0; m < 4; ++m) swap_row_bit(st[t2][2 * m], st[t2][2 * m + 1]);
+  f32x4_t U[2], W[2], X = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int t2 = 0; t2 < 2; ++t2) U[t2] = f32x4_t{0.f, 0.f, 0.f, 0.f}, W[t2] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    const float4 kf4 = *reinterpret_cast<const float4*>(sK + li * kKPad + 16 * c + 4 * kq);
+    const float4 qf4 = *reinterpret_cast<const float4*>(sQ + li * kKPad + 16 * c + 4 * kq);
+    const float kf[4] = {kf4.x, kf4.y, kf4.z, kf4.w};
+    const float qf[4] = {qf4.x, qf4.y, qf4.z, qf4.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2) {
+        U[t2] = mfma4(st[t2][c][e], kf[e], U[t2]);
+        W[t2] = mfma4(st[t2][c][e], qf[e], W[t2]);
+      }
+      if (wave == 1) X = mfma4(kf[e], kf[e], X);  // [s][t] = k_s . k_t
+      if (wave == 2) X = mfma4(kf[e], qf[e], X);  // [s][t] = k_s . q_t
+    }
+  }
+  {
+    const int t = li;
+    const float ct = sC[t], bt = sBeta[t];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int sx = 4 * kq + r;
+      const float rat = sRat[t * 16 + sx];  // 0 for s > t
+      if (wave == 1) sL[t * 16 + sx] = sx < t ? bt * rat * X[r] : 0.f;
+      if (wave == 2) sLq[t * 16 + sx] = rat * X[r];
+    }
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      const int row0 = 32 * wave + 16 * t2 + 4 * kq;
+      const float4 v4 = *reinterpret_cast<const float4*>(sV + t * 128 + row0);
+      sR[(row0 + 0) * kRPad + t] = bt * (v4.x - ct * U[t2][0]);
+      sR[(row0 + 1) * kRPad + t] = bt * (v4.y - ct * U[t2][1]);
+      sR[(row0 + 2) * kRPad + t] = bt * (v4.z - ct * U[t2][2]);
+      sR[(row0 + 3) * kRPad + t] = bt * (v4.w - ct * U[t2][3]);
+    }
+  }
+  __syncthreads();  // L, Lq and R are complete; nobody reads Q any more
+
+  // ---- M = (I + L)^-1, column li per lane -----------------------------------------------------
+  if (wave == 1) {
+    float x[16];
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      float acc = t == li ? 1.f : 0.f;
+#pragma unroll
+      for (int sx = 0; sx < t; ++sx) acc -= sL[t * 16 + sx] * x[sx];
+      x[t] = acc;
+      if (kq == 0) sM[t * 16 + li] = acc;
+    }
+  }
+  __syncthreads();
+
+  // ---- Delta = R M^T: rows of this wave, accumulator (row 4kq + r, column t = li) ---------------
+  f32x4_t D[2];
+#pragma unroll
+  for (int t2 = 0; t2 < 2; ++t2) {
+    D[t2] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      D[t2] = mfma4(sR[(32 * wave + 16 * t2 + li) * kRPad + 4 * j + kq], sM[li * 16 + 4 * j + kq], D[t2]);
+  }
+  const size_t obase = ((slotT + li) * a.Hv + hv) * 128;  // step li of this head in y and the tape
+#pragma unroll
+  for (int t2 = 0; t2 < 2; ++t2) {
+    const int row0 = 32 * wave + 16 * t2 + 4 * kq;
+    *reinterpret_cast<f32x4_t*>(sD + li * 128 + row0) = D[t2];
+    if (li < T) *reinterpret_cast<f32x4_t*>(a.tape + obase + row0) = D[t2];
+  }
+  __syncthreads();
+
+  // ---- Y = c W + Delta Lq^T -----------------------------------------------------------------------
+  float dA[2][4];  // Delta[row 16 t2 + li][s = 4j + kq]
+#pragma unroll
+  for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dA[t2][j] = sD[(4 * j + kq) * 128 + 32 * wave + 16 * t2 + li];
+  {
+    const float ct = sC[li];
+    const bool on = li < T && (a.mask == nullptr || a.mask[slotT + li] != 0);
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      f32x4_t Y = W[t2] * ct;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) Y = mfma4(dA[t2][j], sLq[li * 16 + 4 * j + kq], Y);
+      if (!on) Y = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if (li < T) store4_from_f32(a.y, obase + 32 * wave + 16 * t2 + 4 * kq, Y, a.in_dtype);
+    }
+  }
+
+  // ---- S_T^T = c_T S0^T + K^T diag(c_T / c_s) Delta^T -----------------------------------------------
+  {
+    const float cT = sC[T - 1];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float cf = sRat[(T - 1) * 16 + 4 * j + kq];  // 0 beyond step T - 1
+      dA[0][j] *= cf;
+      dA[1][j] *= cf;
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      float kA[4];  // K[s = 4j + kq][16c + li]
+#pragma unroll
+      for (int j = 0; j < 4; ++j) kA[j] = sK[(4 * j + kq) * kKPad + 16 * c + li];
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2) {
+        f32x4_t acc = st[t2][c] * cT;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc = mfma4(kA[j], dA[t2][j], acc);
+        st[t2][c] = acc;
+      }
+    }
+  }
+  {
+    f32x4_t* out = reinterpret_cast<f32x4_t*>((float*)a.state_out + sbase);
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int m = 0; m < 4; ++m) swap_row_bit(st[t2][2 * m], st[t2][2 * m + 1]);
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int c = 0; c < 8; ++c)
+        __builtin_nontemporal_store(st[t2][c], &out[memory_index(wave, li, kq, t2, c)]);
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Any Dk, Dv: one workgroup per (slot, head), a thread walks whole rows of S, which lives in
 // state_out between steps (so it is rounded through the state dtype after every step by
 // construction).  Slow and simple; the 128 x 128 kernel above is the one that is measured.
@@ -343,7 +664,12 @@ extern "C" int dflash_gdn_forward_tape(const void* q, const void* k, const void*
   const bool fast = Dk == 128 && Dv == 128 && T >= 1 && smem <= 64 * 1024 &&
                     (state_dtype != DFLASH_FP32 ||
                      (((uintptr_t)state_in % 16) == 0 && ((uintptr_t)state_out % 16) == 0));
-  if (fast) {
+  static const bool no_chunk = [] { const char* e = getenv("DFLASH_GDN_SEQUENTIAL"); return e && e[0] == '1'; }();
+  const bool aligned16 = (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)y | (uintptr_t)tape) % 16) == 0;
+  const bool chunk = fast && !g_per_dk && state_dtype == DFLASH_FP32 && T <= 16 && aligned16 && !no_chunk;
+  if (chunk) {
+    hipLaunchKernelGGL(gdn_forward_chunk_128, grid, block, kChunkLdsFloats * sizeof(float), s, a);
+  } else if (fast) {
     if (g_per_dk) {
       hipLaunchKernelGGL((gdn_forward_128<true, false>), grid, block, smem, s, a);
     } else if (state_dtype == DFLASH_FP32) {
