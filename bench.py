@@ -263,8 +263,10 @@ def bench_gdn_forward(device: str, steps: int, warmup: int):
     once out, v, y (bf16) and the tape (fp32) once, its share of q and k, g and beta."""
     import torch
 
-    from dflash_mlx_amd.kernels import gated_delta_kernel_with_tape
+    from dflash_mlx_amd import _native
+    from dflash_mlx_amd.kernels import _DTYPE_CODE
 
+    lib = _native.lib()
     L, Hk, Hv, T, D = 48, 16, 32, 16, 128
     gen = torch.Generator(device=device).manual_seed(0xDF1A + 2500)
     sets = []
@@ -277,10 +279,20 @@ def bench_gdn_forward(device: str, steps: int, warmup: int):
         g = torch.exp(-torch.nn.functional.softplus(torch.randn((L, T, Hv), generator=gen, device=device)))
         beta = torch.sigmoid(torch.randn((L, T, Hv), generator=gen, device=device)).to(torch.bfloat16)
         state = torch.randn((L, Hv, D, D), generator=gen, device=device) * 0.1
-        sets.append((q, k, v, g, beta, state))
+        # outputs allocated once: the timed region holds kernel launches only
+        outs = (torch.empty_like(state), torch.empty_like(v),
+                torch.empty((L, T, Hv, D), dtype=torch.float32, device=device))
+        sets.append((q, k, v, g, beta, state) + outs)
+    stream = torch.cuda.current_stream(device).cuda_stream
 
     def one_pass(i):
-        return gated_delta_kernel_with_tape(*sets[i % 4])
+        q, k, v, g, beta, state, state_out, y, tape = sets[i % 4]
+        rc = lib.dflash_gdn_forward_tape(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), beta.data_ptr(),
+            state.data_ptr(), state_out.data_ptr(), y.data_ptr(), tape.data_ptr(), None,
+            L, T, Hk, Hv, D, D, _DTYPE_CODE[q.dtype], _DTYPE_CODE[g.dtype], _DTYPE_CODE[beta.dtype],
+            _DTYPE_CODE[state.dtype], 0, stream)
+        _native.check(rc, "dflash_gdn_forward_tape")
 
     for i in range(max(warmup, 4)):
         one_pass(i)

@@ -298,34 +298,38 @@ constexpr int kOffQ = kOffK + 16 * kKPad;  // Q, then Delta[t][dv]
 constexpr int kOffV = kOffQ + 16 * kKPad;
 constexpr int kOffR = kOffV + 16 * 128;
 constexpr int kOffRat = kOffR + 128 * kRPad;  // c_t / c_s, 0 above the diagonal
-constexpr int kOffL = kOffRat + 256;
-constexpr int kOffLq = kOffL + 256;
+constexpr int kOffLq = kOffRat + 256;
 constexpr int kOffM = kOffLq + 256;  // (I + L)^-1
 constexpr int kOffC = kOffM + 256;
 constexpr int kOffBeta = kOffC + 16;   // 0 for masked and missing steps
 constexpr int kOffGate = kOffBeta + 16;  // 1 for masked and missing steps
 constexpr int kChunkLdsFloats = kOffGate + 16;
 
+// Eight consecutive elements of q, k or v as loaded: 16 bytes for the 16-bit types (WIDE = false),
+// 32 bytes for fp32.
+template <bool WIDE>
 struct Raw8 {
-  uint4 lo, hi;
+  uint4 w[WIDE ? 2 : 1];
 };
 // Eight consecutive elements from element i (a multiple of 8) of a 16-byte aligned array.
-__device__ __forceinline__ Raw8 load8_raw(const void* p, size_t i, int dt) {
-  Raw8 r;
-  r.hi = uint4{0u, 0u, 0u, 0u};
-  if (dt == DFLASH_FP32) {
+template <bool WIDE>
+__device__ __forceinline__ Raw8<WIDE> load8_raw(const void* p, size_t i) {
+  Raw8<WIDE> r;
+  if (WIDE) {
     const uint4* src = reinterpret_cast<const uint4*>((const float*)p + i);
-    r.lo = src[0];
-    r.hi = src[1];
+    r.w[0] = src[0];
+    r.w[WIDE ? 1 : 0] = src[1];
   } else {
-    r.lo = *reinterpret_cast<const uint4*>((const uint16_t*)p + i);
+    r.w[0] = *reinterpret_cast<const uint4*>((const uint16_t*)p + i);
   }
   return r;
 }
-__device__ __forceinline__ void raw8_to_lds(const Raw8& r, int dt, float* dst) {
-  const uint32_t w[8] = {r.lo.x, r.lo.y, r.lo.z, r.lo.w, r.hi.x, r.hi.y, r.hi.z, r.hi.w};
+template <bool WIDE>
+__device__ __forceinline__ void raw8_to_lds(const Raw8<WIDE>& r, int dt, float* dst) {
+  const uint4 hi = r.w[WIDE ? 1 : 0];
+  const uint32_t w[8] = {r.w[0].x, r.w[0].y, r.w[0].z, r.w[0].w, hi.x, hi.y, hi.z, hi.w};
   float o[8];
-  if (dt == DFLASH_FP32) {
+  if (WIDE) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) o[j] = __uint_as_float(w[j]);
   } else if (dt == DFLASH_BF16) {
@@ -379,6 +383,46 @@ __device__ __forceinline__ void swap_row_bit(f32x4_t& even, f32x4_t& odd) {
   }
 }
 
+// What one (slot, head) item brings in from memory, as it sits in registers while in flight.
+template <bool WIDE>
+struct Incoming {
+  Raw8<WIDE> k, q, v;
+  float gate, beta;
+  f32x4_t st[2][8];
+};
+template <bool WIDE>
+__device__ __forceinline__ void issue_item_loads(const GdnArgs& a, int item, int tid, Incoming<WIDE>& in) {
+  const int T = a.T;
+  const int slot = item / a.Hv, hv = item % a.Hv, hk = hv / (a.Hv / a.Hk);
+  const size_t slotT = (size_t)slot * T;
+  const int lane = tid & 63, wave = tid >> 6, li = lane & 15, kq = lane >> 4;
+  // the block's operands first, the state behind them: loads complete in order
+#pragma unroll
+  for (int j = 0; j < (WIDE ? 2 : 1); ++j) in.k.w[j] = in.q.w[j] = in.v.w[j] = uint4{0u, 0u, 0u, 0u};
+  const int t = tid >> 4, seg = tid & 15;
+  if (t < T) {
+    const size_t kq_at = ((slotT + t) * a.Hk + hk) * 128 + 8 * seg;
+    const size_t v_at = ((slotT + t) * a.Hv + hv) * 128 + 8 * seg;
+    in.k = load8_raw<WIDE>(a.k, kq_at);
+    in.q = load8_raw<WIDE>(a.q, kq_at);
+    in.v = load8_raw<WIDE>(a.v, v_at);
+  }
+  in.gate = 1.f;
+  in.beta = 0.f;
+  if (tid < T && (a.mask == nullptr || a.mask[slotT + tid] != 0)) {
+    in.gate = load_as_f32(a.g, (slotT + tid) * a.Hv + hv, a.g_dtype);
+    in.beta = load_as_f32(a.beta, (slotT + tid) * a.Hv + hv, a.beta_dtype);
+  }
+  const f32x4_t* src = reinterpret_cast<const f32x4_t*>((const float*)a.state_in + (size_t)item * 128 * 128);
+#pragma unroll
+  for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+      in.st[t2][c] = __builtin_nontemporal_load(&src[memory_index(wave, li, kq, t2, c)]);
+}
+
+// One workgroup per (slot, head); the register cap keeps at least three on a compute unit.
+template <bool WIDE>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void gdn_forward_chunk_128(GdnArgs a) {
   extern __shared__ __align__(16) float smem[];
   float* sK = smem + kOffK;
@@ -387,7 +431,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
   float* sV = smem + kOffV;
   float* sR = smem + kOffR;
   float* sRat = smem + kOffRat;
-  float* sL = smem + kOffL;
   float* sLq = smem + kOffLq;
   float* sM = smem + kOffM;
   float* sC = smem + kOffC;
@@ -395,60 +438,41 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
   float* sGate = smem + kOffGate;
 
   const int T = a.T;
-  const int slot = blockIdx.x / a.Hv, hv = blockIdx.x % a.Hv;
-  const int hk = hv / (a.Hv / a.Hk);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: branches on it are real branches
   const int li = lane & 15, kq = lane >> 4;
-  const size_t slotT = (size_t)slot * T;
-  const size_t sbase = (size_t)blockIdx.x * 128 * 128;
 
-  // ---- the block's operands first, the state behind them ------------------------------------
-  Raw8 rk, rq, rv;
-  rk.lo = rk.hi = rq.lo = rq.hi = rv.lo = rv.hi = uint4{0u, 0u, 0u, 0u};
+  Incoming<WIDE> cur;
+  const int item = blockIdx.x;
+  issue_item_loads(a, item, tid, cur);
+  const int slot = item / a.Hv, hv = item % a.Hv;
+  const size_t slotT = (size_t)slot * T;
+  const size_t sbase = (size_t)item * 128 * 128;
+  f32x4_t (&st)[2][8] = cur.st;
   {
     const int t = tid >> 4, seg = tid & 15;
-    if (t < T) {
-      const size_t kq_at = ((slotT + t) * a.Hk + hk) * 128 + 8 * seg;
-      const size_t v_at = ((slotT + t) * a.Hv + hv) * 128 + 8 * seg;
-      rk = load8_raw(a.k, kq_at, a.in_dtype);
-      rq = load8_raw(a.q, kq_at, a.in_dtype);
-      rv = load8_raw(a.v, v_at, a.in_dtype);
-    }
-  }
-  float gate = 1.f, beta = 0.f;
-  if (tid < T && (a.mask == nullptr || a.mask[slotT + tid] != 0)) {
-    gate = load_as_f32(a.g, (slotT + tid) * a.Hv + hv, a.g_dtype);
-    beta = load_as_f32(a.beta, (slotT + tid) * a.Hv + hv, a.beta_dtype);
-  }
-  f32x4_t st[2][8];
-  {
-    const f32x4_t* in = reinterpret_cast<const f32x4_t*>((const float*)a.state_in + sbase);
-#pragma unroll
-    for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-      for (int c = 0; c < 8; ++c)
-        st[t2][c] = __builtin_nontemporal_load(&in[memory_index(wave, li, kq, t2, c)]);
-  }
-  {
-    const int t = tid >> 4, seg = tid & 15;
-    raw8_to_lds(rk, a.in_dtype, sK + t * kKPad + 8 * seg);
-    raw8_to_lds(rq, a.in_dtype, sQ + t * kKPad + 8 * seg);
-    raw8_to_lds(rv, a.in_dtype, sV + t * 128 + 8 * seg);
+    raw8_to_lds(cur.k, a.in_dtype, sK + t * kKPad + 8 * seg);
+    raw8_to_lds(cur.q, a.in_dtype, sQ + t * kKPad + 8 * seg);
+    raw8_to_lds(cur.v, a.in_dtype, sV + t * 128 + 8 * seg);
   }
   if (tid < 16) {
-    sGate[tid] = gate;
-    sBeta[tid] = beta;
+    sGate[tid] = cur.gate;
+    sBeta[tid] = cur.beta;
   }
   __syncthreads();
   {  // c_t / c_s = prod_{s < u <= t} g_u for s <= t, and c_t itself
     const int t = tid >> 4, sx = tid & 15;
-    float r = 0.f;
-    if (sx <= t) {
-      r = 1.f;
-      for (int u = sx + 1; u <= t; ++u) r *= sGate[u];
+    float gates[16];
+#pragma unroll
+    for (int u = 0; u < 16; u += 4) {
+      const float4 g4 = *reinterpret_cast<const float4*>(sGate + u);
+      gates[u] = g4.x, gates[u + 1] = g4.y, gates[u + 2] = g4.z, gates[u + 3] = g4.w;
     }
+    float r = sx <= t ? 1.f : 0.f;
+#pragma unroll
+    for (int u = 1; u < 16; ++u) r *= (u > sx && u <= t) ? gates[u] : 1.f;
     sRat[tid] = r;
-    if (sx == 0) sC[t] = r * sGate[0];
+    if (sx == 0) sC[t] = r * gates[0];
   }
   __syncthreads();
 
@@ -480,12 +504,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
   {
     const int t = li;
     const float ct = sC[t], bt = sBeta[t];
+    float Lr[4];  // wave 1: L[t][4kq + r], wave 2: Lq[t][4kq + r]
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int sx = 4 * kq + r;
       const float rat = sRat[t * 16 + sx];  // 0 for s > t
-      if (wave == 1) sL[t * 16 + sx] = sx < t ? bt * rat * X[r] : 0.f;
-      if (wave == 2) sLq[t * 16 + sx] = rat * X[r];
+      Lr[r] = wave == 1 ? (sx < t ? bt * rat * X[r] : 0.f) : rat * X[r];
+      if (wave == 2) sLq[t * 16 + sx] = Lr[r];
     }
 #pragma unroll
     for (int t2 = 0; t2 < 2; ++t2) {
@@ -496,22 +521,24 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
       sR[(row0 + 2) * kRPad + t] = bt * (v4.z - ct * U[t2][2]);
       sR[(row0 + 3) * kRPad + t] = bt * (v4.w - ct * U[t2][3]);
     }
-  }
-  __syncthreads();  // L, Lq and R are complete; nobody reads Q any more
-
-  // ---- M = (I + L)^-1, column li per lane -----------------------------------------------------
-  if (wave == 1) {
-    float x[16];
+    // ---- M = (I + L)^-1 by forward substitution, column li per lane.  L[t][s] sits in lane
+    // 16 (s / 4) + t, register s % 4 of this wave and reaches the others through v_readlane.
+    if (wave == 1) {
+      float x[16];
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-      float acc = t == li ? 1.f : 0.f;
+      for (int tt = 0; tt < 16; ++tt) {
+        float acc = tt == li ? 1.f : 0.f;
 #pragma unroll
-      for (int sx = 0; sx < t; ++sx) acc -= sL[t * 16 + sx] * x[sx];
-      x[t] = acc;
-      if (kq == 0) sM[t * 16 + li] = acc;
+        for (int sx = 0; sx < tt; ++sx) {
+          const float l = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(Lr[sx & 3]), 16 * (sx >> 2) + tt));
+          acc -= l * x[sx];
+        }
+        x[tt] = acc;
+        if (kq == 0) sM[tt * 16 + li] = acc;
+      }
     }
   }
-  __syncthreads();
+  __syncthreads();  // Lq, R and M are complete; nobody reads Q any more
 
   // ---- Delta = R M^T: rows of this wave, accumulator (row 4kq + r, column t = li) ---------------
   f32x4_t D[2];
@@ -664,11 +691,18 @@ extern "C" int dflash_gdn_forward_tape(const void* q, const void* k, const void*
   const bool fast = Dk == 128 && Dv == 128 && T >= 1 && smem <= 64 * 1024 &&
                     (state_dtype != DFLASH_FP32 ||
                      (((uintptr_t)state_in % 16) == 0 && ((uintptr_t)state_out % 16) == 0));
-  static const bool no_chunk = [] { const char* e = getenv("DFLASH_GDN_SEQUENTIAL"); return e && e[0] == '1'; }();
+  // DFLASH_GDN_SEQUENTIAL=1 keeps the step-by-step kernel for every shape (read per call: A/B runs)
+  const char* sequential_env = getenv("DFLASH_GDN_SEQUENTIAL");
+  const bool no_chunk = sequential_env && sequential_env[0] == '1';
   const bool aligned16 = (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)y | (uintptr_t)tape) % 16) == 0;
   const bool chunk = fast && !g_per_dk && state_dtype == DFLASH_FP32 && T <= 16 && aligned16 && !no_chunk;
   if (chunk) {
-    hipLaunchKernelGGL(gdn_forward_chunk_128, grid, block, kChunkLdsFloats * sizeof(float), s, a);
+    const size_t lds = kChunkLdsFloats * sizeof(float);
+    if (in_dtype == DFLASH_FP32) {
+      hipLaunchKernelGGL(gdn_forward_chunk_128<true>, grid, block, lds, s, a);
+    } else {
+      hipLaunchKernelGGL(gdn_forward_chunk_128<false>, grid, block, lds, s, a);
+    }
   } else if (fast) {
     if (g_per_dk) {
       hipLaunchKernelGGL((gdn_forward_128<true, false>), grid, block, smem, s, a);

@@ -124,6 +124,49 @@ def test_other_shapes(native_lib, shape):
     assert _rel(_f64(s), so) <= 2e-5 and _rel(_f64(tape), to) <= 2e-5 and _rel(_f64(y), yo) <= 4e-3
 
 
+@pytest.mark.parametrize("T", [1, 2, 7, 15, 16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_closed_form_block_lengths(native_lib, T, dtype):
+    """Scalar gate, fp32 state, 128 x 128 heads, T <= 16: the block kernel on the matrix cores,
+    every block length with a ragged mask, against the fp64 oracle."""
+    args = _case(B=2, T=T, Hk=2, Hv=4, seed=20 + T, dtype=dtype)
+    mask = torch.ones((2, T), dtype=torch.bool)
+    mask[1, T // 2] = False
+    y, s, tape = _run(args, mask)
+    yo, so, to = O.gated_delta_ops_with_tape(*[_f64(t) for t in args], mask=mask.numpy())
+    assert _rel(_f64(s), so) <= 2e-5 and _rel(_f64(tape), to) <= 2e-5
+    eps = {torch.bfloat16: 2.0 ** -8, torch.float32: 2.0 ** -20}[dtype]
+    assert np.all(np.abs(_f64(y) - yo) <= eps * np.abs(yo) + 2e-5 * np.abs(yo).max())
+
+
+def test_closed_form_with_vanishing_gates(native_lib):
+    """Gates near 1e-4 per step: the running product leaves the fp32 range after a few steps,
+    the ratios c_t / c_s between neighbouring steps do not.  Also gates of exactly 0 and 1."""
+    q, k, v, gate, beta, state = _case(B=2, Hk=2, Hv=4, seed=31)
+    gate = gate * 1e-4
+    gate[0, 3, 1] = 0.0
+    gate[1, :, 2] = 1.0
+    args = (q, k, v, gate, beta, state)
+    y, s, tape = _run(args)
+    yo, so, to = O.gated_delta_ops_with_tape(*[_f64(t) for t in args])
+    assert np.all(np.isfinite(_f64(s))) and np.all(np.isfinite(_f64(tape)))
+    assert _rel(_f64(s), so) <= 2e-5 and _rel(_f64(tape), to) <= 2e-5 and _rel(_f64(y), yo) <= 4e-3
+
+
+def test_closed_form_equals_the_sequential_kernel(native_lib, monkeypatch):
+    """The two kernels for the same shape differ only in the order of fp32 additions."""
+    args = _case(B=2, Hk=4, Hv=8, seed=33)
+    mask = torch.ones((2, 16), dtype=torch.bool)
+    mask[0, 5:8] = False
+    block = _run(args, mask)
+    monkeypatch.setenv("DFLASH_GDN_SEQUENTIAL", "1")
+    steps = _run(args, mask)
+    monkeypatch.delenv("DFLASH_GDN_SEQUENTIAL")
+    for a, b in zip(block, steps):
+        assert _rel(_f64(a), _f64(b)) <= 2e-5
+    assert _rel(_f64(block[2]), _f64(steps[2])) > 0     # two different kernels did run
+
+
 def test_errors_and_host_tensors(native_lib):
     q, k, v, gate, beta, state = _case(B=1, T=2, Hk=3, Hv=4, Dk=32, Dv=8)
     with pytest.raises(ValueError, match="Cannot align"):
