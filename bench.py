@@ -313,6 +313,68 @@ def bench_gdn_forward(device: str, steps: int, warmup: int):
                 frac_hbm=total / (us * 1e-6) / HBM_PEAK, bytes=total, layers=L, heads=Hv, steps=T)
 
 
+def bench_gdn_glue(device: str, steps: int, warmup: int):
+    """The operators around the recurrence of one GatedDeltaNet layer at the verify shape
+    (1 x 16 tokens, 16 key and 32 value heads of 128, conv over 8192 channels): the two fused
+    launches through the C ABI (outputs allocated beforehand), the same through the Python
+    wrappers (allocations included), and the same operators one by one in torch on the device."""
+    import torch
+
+    from dflash_mlx_amd import _native
+    from dflash_mlx_amd import gdn_layer as G
+    from dflash_mlx_amd.kernels import _DTYPE_CODE
+
+    lib = _native.lib()
+    B, S, Hk, Hv, D, K = 1, 16, 16, 32, 128, 4
+    C = 2 * Hk * D + Hv * D
+    gen = torch.Generator(device=device).manual_seed(0xDF1A + 2600)
+    bf = torch.bfloat16
+    rnd = lambda *shape: torch.randn(shape, generator=gen, device=device)
+    qkv, conv_state, conv_w = rnd(B, S, C).to(bf), rnd(B, K - 1, C).to(bf), (rnd(C, K) * 0.4).to(bf)
+    a, b, A_log, dt_bias = rnd(B, S, Hv).to(bf), rnd(B, S, Hv).to(bf), rnd(Hv).to(bf), rnd(Hv).to(bf)
+    x, z, w = rnd(B, S, Hv, D).to(bf), rnd(B, S, Hv, D).to(bf), (1 + 0.1 * rnd(D)).to(bf)
+    conv_next = torch.empty((B, K - 1, C), dtype=bf, device=device)
+    q, k = (torch.empty((B, S, Hk, D), dtype=bf, device=device) for _ in range(2))
+    v, y = (torch.empty((B, S, Hv, D), dtype=bf, device=device) for _ in range(2))
+    g = torch.empty((B, S, Hv), dtype=torch.float32, device=device)
+    beta = torch.empty((B, S, Hv), dtype=bf, device=device)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    code = _DTYPE_CODE[bf]
+
+    def abi():
+        rc = lib.dflash_gdn_prepare(qkv.data_ptr(), conv_state.data_ptr(), conv_w.data_ptr(), a.data_ptr(),
+                                    b.data_ptr(), A_log.data_ptr(), dt_bias.data_ptr(), None, conv_next.data_ptr(),
+                                    q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), beta.data_ptr(),
+                                    B, S, Hk, Hv, D, D, K, code, code, 1e-6, stream)
+        rc |= lib.dflash_gdn_gated_norm(x.data_ptr(), z.data_ptr(), w.data_ptr(), y.data_ptr(), B * S * Hv, D,
+                                        code, code, 1e-6, stream)
+        _native.check(rc, "gdn glue")
+
+    def wrappers():
+        G.gdn_prepare(qkv, conv_state, conv_w, a, b, A_log, dt_bias, None, Hk=Hk, Hv=Hv, Dk=D, Dv=D)
+        G.gated_norm(x, z, w)
+
+    def array_ops():
+        G.gdn_prepare_ops(qkv, conv_state, conv_w, a, b, A_log, dt_bias, None, Hk=Hk, Hv=Hv, Dk=D, Dv=D)
+        G.gated_norm_ops(x, z, w)
+
+    out = {}
+    n = max(steps * 10, 48)
+    for name, fn in (("fused_c_abi", abi), ("fused_python_wrappers", wrappers), ("torch_array_ops", array_ops)):
+        for _ in range(max(warmup, 3)):
+            fn()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(n):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        out[name + "_us_per_layer"] = start.elapsed_time(stop) / n * 1e3
+    out["launches_fused"] = 2
+    return out
+
+
 def bench_cpu_baseline(stack: str, budget_s: float = 12.0):
     """The oracle's C port of the reference kernel arithmetic (bf16-rounded dequantised
     weights, fp32 accumulation) on the host cores: whole layers of the same stack, one
@@ -400,6 +462,8 @@ def main() -> int:
         fw = bench_gdn_forward(device, args.steps, args.warmup)
         log(f"forward with tape: {fw['us_per_layer']:.3f} us/layer, {fw['gbps']:.0f} GB/s")
         extra["gdn_forward_with_tape"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in fw.items()}
+        gl = bench_gdn_glue(device, args.steps, args.warmup)
+        extra["gdn_layer_glue"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in gl.items()}
         log(f"[bench] replay: {rp['us_per_layer']:.3f} us/layer, {rp['gbps']:.0f} GB/s")
 
     achieved = main_res["bytes_per_launch"] / (main_res["avg_launch_us"] * 1e-6) / 1e9

@@ -61,6 +61,17 @@ __device__ __forceinline__ float load_as_f32(const void* p, size_t i, int dt) {
   return ((const float*)p)[i];
 }
 
+// Store v as element i of an array whose element type is one of the DFLASH_* dtypes (RNE).
+__device__ __forceinline__ void store_from_f32(void* p, size_t i, float v, int dt) {
+  if (dt == DFLASH_BF16) {
+    ((uint16_t*)p)[i] = (uint16_t)f32_to_bf16_bits(v);
+  } else if (dt == DFLASH_FP16) {
+    ((uint16_t*)p)[i] = (uint16_t)f32_to_f16_bits(v);
+  } else {
+    ((float*)p)[i] = v;
+  }
+}
+
 __device__ __forceinline__ float round_through(float v, int dt) {
   if (dt == DFLASH_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(v));
   if (dt == DFLASH_FP16) return f16_bits_to_f32(f32_to_f16_bits(v));

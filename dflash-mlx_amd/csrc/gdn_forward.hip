@@ -52,16 +52,6 @@ struct GdnArgs {
   int in_dtype, g_dtype, beta_dtype, state_dtype, g_per_dk;
 };
 
-__device__ __forceinline__ void store_from_f32(void* p, size_t i, float v, int dt) {
-  if (dt == DFLASH_BF16) {
-    ((uint16_t*)p)[i] = (uint16_t)f32_to_bf16_bits(v);
-  } else if (dt == DFLASH_FP16) {
-    ((uint16_t*)p)[i] = (uint16_t)f32_to_f16_bits(v);
-  } else {
-    ((float*)p)[i] = v;
-  }
-}
-
 // v + (v of the lane the DPP control names): butterfly steps inside a row of 16 lanes -
 // quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror (lanes of an aligned group of 8),
 // row_mirror (the two groups of 8).

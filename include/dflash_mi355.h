@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 4
+#define DFLASH_ABI_VERSION 5
 
 enum {
   DFLASH_OK = 0,
@@ -157,14 +157,49 @@ int dflash_tape_replay(const void* tape, const void* k, const void* g, const voi
  *   y         [slots, T, Hv, Dv]   in_dtype (output)
  *   tape      [slots, T, Hv, Dv]   fp32 (output)
  *   mask      [slots, T] uint8 or NULL
- * 128 x 128 heads with T*(3*128 + (g_per_dk ? 128 : 1) + 2)*4 bytes <= 64 KiB of LDS take the
- * register-resident kernel; every other shape a simple one that keeps S in state_out.
+ * 128 x 128 heads take register-resident kernels: one gate per head with an fp32 state and
+ * T <= 16 the block kernel on the fp32 matrix cores (closed form of the recurrence; the
+ * environment variable DFLASH_GDN_SEQUENTIAL=1 turns it off), the rest a step-by-step kernel
+ * while T*(3*128 + (g_per_dk ? 128 : 1) + 2)*4 bytes fit 64 KiB of LDS; every other shape a
+ * simple kernel that keeps S in state_out.
  */
 int dflash_gdn_forward_tape(const void* q, const void* k, const void* v, const void* g,
                             const void* beta, const void* state_in, void* state_out, void* y,
                             float* tape, const uint8_t* mask, int slots, int T, int Hk, int Hv,
                             int Dk, int Dv, int in_dtype, int g_dtype, int beta_dtype,
                             int state_dtype, int g_per_dk, void* stream);
+
+/*
+ * GatedDeltaNet layer, everything between the input projections and the recurrence, in one
+ * launch.  Replaces the array operators of dflash_mlx/runtime.py:381-407:
+ *     qkv <- where(mask, qkv, 0);  conv_input = [conv_state | qkv] along the steps;
+ *     conv_next = last conv_kernel-1 rows of conv_input;
+ *     act = silu(depthwise_conv(conv_input));  q, k, v = split(act) into heads;
+ *     q = Dk^-1 * rms_norm(q, eps);  k = Dk^-1/2 * rms_norm(k, eps);
+ *     g = exp(-exp(A_log) * softplus(a + dt_bias));  beta = sigmoid(b).
+ * Each of those operators rounds to `dtype` once (fp32 inside), a + dt_bias and the softplus
+ * to the promoted type of `dtype` and `param_dtype`; g is fp32.
+ *
+ *   qkv         [B, S, C]  dtype, C = 2*Hk*Dk + Hv*Dv (q heads, k heads, v heads)
+ *   conv_state  [B, conv_kernel-1, C] dtype, or NULL for zeros
+ *   conv_w      [C, conv_kernel] dtype; tap j multiplies conv_input row s + j
+ *   a, b        [B, S, Hv] dtype;  A_log, dt_bias [Hv] param_dtype;  mask [B, S] uint8 or NULL
+ *   outputs: conv_next [B, conv_kernel-1, C], q, k [B, S, Hk, Dk], v [B, S, Hv, Dv], beta
+ *   [B, S, Hv] in dtype; g [B, S, Hv] fp32.  Dk, Dv multiples of 64 up to 256.
+ */
+int dflash_gdn_prepare(const void* qkv, const void* conv_state, const void* conv_w, const void* a,
+                       const void* b, const void* A_log, const void* dt_bias, const uint8_t* mask,
+                       void* conv_next, void* q, void* k, void* v, float* g, void* beta, int B,
+                       int S, int Hk, int Hv, int Dk, int Dv, int conv_kernel, int dtype,
+                       int param_dtype, float eps, void* stream);
+
+/*
+ * Gated output norm of a GatedDeltaNet layer: y = silu(z) * rms_norm(x, weight, eps) over rows of
+ * length D (a multiple of 64 up to 256), x, z, y [rows, D] in dtype, weight [D] in weight_dtype.
+ * Replaces `self.norm(out, z)` at dflash_mlx/runtime.py:448 (mlx-lm's Qwen3NextRMSNormGated).
+ */
+int dflash_gdn_gated_norm(const void* x, const void* z, const void* weight, void* y, long long rows,
+                          int D, int dtype, int weight_dtype, float eps, void* stream);
 
 /*
  * Conv-window rebuild of a GatedDeltaNet layer after a partial acceptance: output

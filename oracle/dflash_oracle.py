@@ -27,8 +27,11 @@ a re-typed formula):
   acceptance     - exhaustive brute force over all small index patterns.
 * parity unpinned: bit-level rounding/accumulation order of MLX's own
   ``mx.quantized_matmul`` on ``mx.cpu`` (third-party mlx >= 0.25, not present
-  in this build environment) - absorbed by the stated tolerance band; and the
-  gathered per-expert qmm, which has no counterpart in the reference.
+  in this build environment) - absorbed by the stated tolerance band; the
+  gathered per-expert qmm, which has no counterpart in the reference; and the
+  rounding points inside the GatedDeltaNet layer glue (gdn_prepare, gdn_gated_norm),
+  whose operators belong to mlx / mlx-lm - their mathematics is pinned against torch
+  and fp64 closed forms, the placement of single bf16 roundings is not.
 """
 from __future__ import annotations
 
@@ -413,6 +416,97 @@ def tape_replay_unrolled(tape, k, g, state, steps: int):
                 acc = acc + c * np.outer(tape[b, t, hv], k[b, t, hk])
             out[b, hv] = acc
     return out
+
+
+# ----------------------------------------------------------------------------
+# GatedDeltaNet layer glue around the forward kernel (runtime.py:344-455)
+# ----------------------------------------------------------------------------
+# The reference's speculative call strings together operators of the third-party
+# packages mlx (conv1d, mx.fast.rms_norm, sigmoid, softplus) and mlx-lm >= 0.31
+# (gated_delta.compute_g, Qwen3NextRMSNormGated); neither is present here, so the
+# formulas below are their published definitions and the *rounding points* (one
+# rounding to the array dtype after every array-level operator, fp32 inside an
+# operator) are this restatement's choice: parity unpinned at the level of single
+# roundings.  What the tests pin is the mathematics: the depthwise convolution
+# against torch.nn.functional.conv1d, the norms and gates against fp64 closed forms,
+# the conv-state hand-over against rebuild_conv_state, and the whole call against a
+# step-by-step evaluation with the layer's plain (non-speculative) path.
+
+
+def _sigmoid32(x):
+    x = np.asarray(x, dtype=np.float32)
+    return (np.float32(1.0) / (np.float32(1.0) + np.exp(-x))).astype(np.float32)
+
+
+def _softplus32(x):
+    x = np.asarray(x, dtype=np.float32)
+    return np.logaddexp(x, np.float32(0.0)).astype(np.float32)
+
+
+def silu_rounded(x, dtype: str):
+    """mlx.nn.silu = x * sigmoid(x), each operator rounded to the array dtype."""
+    x = np.asarray(x, dtype=np.float32)
+    return round_to(x * round_to(_sigmoid32(x), dtype), dtype)
+
+
+def rms_norm_rounded(x, weight, eps: float, dtype: str):
+    """mx.fast.rms_norm: x * rsqrt(mean(x^2) + eps) [* weight], fp32 inside, one rounding."""
+    x = np.asarray(x, dtype=np.float32)
+    ms = np.mean(x * x, axis=-1, keepdims=True, dtype=np.float32)
+    y = x * (np.float32(1.0) / np.sqrt(ms + np.float32(eps)))
+    if weight is not None:
+        y = y * np.asarray(weight, dtype=np.float32)
+    return round_to(y, dtype)
+
+
+def compute_g(A_log, a, dt_bias, dtype: str, bias_dtype: Optional[str] = None):
+    """mlx_lm gated_delta.compute_g: exp(-exp(A_log as fp32) * softplus(a + dt_bias)), fp32 out.
+    a + dt_bias and the softplus live in the promoted dtype of a and dt_bias."""
+    sum_dtype = "fp32" if (bias_dtype or dtype) == "fp32" else dtype
+    apb = round_to(np.asarray(a, np.float32) + np.asarray(dt_bias, np.float32), sum_dtype)
+    sp = round_to(_softplus32(apb), sum_dtype)
+    return np.exp(-np.exp(np.asarray(A_log, np.float32)) * sp).astype(np.float32)
+
+
+def gdn_prepare(qkv, conv_state, conv_w, a, b, A_log, dt_bias, *, Hk: int, Hv: int, Dk: int, Dv: int,
+                mask=None, dtype: str = "bf16", bias_dtype: Optional[str] = None, eps: float = 1e-6):
+    """runtime.py:381-407: everything between the input projections and the recurrence.
+    qkv [B,S,C] with C = 2*Hk*Dk + Hv*Dv, conv_state [B,K-1,C] or None, conv_w [C,K]
+    (depthwise taps, tap j multiplies conv_input[:, s+j]), a, b [B,S,Hv].  Values are fp32
+    arrays already representable in ``dtype``.  Returns (conv_next, q, k, v, g, beta)."""
+    qkv = np.asarray(qkv, dtype=np.float32)
+    conv_w = np.asarray(conv_w, dtype=np.float32)
+    B, S, C = qkv.shape
+    K = conv_w.shape[1]
+    keep = K - 1
+    key_dim = Hk * Dk
+    assert C == 2 * key_dim + Hv * Dv and conv_w.shape[0] == C
+    if mask is not None:
+        qkv = np.where(np.asarray(mask, dtype=bool)[..., None], qkv, np.float32(0.0))
+    prefix = np.zeros((B, keep, C), np.float32) if conv_state is None else np.asarray(conv_state, np.float32)
+    conv_input = np.concatenate([prefix, qkv], axis=1)
+    conv_next = np.ascontiguousarray(conv_input[:, conv_input.shape[1] - keep:])
+    acc = np.zeros((B, S, C), np.float32)
+    for j in range(K):
+        acc = acc + conv_input[:, j:j + S] * conv_w[None, None, :, j]
+    act = silu_rounded(round_to(acc, dtype), dtype)
+    q = act[..., :key_dim].reshape(B, S, Hk, Dk)
+    k = act[..., key_dim:2 * key_dim].reshape(B, S, Hk, Dk)
+    v = np.ascontiguousarray(act[..., 2 * key_dim:].reshape(B, S, Hv, Dv))
+    inv_scale = float(Dk) ** -0.5
+    scale_q = round_to(np.float32(inv_scale ** 2), dtype)
+    scale_k = round_to(np.float32(inv_scale), dtype)
+    q = round_to(scale_q * rms_norm_rounded(q, None, eps, dtype), dtype)
+    k = round_to(scale_k * rms_norm_rounded(k, None, eps, dtype), dtype)
+    g = compute_g(A_log, a, dt_bias, dtype, bias_dtype)
+    beta = round_to(_sigmoid32(b), dtype)
+    return conv_next, q, k, v, g, beta
+
+
+def gdn_gated_norm(x, z, weight, dtype: str = "bf16", eps: float = 1e-6):
+    """Qwen3NextRMSNormGated (mlx-lm): silu(z) * rms_norm(x, weight, eps); x, z [..., Dv]."""
+    y = rms_norm_rounded(x, weight, eps, dtype)
+    return round_to(silu_rounded(z, dtype) * y, dtype)
 
 
 # ----------------------------------------------------------------------------
