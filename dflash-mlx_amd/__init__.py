@@ -9,5 +9,8 @@ meaning and fallback behaviour), backed by hand-written gfx950 kernels in
 * ``RecurrentRollbackCache`` / ``tape_replay_kernel`` - GatedDeltaNet tape-replay
   rollback; ``RollbackArena`` - the same for all layers in one launch;
   ``KVCache.trim`` - attention-cache trim.
+* ``gated_delta_kernel_with_tape`` - the GatedDeltaNet forward that records the tape;
+  ``gdn_layer`` - the layer call around it (fused glue kernels, pad-to-16 projections);
+  ``loader`` - MLX-format 4-bit checkpoints; ``generate`` - the speculative cycle.
 """
 __version__ = "0.1.0"

@@ -1,0 +1,85 @@
+"""End to end on the device: the small hybrid model in bf16 with its 4-bit projections swapped
+to the verify kernel, GatedDeltaNet layers on the fused glue and recurrence kernels, rollback by
+tape replay, conv rebuild and KV trim - driven by the speculative cycle.
+
+Every committed token comes out of a 16-row verify forward, whatever the draft proposed, so
+runs with different drafts must agree token for token.  Against plain token-by-token decoding
+(1-row forwards through the stock matmul) bf16 rounding differs, so there the sequences may
+part ways only where the two best logits are nearly tied."""
+import pytest
+import torch
+
+from dflash_mlx_amd.generate import generate_greedy, generate_speculative
+from dflash_mlx_amd.runtime import make_target_cache
+from dflash_mlx_amd.verify_linear import VerifyQuantizedLinear, install_verify_linears
+from _toy_lm import ToyHybridLM, drafts
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _model(seed):
+    model = ToyHybridLM(seed=seed, hidden=512, Hk=2, Hv=4, D=128, dtype=torch.bfloat16).to(DEV)
+    swapped = install_verify_linears(model)
+    assert swapped == sum(isinstance(m, VerifyQuantizedLinear) for m in model.modules()) > 0
+    return model.install_hooks()
+
+
+def _cache(model, fp32_state):
+    cache = make_target_cache(model.pattern)
+    if fp32_state:
+        for layer, c in zip(model.layers, cache):
+            if layer.is_linear:
+                la = layer.linear_attn
+                c[1] = torch.zeros((1, la.num_v_heads, la.head_v_dim, la.head_k_dim), dtype=torch.float32, device=DEV)
+    return cache
+
+
+def _same_or_parting_at_a_near_tie(model, prompt, a, b, fp32_state):
+    """Two token sequences are equal, or where they first differ the plain path's two best
+    logits are within 5 % of the logits' spread and are exactly those two tokens."""
+    n = min(a.shape[0], b.shape[0])
+    diverged = (a[:n] != b[:n]).nonzero()
+    if not diverged.numel():
+        return True
+    at = int(diverged[0])
+    with torch.no_grad():
+        logits = model(torch.cat([prompt, a[:at]])[None], _cache(model, fp32_state))[0, -1]
+    top = torch.topk(logits, 2)
+    assert float(top.values[0] - top.values[1]) < 0.05 * float(logits.std()), (at, top.values)
+    assert {int(a[at]), int(b[at])} == set(top.indices.tolist())
+    return False
+
+
+@pytest.mark.parametrize("fp32_state", [True, False])
+def test_speculative_decoding_on_the_device(native_lib, monkeypatch, fp32_state):
+    monkeypatch.setenv("DFLASH_VERIFY_QMM", "1")
+    model = _model(11)
+    target = lambda ids, cache: model(ids, cache)
+    prompt = torch.randint(0, 384, (11,), generator=torch.Generator().manual_seed(5)).to(DEV)
+    n_new = 64
+    greedy = generate_greedy(target, _cache(model, fp32_state), prompt, n_new)
+
+    # a draft that is never right: every committed token is the target's own
+    histories = {"random": [], "perfect": [], "partly": []}
+    spec = generate_speculative(target, drafts(greedy.cpu(), 384, seed=3)["random"], _cache(model, fp32_state),
+                                prompt, n_new, block_tokens=16, acceptance_history=histories["random"])
+    assert max(histories["random"]) <= 2
+    # drafts that know that sequence: whole blocks are accepted, and nothing changes
+    runs = {}
+    for kind in ("perfect", "partly"):
+        runs[kind] = generate_speculative(target, drafts(spec.cpu(), 384, seed=3)[kind], _cache(model, fp32_state),
+                                          prompt, n_new, block_tokens=16, acceptance_history=histories[kind])
+    torch.cuda.synchronize()
+    if fp32_state:
+        # an fp32 state is the same to ~1e-7 however the blocks fall: no token moves
+        assert torch.equal(runs["perfect"], spec) and torch.equal(runs["partly"], spec)
+        assert histories["perfect"][:3] == [15, 15, 15] and len(histories["perfect"]) == 4
+    else:
+        # a bf16 state is rounded after every step, by the forward and by the replay: block
+        # boundaries move single roundings, which may decide a near-tie
+        for kind in ("perfect", "partly"):
+            _same_or_parting_at_a_near_tie(model, prompt, runs[kind], spec, fp32_state)
+    assert 0 < sum(histories["partly"]) < n_new
+    # against 1-row decoding through the stock matmul
+    _same_or_parting_at_a_near_tie(model, prompt, spec, greedy, fp32_state)
