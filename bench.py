@@ -375,6 +375,65 @@ def bench_gdn_glue(device: str, steps: int, warmup: int):
     return out
 
 
+def bench_sdpa(device: str, steps: int, warmup: int):
+    """Attention of the 16-token verify block over the KV caches of config[2]'s 16 full-attention
+    layers: 8 key/value heads of 256 over 4096 + 16 positions (bf16, read in place from buffers of
+    capacity 4352), 32 query heads.  Algorithmic bytes per layer: K and V once, q and out once."""
+    import torch
+
+    from dflash_mlx_amd import _native
+    from dflash_mlx_amd.kernels import _DTYPE_CODE
+
+    lib = _native.lib()
+    L, B, Hq, Hk, N, D, cap = 16, 1, 32, 8, 4112, 256, 4352
+    bf = torch.bfloat16
+    gen = torch.Generator(device=device).manual_seed(0xDF1A + 2700)
+    caches = [(torch.randn((B, Hk, cap, D), generator=gen, device=device).to(bf),
+               torch.randn((B, Hk, cap, D), generator=gen, device=device).to(bf)) for _ in range(L)]
+    q = torch.randn((B, Hq, 16, D), generator=gen, device=device).to(bf)
+    out = torch.empty_like(q)
+    need = int(lib.dflash_sdpa_q16_workspace_bytes(B, Hq, Hk, N, D))
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    scale = D ** -0.5
+
+    def kernel_pass():
+        for kbuf, vbuf in caches:
+            rc = lib.dflash_sdpa_q16(q.data_ptr(), kbuf.data_ptr(), vbuf.data_ptr(), None, out.data_ptr(),
+                                     ws.data_ptr(), ws.numel(), B, Hq, Hk, N, D, kbuf.stride(0), kbuf.stride(1),
+                                     kbuf.stride(2), vbuf.stride(0), vbuf.stride(1), vbuf.stride(2), scale,
+                                     _DTYPE_CODE[bf], stream)
+            _native.check(rc, "dflash_sdpa_q16")
+
+    allow = (torch.arange(N, device=device)[None, :] <= (N - 16 + torch.arange(16, device=device))[:, None])
+
+    def torch_pass():
+        for kbuf, vbuf in caches:
+            torch.nn.functional.scaled_dot_product_attention(q, kbuf[:, :, :N], vbuf[:, :, :N], attn_mask=allow,
+                                                             scale=scale, enable_gqa=True)
+
+    res = {}
+    for name, fn in (("kernel", kernel_pass), ("torch_sdpa", torch_pass)):
+        for _ in range(max(warmup, 2)):
+            fn()
+        n = max(steps, 5)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(n):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        res[name + "_us_per_layer"] = start.elapsed_time(stop) / n / L * 1e3
+    per_layer = 2 * B * Hk * N * D * 2 + 2 * B * Hq * 16 * D * 2
+    us = res["kernel_us_per_layer"]
+    res.update(bytes_per_layer=per_layer, gbps=per_layer / us / 1e3, frac_hbm=per_layer / (us * 1e-6) / HBM_PEAK,
+               workspace_bytes=need, layers=L, kv_len=N)
+    del caches
+    torch.cuda.empty_cache()
+    return res
+
+
 def bench_cpu_baseline(stack: str, budget_s: float = 12.0):
     """The oracle's C port of the reference kernel arithmetic (bf16-rounded dequantised
     weights, fp32 accumulation) on the host cores: whole layers of the same stack, one
@@ -462,6 +521,8 @@ def main() -> int:
         fw = bench_gdn_forward(device, args.steps, args.warmup)
         log(f"forward with tape: {fw['us_per_layer']:.3f} us/layer, {fw['gbps']:.0f} GB/s")
         extra["gdn_forward_with_tape"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in fw.items()}
+        sd = bench_sdpa(device, args.steps, args.warmup)
+        extra["sdpa_q16_kv4112"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in sd.items()}
         gl = bench_gdn_glue(device, args.steps, args.warmup)
         extra["gdn_layer_glue"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in gl.items()}
         log(f"[bench] replay: {rp['us_per_layer']:.3f} us/layer, {rp['gbps']:.0f} GB/s")

@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
@@ -30,6 +30,8 @@ EXPORTED_SYMBOLS = (
     "dflash_gdn_forward_tape",
     "dflash_gdn_prepare",
     "dflash_gdn_gated_norm",
+    "dflash_sdpa_q16_workspace_bytes",
+    "dflash_sdpa_q16",
     "dflash_conv_state_rebuild",
 )
 
@@ -65,6 +67,11 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.dflash_gdn_prepare.argtypes = [c.c_void_p] * 14 + [c.c_int] * 9 + [c.c_float, c.c_void_p]
     lib.dflash_gdn_gated_norm.restype = c.c_int
     lib.dflash_gdn_gated_norm.argtypes = [c.c_void_p] * 4 + [c.c_longlong] + [c.c_int] * 3 + [c.c_float, c.c_void_p]
+    lib.dflash_sdpa_q16_workspace_bytes.restype = c.c_size_t
+    lib.dflash_sdpa_q16_workspace_bytes.argtypes = [c.c_int] * 5
+    lib.dflash_sdpa_q16.restype = c.c_int
+    lib.dflash_sdpa_q16.argtypes = ([c.c_void_p] * 6 + [c.c_size_t] + [c.c_int] * 5 + [c.c_longlong] * 6 +
+                                    [c.c_float, c.c_int, c.c_void_p])
     lib.dflash_tape_replay.restype = c.c_int
     lib.dflash_tape_replay.argtypes = (
         [c.c_void_p] * 6 + [c.c_int] + [c.c_void_p] + [c.c_int] * 12 + [c.c_void_p]

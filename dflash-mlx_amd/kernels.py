@@ -208,3 +208,67 @@ def tape_replay_kernel(tape: torch.Tensor, k: torch.Tensor, g: torch.Tensor, sta
     replay_launch(tape_c, k_c, g_c, state_c, state_out, steps=steps, T_alloc=T_tape, mask=mask,
                   slots=bsz)
     return state_out
+
+
+_SDPA_WORKSPACE: dict = {}
+
+
+def _sdpa_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    """Partial results of the key ranges, one buffer per device and stream, grown on demand."""
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    buf = _SDPA_WORKSPACE.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _SDPA_WORKSPACE[key] = buf
+    return buf
+
+
+def batched_sdpa_2pass_exact(queries: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, scale: float,
+                             mask: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """Exact attention of a 16-token verify block over a long KV cache (mirror of
+    dflash_mlx/kernels.py:658-761): queries [B,Hq,16,D], keys / values [B,Hk,N,D] (views of a
+    cache are read in place), mask None, bool or additive, broadcastable to [B,Hq,16,N].
+    Query i attends to keys n <= N - 16 + i.  Returns None - the caller then takes its
+    general attention - for everything the kernel does not cover, as the reference does:
+    host tensors, q_len != 16, dtypes other than bf16 / fp16, head dims other than 128 / 256,
+    more than 8 query heads per key/value head."""
+    if queries.ndim != 4 or keys.ndim != 4 or values.ndim != 4 or not queries.is_cuda:
+        return None
+    bsz, hq, q_len, d = (int(x) for x in queries.shape)
+    hk, n_kv = int(keys.shape[1]), int(keys.shape[2])
+    vdim = int(values.shape[-1])
+    if q_len != 16 or queries.dtype not in (torch.bfloat16, torch.float16):
+        return None
+    if d not in (128, 256) or d != vdim or hk <= 0 or hq % hk != 0 or hq // hk > 8 or n_kv < 16:
+        return None
+    if keys.dtype != queries.dtype or values.dtype != queries.dtype or tuple(values.shape[:3]) != tuple(keys.shape[:3]):
+        return None
+
+    def in_place(t: torch.Tensor) -> torch.Tensor:
+        ok = t.stride(3) == 1 and all(s % 8 == 0 for s in t.stride()[:3]) and t.data_ptr() % 16 == 0
+        return t if ok else t.contiguous()
+
+    queries = queries.contiguous()
+    keys, values = in_place(keys), in_place(values)
+    mask_tensor = None
+    if mask is not None:
+        if mask.dtype == torch.bool:
+            mask_tensor = torch.where(mask, torch.zeros((), dtype=queries.dtype, device=mask.device),
+                                      torch.full((), torch.finfo(queries.dtype).min, dtype=queries.dtype,
+                                                 device=mask.device))
+        else:
+            mask_tensor = mask.to(queries.dtype)
+        mask_tensor = torch.broadcast_to(mask_tensor, (bsz, hq, q_len, n_kv)).contiguous()
+
+    lib = _native.lib()
+    out = torch.empty_like(queries)
+    need = int(lib.dflash_sdpa_q16_workspace_bytes(bsz, hq, hk, n_kv, d))
+    ws = _sdpa_workspace(queries.device, need) if need else None
+    rc = lib.dflash_sdpa_q16(
+        queries.data_ptr(), keys.data_ptr(), values.data_ptr(),
+        None if mask_tensor is None else mask_tensor.data_ptr(), out.data_ptr(),
+        None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), bsz, hq, hk, n_kv, d,
+        keys.stride(0), keys.stride(1), keys.stride(2), values.stride(0), values.stride(1), values.stride(2),
+        float(scale), _DTYPE_CODE[queries.dtype], torch.cuda.current_stream(queries.device).cuda_stream)
+    _native.check(rc, "dflash_sdpa_q16")
+    return out

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 5
+#define DFLASH_ABI_VERSION 6
 
 enum {
   DFLASH_OK = 0,
@@ -200,6 +200,29 @@ int dflash_gdn_prepare(const void* qkv, const void* conv_state, const void* conv
  */
 int dflash_gdn_gated_norm(const void* x, const void* z, const void* weight, void* y, long long rows,
                           int D, int dtype, int weight_dtype, float eps, void* stream);
+
+/*
+ * Exact attention of a verify block of 16 queries over a long KV cache.  Replaces the two
+ * launches of dflash_mlx/kernels.py:735-761 (`batched_sdpa_2pass_partials{,_mask}` and
+ * `batched_sdpa_2pass_reduce`): for batch b, query head hq, hk = hq / (Hq / Hk), query i < 16
+ *     out[b, hq, i, :] = softmax_n(scale * q[b, hq, i, :] . k[b, hk, n, :] + mask[b, hq, i, n]) v[b, hk, n, :]
+ * over the keys n <= N - 16 + i; with a mask, keys whose mask value is below the dtype's lowest
+ * finite value are left out as well; a query without keys gives 0.
+ *
+ *   q, out  [B, Hq, 16, D]  dtype (bf16 / fp16), contiguous;  D = 128 or 256 (= value dim)
+ *   k, v    element (b, h, n, d) at b * batch_stride + h * head_stride + n * seq_stride + d
+ *           (strides in elements, multiples of 8): a KV cache is read in place
+ *   mask    [B, Hq, 16, N] dtype, additive, or NULL
+ *   workspace  dflash_sdpa_q16_workspace_bytes(B, Hq, Hk, N, D) bytes, 16-byte aligned, contents
+ *           irrelevant (partial results of key ranges); may be NULL when that is 0
+ * Hq a multiple of Hk, at most 8 query heads per key/value head; N >= 16.
+ */
+size_t dflash_sdpa_q16_workspace_bytes(int B, int Hq, int Hk, int N, int D);
+int dflash_sdpa_q16(const void* q, const void* k, const void* v, const void* mask, void* out,
+                    void* workspace, size_t workspace_bytes, int B, int Hq, int Hk, int N, int D,
+                    long long k_batch_stride, long long k_head_stride, long long k_seq_stride,
+                    long long v_batch_stride, long long v_head_stride, long long v_seq_stride,
+                    float scale, int dtype, void* stream);
 
 /*
  * Conv-window rebuild of a GatedDeltaNet layer after a partial acceptance: output

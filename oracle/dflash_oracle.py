@@ -32,6 +32,10 @@ a re-typed formula):
   rounding points inside the GatedDeltaNet layer glue (gdn_prepare, gdn_gated_norm),
   whose operators belong to mlx / mlx-lm - their mathematics is pinned against torch
   and fp64 closed forms, the placement of single bf16 roundings is not.
+* 16-query attention - the one-softmax fp64 form against torch's
+  scaled_dot_product_attention with the block's causal mask, against the reference's
+  two kernels restated loop by loop (sdpa_q16_two_pass), and closed forms (one key,
+  equal scores, fully masked rows).
 """
 from __future__ import annotations
 
@@ -507,6 +511,86 @@ def gdn_gated_norm(x, z, weight, dtype: str = "bf16", eps: float = 1e-6):
     """Qwen3NextRMSNormGated (mlx-lm): silu(z) * rms_norm(x, weight, eps); x, z [..., Dv]."""
     y = rms_norm_rounded(x, weight, eps, dtype)
     return round_to(silu_rounded(z, dtype) * y, dtype)
+
+
+# ----------------------------------------------------------------------------
+# Exact attention of a 16-query verify block (kernels.py:442-761)
+# ----------------------------------------------------------------------------
+
+
+def _lowest(dtype: str) -> float:
+    return {"bf16": -3.3895313892515355e38, "fp16": -65504.0}[dtype]
+
+
+def sdpa_q16_exact(q, k, v, scale: float, mask=None, dtype: str = "bf16"):
+    """What the two kernels compute, in one softmax and fp64: q [B,Hq,16,D], k [B,Hk,N,D],
+    v [B,Hk,N,V], mask additive [B,Hq,16,N] or None.  Key n counts for query i iff
+    n <= N - 16 + i (kernels.py:517) and, with a mask, its mask value is not below the
+    dtype's lowest finite value (:452-454); a query without keys gives 0 (:617)."""
+    q, k, v = (np.asarray(t, dtype=np.float64) for t in (q, k, v))
+    B, Hq, M, D = q.shape
+    Hk, N = k.shape[1], k.shape[2]
+    assert M == 16 and Hq % Hk == 0
+    G = Hq // Hk
+    kk, vv = np.repeat(k, G, axis=1), np.repeat(v, G, axis=1)
+    s = scale * np.einsum("bhid,bhnd->bhin", q, kk)
+    use = np.arange(N)[None, :] <= (N - 16 + np.arange(16))[:, None]
+    use = np.broadcast_to(use, s.shape).copy()
+    if mask is not None:
+        mk = np.asarray(mask, dtype=np.float64)
+        use &= mk >= _lowest(dtype)
+        s = s + mk
+    s = np.where(use, s, -np.inf)
+    mx = np.max(s, axis=-1, keepdims=True)
+    mx = np.where(np.isfinite(mx), mx, 0.0)
+    p = np.where(use, np.exp(s - mx), 0.0)
+    den = p.sum(axis=-1, keepdims=True)
+    out = np.einsum("bhin,bhnv->bhiv", p, vv)
+    return np.where(den > 0, out / np.where(den > 0, den, 1.0), out)
+
+
+def sdpa_q16_two_pass(q, k, v, scale: float, blocks: int, mask=None, dtype: str = "bf16"):
+    """The reference's two kernels step by step (fp32): pass 1 (kernels.py:511-560) lets block
+    j walk the keys j, j + blocks, ... with a running max / sum and stores its output rounded
+    to the input dtype; pass 2 (:596-630) merges the blocks.  Pure loops: tiny inputs only."""
+    q32 = np.asarray(q, np.float32)
+    k32, v32 = np.asarray(k, np.float32), np.asarray(v, np.float32)
+    B, Hq, M, D = q32.shape
+    Hk, N, V = k32.shape[1], k32.shape[2], v32.shape[3]
+    G = Hq // Hk
+    out = np.zeros((B, Hq, M, V), np.float32)
+    low = np.float32(_lowest(dtype))
+    fmin = np.float32(np.finfo(np.float32).min)
+    for b in range(B):
+        for h in range(Hq):
+            for i in range(M):
+                qs = np.float32(scale) * q32[b, h, i]
+                part = np.zeros((blocks, V), np.float32)
+                sums = np.zeros(blocks, np.float32)
+                maxs = np.full(blocks, fmin, np.float32)
+                for j in range(blocks):
+                    o = np.zeros(V, np.float32)
+                    mx, sm = fmin, np.float32(0)
+                    for n in range(j, N, blocks):
+                        use = n <= N - M + i
+                        mv = np.float32(0)
+                        if mask is not None:
+                            mv = np.float32(mask[b, h, i, n])
+                            use = use and mv >= low
+                        if not use:
+                            continue
+                        sc = np.float32(np.dot(qs, k32[b, h // G, n])) + mv
+                        new = max(mx, sc)
+                        f, e = np.exp(np.float32(mx - new)), np.exp(np.float32(sc - new))
+                        mx, sm = new, np.float32(sm * f + e)
+                        o = o * f + e * v32[b, h // G, n]
+                    part[j], sums[j], maxs[j] = round_to(o, dtype), sm, mx
+                mx = maxs.max()
+                w = np.exp(maxs - mx)
+                den = np.float32((w * sums).sum())
+                o = (w[:, None] * part).sum(axis=0)
+                out[b, h, i] = o if den == 0 else o / den
+    return out
 
 
 # ----------------------------------------------------------------------------
