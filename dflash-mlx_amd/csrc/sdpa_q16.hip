@@ -32,6 +32,7 @@
 
 #include <cmath>
 #include <cstdlib>
+#include <type_traits>
 
 namespace dflash {
 namespace {
@@ -83,9 +84,13 @@ __device__ __forceinline__ float elem_to_f32(uint16_t h) {
   return FP16 ? f16_bits_to_f32(h) : bf16_bits_to_f32(h);
 }
 
-// One workgroup per (batch, key/value head, split); blockDim.x = 64 * max(G, 4) threads.
-template <int D, bool FP16>
+// One workgroup per (batch, key/value head, split).  Wave w serves query head w % G and the
+// columns [slice * D / CS, (slice + 1) * D / CS) of the output, slice = w / G: with few query
+// heads per key/value head the output columns are split over CS waves (each repeats the cheap
+// K Q^T) so that a SIMD has more than one wave to switch between.  blockDim.x = 64 * max(G * CS, 4).
+template <int D, bool FP16, int CS>
 __global__ __launch_bounds__(512) void sdpa_q16_kernel(SdpaArgs a) {
+  constexpr int kCols = D / 16 / CS;          // 16-column chunks of the output per wave
   constexpr int P = D + kPadElems;            // row pitch of a tile in LDS, elements
   constexpr int kTileElems = kTileKeys * P;   // one K or V tile
   constexpr int kChunks = kTileKeys * D / 8;  // 16-byte pieces of a tile
@@ -101,30 +106,37 @@ __global__ __launch_bounds__(512) void sdpa_q16_kernel(SdpaArgs a) {
   const int n_begin = split * a.keys_per_split;
   const int n_end = n_begin + a.keys_per_split < a.N ? n_begin + a.keys_per_split : a.N;
   const int j = lane & 15, kb = lane >> 4;
-  const bool computes = wave < a.G;
-  const int hq = hk * a.G + (computes ? wave : 0);
+  const bool computes = wave < a.G * CS;
+  const int slice = computes ? wave / a.G : 0;
+  const int hq = hk * a.G + (computes ? wave % a.G : 0);
   const size_t qrow = ((size_t)b * a.Hq + hq) * 16 + j;  // this lane's query
 
   const uint16_t* kbase = a.k + (size_t)b * a.k_batch_stride + (size_t)hk * a.k_head_stride;
   const uint16_t* vbase = a.v + (size_t)b * a.v_batch_stride + (size_t)hk * a.v_head_stride;
 
-  // ---- tile movement: global -> registers (in flight during the arithmetic) -> LDS ------------
-  uint4 kr[kLoads], vr[kLoads];
-  auto fetch = [&](int n0) __attribute__((always_inline)) {
+  // ---- tile movement: global -> registers -> LDS.  Two register stages: the loads of tile i + 2
+  // are issued before the arithmetic of tile i, and tile i + 1 goes from its registers to LDS
+  // after it, a full tile after its loads were issued. -----------------------------------------
+  uint4 kr[2][kLoads], vr[2][kLoads];
+  using Stage0 = std::integral_constant<int, 0>;
+  using Stage1 = std::integral_constant<int, 1>;
+  auto fetch = [&](auto stage, int n0) __attribute__((always_inline)) {
+    constexpr int S = decltype(stage)::value;
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
       const int c = tid + i * threads;
       const int key = c / (D / 8), piece = c % (D / 8);
       const int n = n0 + key;
-      kr[i] = uint4{0u, 0u, 0u, 0u};
-      vr[i] = uint4{0u, 0u, 0u, 0u};
+      kr[S][i] = uint4{0u, 0u, 0u, 0u};
+      vr[S][i] = uint4{0u, 0u, 0u, 0u};
       if (c < kChunks && n < n_end) {
-        kr[i] = *reinterpret_cast<const uint4*>(kbase + (size_t)n * a.k_seq_stride + 8 * piece);
-        vr[i] = *reinterpret_cast<const uint4*>(vbase + (size_t)n * a.v_seq_stride + 8 * piece);
+        kr[S][i] = *reinterpret_cast<const uint4*>(kbase + (size_t)n * a.k_seq_stride + 8 * piece);
+        vr[S][i] = *reinterpret_cast<const uint4*>(vbase + (size_t)n * a.v_seq_stride + 8 * piece);
       }
     }
   };
-  auto stash = [&](int buf) __attribute__((always_inline)) {
+  auto stash = [&](auto stage, int buf) __attribute__((always_inline)) {
+    constexpr int S = decltype(stage)::value;
     uint16_t* sk = lds + buf * 2 * kTileElems;
     uint16_t* sv = sk + kTileElems;
 #pragma unroll
@@ -132,13 +144,14 @@ __global__ __launch_bounds__(512) void sdpa_q16_kernel(SdpaArgs a) {
       const int c = tid + i * threads;
       if (c < kChunks) {
         const int key = c / (D / 8), piece = c % (D / 8);
-        *reinterpret_cast<uint4*>(sk + key * P + 8 * piece) = kr[i];
-        *reinterpret_cast<uint4*>(sv + key * P + 8 * piece) = vr[i];
+        *reinterpret_cast<uint4*>(sk + key * P + 8 * piece) = kr[S][i];
+        *reinterpret_cast<uint4*>(sv + key * P + 8 * piece) = vr[S][i];
       }
     }
   };
 
-  fetch(n_begin);
+  fetch(Stage0{}, n_begin);
+  fetch(Stage1{}, n_begin + kTileKeys);
 
   // ---- this wave's queries, as the B operand of K Q^T -----------------------------------------
   uint4 qreg[D / 32];
@@ -146,19 +159,12 @@ __global__ __launch_bounds__(512) void sdpa_q16_kernel(SdpaArgs a) {
   for (int s = 0; s < D / 32; ++s)
     qreg[s] = computes ? *reinterpret_cast<const uint4*>(a.q + qrow * D + 32 * s + 8 * kb) : uint4{0u, 0u, 0u, 0u};
 
-  f32x4_t O[D / 16];
+  f32x4_t O[kCols];
 #pragma unroll
-  for (int c = 0; c < D / 16; ++c) O[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int c = 0; c < kCols; ++c) O[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m_run = kMasked, l_run = 0.f;  // l_run: this lane's keys only, merged at the end
 
-  stash(0);
-  __syncthreads();
-
-  int buf = 0;
-  for (int n0 = n_begin; n0 < n_end; n0 += kTileKeys) {
-    const bool more = n0 + kTileKeys < n_end;
-    if (more) fetch(n0 + kTileKeys);
-
+  auto compute_tile = [&](int buf, int n0) __attribute__((always_inline)) {
     if (computes) {
       const uint16_t* sk = lds + buf * 2 * kTileElems;
       const uint16_t* sv = sk + kTileElems;
@@ -207,82 +213,115 @@ __global__ __launch_bounds__(512) void sdpa_q16_kernel(SdpaArgs a) {
       m_run = m_new;
       if (__any(factor != 1.f)) {
 #pragma unroll
-        for (int c = 0; c < D / 16; ++c) O[c] *= factor;
+        for (int c = 0; c < kCols; ++c) O[c] *= factor;
       }
       const uint4 pb = {pack2<FP16>(p[0], p[1]), pack2<FP16>(p[2], p[3]), pack2<FP16>(p[4], p[5]),
                         pack2<FP16>(p[6], p[7])};
       // O^T += V^T P^T, 16 columns of V at a time
       const int src = lane & 15;  // source lane inside the group of 16: key 4 kb + src / 4, columns 4 (src % 4) ..+3
-      const uint16_t* vrow = sv + (4 * kb + (src >> 2)) * P + 4 * (src & 3);
+      const uint16_t* vrow = sv + (4 * kb + (src >> 2)) * P + 4 * (src & 3) + 16 * kCols * slice;
 #pragma unroll
-      for (int c = 0; c < D / 16; ++c) {
+      for (int c = 0; c < kCols; ++c) {
         typedef __attribute__((address_space(3))) s16x4_t lds_s16x4;
         const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vrow + 16 * c));
         const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vrow + 16 * P + 16 * c));
-        uint4 vf;
-        vf.x = (uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
-        vf.y = (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
-        vf.z = (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
-        vf.w = (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
-        O[c] = mfma32<FP16>(vf, pb, O[c]);
+        const uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
+        O[c] = mfma32<FP16>(uint4{lo2.x, lo2.y, hi2.x, hi2.y}, pb, O[c]);
       }
     }
 
-    if (more) stash(buf ^ 1);
+  };
+
+  stash(Stage0{}, 0);
+  __syncthreads();
+  for (int n0 = n_begin; n0 < n_end; n0 += 2 * kTileKeys) {
+    // even tile in buffer 0; stage 1 holds the next tile, stage 0 is free
+    if (n0 + 2 * kTileKeys < n_end) fetch(Stage0{}, n0 + 2 * kTileKeys);
+    compute_tile(0, n0);
+    if (n0 + kTileKeys < n_end) stash(Stage1{}, 1);
     __syncthreads();
-    buf ^= 1;
+    if (n0 + kTileKeys >= n_end) break;
+    // odd tile in buffer 1; stage 0 holds the next tile, stage 1 is free
+    if (n0 + 3 * kTileKeys < n_end) fetch(Stage1{}, n0 + 3 * kTileKeys);
+    compute_tile(1, n0 + kTileKeys);
+    if (n0 + 2 * kTileKeys < n_end) stash(Stage0{}, 0);
+    __syncthreads();
   }
 
   if (!computes) return;
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
-  // accumulator r of chunk c is column 16 c + 4 kb + r of query j
+  // accumulator r of chunk c is column 16 (kCols slice + c) + 4 kb + r of query j
+  const int col0 = 16 * kCols * slice + 4 * kb;
   if (a.splits == 1) {
     const float inv = l_run > 0.f ? 1.f / l_run : 1.f;
 #pragma unroll
-    for (int c = 0; c < D / 16; ++c) {
+    for (int c = 0; c < kCols; ++c) {
       const uint2 o = {pack2<FP16>(O[c][0] * inv, O[c][1] * inv), pack2<FP16>(O[c][2] * inv, O[c][3] * inv)};
-      *reinterpret_cast<uint2*>(a.out + qrow * D + 16 * c + 4 * kb) = o;
+      *reinterpret_cast<uint2*>(a.out + qrow * D + col0 + 16 * c) = o;
     }
   } else {
     const size_t prow = (size_t)split * a.B * a.Hq * 16 + qrow;
 #pragma unroll
-    for (int c = 0; c < D / 16; ++c) *reinterpret_cast<f32x4_t*>(a.part_o + prow * D + 16 * c + 4 * kb) = O[c];
-    if (kb == 0) *reinterpret_cast<f32x2_t*>(a.part_ml + prow * 2) = f32x2_t{m_run, l_run};
+    for (int c = 0; c < kCols; ++c) *reinterpret_cast<f32x4_t*>(a.part_o + prow * D + col0 + 16 * c) = O[c];
+    if (kb == 0 && slice == 0) *reinterpret_cast<f32x2_t*>(a.part_ml + prow * 2) = f32x2_t{m_run, l_run};
   }
 }
 
-// Second pass: one workgroup per query row, a thread per 4 output columns.
+// Second pass: one workgroup of 256 threads per query row.  Thread (g, c) adds the partial
+// outputs of the splits s = g, g + 4, ... for 4 output columns; the weights exp(m_s - m) and the
+// total sum are worked out once, by the first wave.
+constexpr int kMaxSplits = 256;
 template <bool FP16>
-__global__ __launch_bounds__(64) void sdpa_q16_merge_kernel(SdpaArgs a, int D) {
+__global__ __launch_bounds__(256) void sdpa_q16_merge_kernel(SdpaArgs a, int D) {
+  __shared__ float weight[kMaxSplits];
+  __shared__ float total;
+  __shared__ f32x4_t acc[4][64];
   const size_t row = blockIdx.x;  // (b * Hq + hq) * 16 + i
   const size_t rows = (size_t)a.B * a.Hq * 16;
-  const int c4 = threadIdx.x;
-  if (4 * c4 >= D) return;
-  float m = kMasked;
-  for (int s = 0; s < a.splits; ++s) m = fmaxf(m, a.part_ml[((size_t)s * rows + row) * 2]);
-  float l = 0.f;
-  f32x4_t o = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < a.splits; ++s) {
-    const size_t prow = (size_t)s * rows + row;
-    const float w = __expf(a.part_ml[prow * 2] - m);
-    l += w * a.part_ml[prow * 2 + 1];
-    o += *reinterpret_cast<const f32x4_t*>(a.part_o + prow * D + 4 * c4) * w;
+  const int tid = threadIdx.x, c4 = tid & 63, g = tid >> 6;
+  if (tid < 64) {
+    float m = kMasked;
+    for (int s = tid; s < a.splits; s += 64) m = fmaxf(m, a.part_ml[((size_t)s * rows + row) * 2]);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    float l = 0.f;
+    for (int s = tid; s < a.splits; s += 64) {
+      const f32x2_t ml = *reinterpret_cast<const f32x2_t*>(a.part_ml + ((size_t)s * rows + row) * 2);
+      const float w = __expf(ml[0] - m);
+      weight[s] = w;
+      l += w * ml[1];
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) l += __shfl_xor(l, off, 64);
+    if (tid == 0) total = l;
   }
-  const float inv = l > 0.f ? 1.f / l : 1.f;
-  const uint2 packed = {pack2<FP16>(o[0] * inv, o[1] * inv), pack2<FP16>(o[2] * inv, o[3] * inv)};
-  *reinterpret_cast<uint2*>(a.out + row * D + 4 * c4) = packed;
+  __syncthreads();
+  f32x4_t o = {0.f, 0.f, 0.f, 0.f};
+  if (4 * c4 < D) {
+    for (int s = g; s < a.splits; s += 4)
+      o += *reinterpret_cast<const f32x4_t*>(a.part_o + ((size_t)s * rows + row) * D + 4 * c4) * weight[s];
+  }
+  acc[g][c4] = o;
+  __syncthreads();
+  if (g == 0 && 4 * c4 < D) {
+    o = acc[0][c4] + acc[1][c4] + acc[2][c4] + acc[3][c4];
+    const float inv = total > 0.f ? 1.f / total : 1.f;
+    const uint2 packed = {pack2<FP16>(o[0] * inv, o[1] * inv), pack2<FP16>(o[2] * inv, o[3] * inv)};
+    *reinterpret_cast<uint2*>(a.out + row * D + 4 * c4) = packed;
+  }
 }
 
 int pick_splits(int B, int Hk, int N, int* keys_per_split) {
-  // About 128 workgroups in flight, and never less than 128 keys per split: every split adds
-  // B * Hq * 16 * (D + 2) * 4 bytes of partial results, written once and read once.
+  // About one workgroup per compute unit, and never less than 128 keys per split: every split
+  // adds B * Hq * 16 * (D + 2) * 4 bytes of partial results, written once and read once.
   // DFLASH_SDPA_SPLITS=n asks for n ranges instead (read per call: experiments and tests)
   const char* env = getenv("DFLASH_SDPA_SPLITS");
   const int forced = env ? atoi(env) : 0;
-  int want = forced > 0 ? forced : (128 + B * Hk - 1) / (B * Hk);
+  int want = forced > 0 ? forced : (256 + B * Hk - 1) / (B * Hk);
   const int most = (N + 127) / 128;
   if (want > most) want = most;
+  if (want > kMaxSplits) want = kMaxSplits;
   if (want < 1) want = 1;
   int per = (N + want - 1) / want;
   per = (per + kTileKeys - 1) / kTileKeys * kTileKeys;
@@ -345,14 +384,24 @@ extern "C" int dflash_sdpa_q16(const void* q, const void* k, const void* v, cons
   }
 
   hipStream_t s = (hipStream_t)stream;
-  const int waves = a.G < 4 ? 4 : a.G;
+  // column split: as many waves as fit eight, in powers of two
+  const int cs = a.G <= 2 ? 4 : a.G <= 4 ? 2 : 1;
+  const int waves = a.G * cs < 4 ? 4 : a.G * cs;
   const size_t lds_bytes = (size_t)2 * 2 * kTileKeys * (D + kPadElems) * sizeof(uint16_t);
-  const void* fn = D == 256 ? (dtype == DFLASH_FP16 ? (const void*)sdpa_q16_kernel<256, true>
-                                                    : (const void*)sdpa_q16_kernel<256, false>)
-                            : (dtype == DFLASH_FP16 ? (const void*)sdpa_q16_kernel<128, true>
-                                                    : (const void*)sdpa_q16_kernel<128, false>);
-  static bool attr_set[4] = {};
-  const int idx = (D == 256 ? 2 : 0) + (dtype == DFLASH_FP16 ? 1 : 0);
+  const bool f16 = dtype == DFLASH_FP16;
+  const void* table[2][2][3] = {
+      {{(const void*)sdpa_q16_kernel<128, false, 1>, (const void*)sdpa_q16_kernel<128, false, 2>,
+        (const void*)sdpa_q16_kernel<128, false, 4>},
+       {(const void*)sdpa_q16_kernel<128, true, 1>, (const void*)sdpa_q16_kernel<128, true, 2>,
+        (const void*)sdpa_q16_kernel<128, true, 4>}},
+      {{(const void*)sdpa_q16_kernel<256, false, 1>, (const void*)sdpa_q16_kernel<256, false, 2>,
+        (const void*)sdpa_q16_kernel<256, false, 4>},
+       {(const void*)sdpa_q16_kernel<256, true, 1>, (const void*)sdpa_q16_kernel<256, true, 2>,
+        (const void*)sdpa_q16_kernel<256, true, 4>}}};
+  const int ics = cs == 1 ? 0 : cs == 2 ? 1 : 2;
+  const void* fn = table[D == 256][f16][ics];
+  static bool attr_set[12] = {};
+  const int idx = ((D == 256) * 2 + f16) * 3 + ics;
   if (!attr_set[idx]) {
     DFLASH_HIP_OK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
     attr_set[idx] = true;
@@ -361,9 +410,9 @@ extern "C" int dflash_sdpa_q16(const void* q, const void* k, const void* v, cons
   DFLASH_HIP_OK(hipLaunchKernel(fn, dim3((unsigned)(B * Hk * a.splits)), dim3(64 * waves), args, lds_bytes, s));
   if (a.splits > 1) {
     if (dtype == DFLASH_FP16) {
-      hipLaunchKernelGGL(sdpa_q16_merge_kernel<true>, dim3((unsigned)(B * Hq * 16)), dim3(64), 0, s, a, D);
+      hipLaunchKernelGGL(sdpa_q16_merge_kernel<true>, dim3((unsigned)(B * Hq * 16)), dim3(256), 0, s, a, D);
     } else {
-      hipLaunchKernelGGL(sdpa_q16_merge_kernel<false>, dim3((unsigned)(B * Hq * 16)), dim3(64), 0, s, a, D);
+      hipLaunchKernelGGL(sdpa_q16_merge_kernel<false>, dim3((unsigned)(B * Hq * 16)), dim3(256), 0, s, a, D);
     }
     DFLASH_HIP_OK(hipGetLastError());
   }

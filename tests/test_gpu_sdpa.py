@@ -111,3 +111,33 @@ def test_gates_and_errors(native_lib):
                                     1, 4, 2, 4096, 128, 0, 4096 * 128, 128, 0, 4096 * 128, 128, 1.0, nat.BF16, None)
     assert rc == nat.ERR_WORKSPACE if hasattr(nat, "ERR_WORKSPACE") else rc != 0
     torch.cuda.synchronize()
+
+
+def test_attention_layer_takes_the_kernel_for_a_verify_block_over_a_long_prefix(native_lib, monkeypatch):
+    """The layer hook (dflash_mlx/runtime.py:508-616) on the device: 16 new tokens over 1100 cached
+    ones go through the kernel and agree with the layer's plain causal call."""
+    from dflash_mlx_amd import attention_layer as A
+    from dflash_mlx_amd import kernels as K
+    from dflash_mlx_amd.cache import KVCache
+    from test_attention_layer import _Layer, _attn
+
+    attn = _attn(dtype=torch.bfloat16, heads=8, kv_heads=2, head_dim=128, hidden=256, seed=5).to(DEV)
+    A.configure_full_attention_split([_Layer(attn)], enabled=True)
+    original = type(attn)._dflash_original_call
+    calls = []
+    real = K.batched_sdpa_2pass_exact
+    monkeypatch.setattr(A, "batched_sdpa_2pass_exact",
+                        lambda **kw: calls.append(tuple(kw["keys"].shape)) or real(**kw))
+    gen = torch.Generator().manual_seed(1)
+    prefix = torch.randn((1, 1100, 256), generator=gen).to(torch.bfloat16).to(DEV)
+    block = torch.randn((1, 16, 256), generator=gen).to(torch.bfloat16).to(DEV)
+    outs = []
+    with torch.no_grad():
+        for call in (lambda x, c: attn(x, mask="causal", cache=c), lambda x, c: original(attn, x, mask="causal", cache=c)):
+            cache = KVCache()
+            call(prefix, cache)
+            outs.append(call(block, cache).float())
+    torch.cuda.synchronize()
+    assert calls == [(1, 2, 1116, 128)]              # the cache view, read in place; the prefill took the plain path
+    rel = float((outs[0] - outs[1]).norm() / outs[1].norm())
+    assert rel < 1e-2
