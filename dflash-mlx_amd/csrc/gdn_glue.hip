@@ -53,67 +53,110 @@ __device__ __forceinline__ float silu_rounded(float x, int dt) {
   return round_through(x * round_through(sigmoid_f32(x), dt), dt);
 }
 
-// One wave per (batch, step, head); heads 0..Hk-1 are q, Hk..2Hk-1 are k, the rest v.
-__global__ __launch_bounds__(kWavesPerGroup * 64) void gdn_prepare_kernel(PrepareArgs p) {
-  const int lane = threadIdx.x & 63;
-  const int heads = 2 * p.Hk + p.Hv;
-  const long long w = (long long)blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
-  if (w >= (long long)p.B * p.S * heads) return;
-  const int h = (int)(w % heads);
-  const int s = (int)((w / heads) % p.S);
-  const int b = (int)(w / ((long long)heads * p.S));
+// PER adjacent elements of an array of dtype dt, starting at element i (a multiple of PER):
+// 2-byte types in 64-bit accesses when PER is a multiple of 4, one 32-bit access for a pair.
+template <int PER>
+__device__ __forceinline__ void load_adjacent(const void* p, size_t i, int dt, float (&out)[PER]) {
+  if (dt == DFLASH_FP32) {
+    const float* src = (const float*)p + i;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) out[e] = src[e];
+    return;
+  }
+  uint16_t h[PER];
+  if (PER % 4 == 0) {
+#pragma unroll
+    for (int e = 0; e < PER; e += 4) {
+      const uint2 w = *reinterpret_cast<const uint2*>((const uint16_t*)p + i + e);
+      h[e] = (uint16_t)w.x, h[e + 1 < PER ? e + 1 : 0] = (uint16_t)(w.x >> 16);
+      h[e + 2 < PER ? e + 2 : 0] = (uint16_t)w.y, h[e + 3 < PER ? e + 3 : 0] = (uint16_t)(w.y >> 16);
+    }
+  } else if (PER == 2) {
+    const uint32_t w = *reinterpret_cast<const uint32_t*>((const uint16_t*)p + i);
+    h[0] = (uint16_t)w, h[PER > 1 ? 1 : 0] = (uint16_t)(w >> 16);
+  } else {
+#pragma unroll
+    for (int e = 0; e < PER; ++e) h[e] = ((const uint16_t*)p)[i + e];
+  }
+#pragma unroll
+  for (int e = 0; e < PER; ++e) out[e] = dt == DFLASH_BF16 ? bf16_bits_to_f32(h[e]) : f16_bits_to_f32(h[e]);
+}
+
+// One wave per (batch, step, head); heads 0..Hk-1 are q, Hk..2Hk-1 are k, the rest v.  A lane
+// holds PER = D / 64 adjacent channels of its head, so a row of the head is one access per lane
+// and the K taps of those channels are PER * K adjacent weights.  All loads of a wave are issued
+// before anything is computed: the kernel moves a few hundred KB and lives on latency.
+template <int PER, int K>
+__device__ __forceinline__ void prepare_head(const PrepareArgs& p, int b, int s, int h, int lane) {
   const int key_dim = p.Hk * p.Dk;
   const int C = 2 * key_dim + p.Hv * p.Dv;
-  const int keep = p.K - 1;
+  constexpr int keep = K - 1;
   const bool is_v = h >= 2 * p.Hk;
-  const int D = is_v ? p.Dv : p.Dk;
+  const int D = PER * 64;
   const int cb = is_v ? 2 * key_dim + (h - 2 * p.Hk) * p.Dv : h * p.Dk;  // q and k heads are contiguous
-  const int per_lane = D / 64;
+  const int c = cb + PER * lane;
 
-  float act[kMaxPerLane];
+  float x[K][PER], w[PER * K];
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    const int r = s + j;  // row of [conv_state | qkv]
+#pragma unroll
+    for (int e = 0; e < PER; ++e) x[j][e] = 0.f;
+    if (r < keep) {
+      if (p.conv_state) load_adjacent<PER>(p.conv_state, ((size_t)b * keep + r) * C + c, p.dt, x[j]);
+    } else if (p.mask == nullptr || p.mask[(size_t)b * p.S + (r - keep)]) {
+      load_adjacent<PER>(p.qkv, ((size_t)b * p.S + (r - keep)) * C + c, p.dt, x[j]);
+    }
+  }
+  load_adjacent<PER * K>(p.conv_w, (size_t)c * K, p.dt, w);
+  float gate_a = 0.f, gate_b = 0.f, a_log = 0.f, bias = 0.f;
+  const int hv = h - 2 * p.Hk;
+  const size_t vrow = ((size_t)b * p.S + s) * p.Hv + (is_v ? hv : 0);
+  if (is_v && lane == 0) {
+    gate_a = load_as_f32(p.a, vrow, p.dt);
+    gate_b = load_as_f32(p.b, vrow, p.dt);
+    a_log = load_as_f32(p.A_log, hv, p.param_dt);
+    bias = load_as_f32(p.dt_bias, hv, p.param_dt);
+  }
+
+  // the last `keep` rows of [conv_state | qkv] are the next conv state
+  if (s + keep >= p.S) {
+#pragma unroll
+    for (int e = 0; e < PER; ++e)
+      store_from_f32(p.conv_next, ((size_t)b * keep + (s + keep - p.S)) * C + c + e, x[K - 1][e], p.dt);
+  }
+  if (s == 0) {
+    for (int r = p.S; r < keep; ++r) {  // blocks shorter than the state: old rows move up
+      float old[PER];
+#pragma unroll
+      for (int e = 0; e < PER; ++e) old[e] = 0.f;
+      if (p.conv_state) load_adjacent<PER>(p.conv_state, ((size_t)b * keep + r) * C + c, p.dt, old);
+#pragma unroll
+      for (int e = 0; e < PER; ++e) store_from_f32(p.conv_next, ((size_t)b * keep + (r - p.S)) * C + c + e, old[e], p.dt);
+    }
+  }
+
+  float act[PER];
   float ss = 0.f;
 #pragma unroll
-  for (int i = 0; i < kMaxPerLane; ++i) {
-    act[i] = 0.f;
-    if (i >= per_lane) continue;
-    const int c = cb + lane + 64 * i;
-    float acc = 0.f, newest = 0.f;
-    for (int j = 0; j < p.K; ++j) {
-      const int r = s + j;  // row of [conv_state | qkv]
-      float x = 0.f;
-      if (r < keep) {
-        if (p.conv_state) x = load_as_f32(p.conv_state, ((size_t)b * keep + r) * C + c, p.dt);
-      } else if (p.mask == nullptr || p.mask[(size_t)b * p.S + (r - keep)]) {
-        x = load_as_f32(p.qkv, ((size_t)b * p.S + (r - keep)) * C + c, p.dt);
-      }
-      acc += x * load_as_f32(p.conv_w, (size_t)c * p.K + j, p.dt);
-      newest = x;
-    }
-    // the last `keep` rows of [conv_state | qkv] are the next conv state
-    if (s + keep >= p.S) store_from_f32(p.conv_next, ((size_t)b * keep + (s + keep - p.S)) * C + c, newest, p.dt);
-    if (s == 0) {
-      for (int r = p.S; r < keep; ++r) {  // blocks shorter than the state: old rows move up
-        const float x = p.conv_state ? load_as_f32(p.conv_state, ((size_t)b * keep + r) * C + c, p.dt) : 0.f;
-        store_from_f32(p.conv_next, ((size_t)b * keep + (r - p.S)) * C + c, x, p.dt);
-      }
-    }
-    act[i] = silu_rounded(round_through(acc, p.dt), p.dt);
-    ss += act[i] * act[i];
+  for (int e = 0; e < PER; ++e) {
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < K; ++j) acc += x[j][e] * w[e * K + j];
+    act[e] = silu_rounded(round_through(acc, p.dt), p.dt);
+    ss += act[e] * act[e];
   }
 
   if (is_v) {
-    const int hv = h - 2 * p.Hk;
-    const size_t row = ((size_t)b * p.S + s) * p.Hv + hv;
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i)
-      if (i < per_lane) store_from_f32(p.v, row * p.Dv + lane + 64 * i, act[i], p.dt);
+    for (int e = 0; e < PER; ++e) store_from_f32(p.v, vrow * p.Dv + PER * lane + e, act[e], p.dt);
     if (lane == 0) {
       // a + dt_bias and the softplus live in the promoted dtype of the two operands
       const int sum_dt = p.param_dt == DFLASH_FP32 ? DFLASH_FP32 : p.dt;
-      const float apb = round_through(load_as_f32(p.a, row, p.dt) + load_as_f32(p.dt_bias, hv, p.param_dt), sum_dt);
+      const float apb = round_through(gate_a + bias, sum_dt);
       const float sp = round_through(fmaxf(apb, 0.f) + log1pf(expf(-fabsf(apb))), sum_dt);
-      p.g[row] = expf(-expf(load_as_f32(p.A_log, hv, p.param_dt)) * sp);
-      store_from_f32(p.beta, row, sigmoid_f32(load_as_f32(p.b, row, p.dt)), p.dt);
+      p.g[vrow] = expf(-expf(a_log) * sp);
+      store_from_f32(p.beta, vrow, sigmoid_f32(gate_b), p.dt);
     }
     return;
   }
@@ -124,9 +167,25 @@ __global__ __launch_bounds__(kWavesPerGroup * 64) void gdn_prepare_kernel(Prepar
   void* out = is_q ? p.q : p.k;
   const size_t row = ((size_t)b * p.S + s) * p.Hk + (is_q ? h : h - p.Hk);
 #pragma unroll
-  for (int i = 0; i < kMaxPerLane; ++i)
-    if (i < per_lane)
-      store_from_f32(out, row * p.Dk + lane + 64 * i, scale * round_through(act[i] * inv_rms, p.dt), p.dt);
+  for (int e = 0; e < PER; ++e)
+    store_from_f32(out, row * p.Dk + PER * lane + e, scale * round_through(act[e] * inv_rms, p.dt), p.dt);
+}
+
+template <int K>
+__global__ __launch_bounds__(kWavesPerGroup * 64) void gdn_prepare_kernel(PrepareArgs p) {
+  const int lane = threadIdx.x & 63;
+  const int heads = 2 * p.Hk + p.Hv;
+  const long long w = (long long)blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
+  if (w >= (long long)p.B * p.S * heads) return;
+  const int h = (int)(w % heads);
+  const int s = (int)((w / heads) % p.S);
+  const int b = (int)(w / ((long long)heads * p.S));
+  switch ((h >= 2 * p.Hk ? p.Dv : p.Dk) / 64) {
+    case 1: prepare_head<1, K>(p, b, s, h, lane); break;
+    case 2: prepare_head<2, K>(p, b, s, h, lane); break;
+    case 3: prepare_head<3, K>(p, b, s, h, lane); break;
+    default: prepare_head<4, K>(p, b, s, h, lane); break;
+  }
 }
 
 struct NormArgs {
@@ -195,8 +254,8 @@ extern "C" int dflash_gdn_prepare(const void* qkv, const void* conv_state, const
                  DFLASH_ERR_ARG, "dflash_gdn_prepare: null operand");
   DFLASH_REQUIRE(known_dtype(dtype) && known_dtype(param_dtype), DFLASH_ERR_ARG,
                  "dflash_gdn_prepare: unknown dtype code");
-  DFLASH_REQUIRE(B >= 0 && S >= 0 && Hk > 0 && Hv > 0 && conv_kernel >= 2 && conv_kernel <= 8, DFLASH_ERR_SHAPE,
-                 "dflash_gdn_prepare: bad dimension");
+  DFLASH_REQUIRE(B >= 0 && S >= 0 && Hk > 0 && Hv > 0 && conv_kernel >= 2 && conv_kernel <= 4, DFLASH_ERR_SHAPE,
+                 "dflash_gdn_prepare: bad dimension (conv kernels of 2 to 4 taps)");
   DFLASH_REQUIRE(head_dim_ok(Dk) && head_dim_ok(Dv), DFLASH_ERR_SHAPE,
                  "dflash_gdn_prepare: head dims must be multiples of 64 up to 256, got %d and %d", Dk, Dv);
   const long long waves = (long long)B * S * (2 * Hk + Hv);
@@ -212,7 +271,14 @@ extern "C" int dflash_gdn_prepare(const void* qkv, const void* conv_state, const
   p.scale_q = as_array_scalar(inv_scale * inv_scale, dtype);
   p.scale_k = as_array_scalar(inv_scale, dtype);
   const unsigned groups = (unsigned)((waves + kWavesPerGroup - 1) / kWavesPerGroup);
-  hipLaunchKernelGGL(gdn_prepare_kernel, dim3(groups), dim3(kWavesPerGroup * 64), 0, (hipStream_t)stream, p);
+  const dim3 grid(groups), block(kWavesPerGroup * 64);
+  if (conv_kernel == 4) {
+    hipLaunchKernelGGL(gdn_prepare_kernel<4>, grid, block, 0, (hipStream_t)stream, p);
+  } else if (conv_kernel == 3) {
+    hipLaunchKernelGGL(gdn_prepare_kernel<3>, grid, block, 0, (hipStream_t)stream, p);
+  } else {
+    hipLaunchKernelGGL(gdn_prepare_kernel<2>, grid, block, 0, (hipStream_t)stream, p);
+  }
   DFLASH_HIP_OK(hipGetLastError());
   return DFLASH_OK;
 }

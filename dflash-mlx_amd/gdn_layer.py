@@ -109,7 +109,7 @@ def gdn_prepare(qkv: torch.Tensor, conv_state: Optional[torch.Tensor], conv_w: t
         raise ValueError(f"conv_dim {C} does not match 2*{Hk}*{Dk} + {Hv}*{Dv}")
     same = (conv_w.dtype == a.dtype == b.dtype == qkv.dtype and A_log.dtype == dt_bias.dtype and
             A_log.dtype in _DTYPE_CODE and (conv_state is None or conv_state.dtype == qkv.dtype))
-    if not (_kernel_covers(qkv, Dk, Dv) and same and S > 0 and 2 <= K <= 8):
+    if not (_kernel_covers(qkv, Dk, Dv) and same and S > 0 and 2 <= K <= 4):
         return gdn_prepare_ops(qkv, conv_state, conv_w, a, b, A_log, dt_bias, mask,
                                Hk=Hk, Hv=Hv, Dk=Dk, Dv=Dv, eps=eps)
     lib = _native.lib()

@@ -185,7 +185,7 @@ int dflash_gdn_forward_tape(const void* q, const void* k, const void* v, const v
  *   conv_w      [C, conv_kernel] dtype; tap j multiplies conv_input row s + j
  *   a, b        [B, S, Hv] dtype;  A_log, dt_bias [Hv] param_dtype;  mask [B, S] uint8 or NULL
  *   outputs: conv_next [B, conv_kernel-1, C], q, k [B, S, Hk, Dk], v [B, S, Hv, Dv], beta
- *   [B, S, Hv] in dtype; g [B, S, Hv] fp32.  Dk, Dv multiples of 64 up to 256.
+ *   [B, S, Hv] in dtype; g [B, S, Hv] fp32.  Dk, Dv multiples of 64 up to 256; conv_kernel 2 to 4.
  */
 int dflash_gdn_prepare(const void* qkv, const void* conv_state, const void* conv_w, const void* a,
                        const void* b, const void* A_log, const void* dt_bias, const uint8_t* mask,

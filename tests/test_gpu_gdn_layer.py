@@ -72,6 +72,17 @@ def test_prepare_head_shapes_and_fp32_parameters(native_lib, dims):
     _check(got, want, "bf16")
 
 
+@pytest.mark.parametrize("K", [2, 3])
+def test_prepare_shorter_conv_kernels(native_lib, K):
+    t, dims = _inputs(B=1, S=5, Hk=1, Hv=2, Dk=128, Dv=64, K=K, seed=80 + K)
+    want = O.gdn_prepare(**t, **dims, dtype="bf16")
+    d = _dev(t, torch.bfloat16)
+    got = G.gdn_prepare(d["qkv"], d["conv_state"], d["conv_w"], d["a"], d["b"], d["A_log"], d["dt_bias"], None, **dims)
+    torch.cuda.synchronize()
+    assert tuple(got[0].shape) == (1, K - 1, 256)
+    _check(got, want, "bf16")
+
+
 def test_prepare_takes_the_array_ops_for_other_head_sizes(native_lib):
     t, dims = _inputs(B=1, S=4, Hk=1, Hv=2, Dk=32, Dv=96, seed=60)
     want = O.gdn_prepare(**t, **dims, dtype="bf16")
