@@ -79,7 +79,7 @@ def test_prepare_shorter_conv_kernels(native_lib, K):
     d = _dev(t, torch.bfloat16)
     got = G.gdn_prepare(d["qkv"], d["conv_state"], d["conv_w"], d["a"], d["b"], d["A_log"], d["dt_bias"], None, **dims)
     torch.cuda.synchronize()
-    assert tuple(got[0].shape) == (1, K - 1, 256)
+    assert tuple(got[0].shape) == (1, K - 1, 2 * 128 + 2 * 64)
     _check(got, want, "bf16")
 
 
