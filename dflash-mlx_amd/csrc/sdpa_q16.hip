@@ -26,8 +26,8 @@
 //                 element t % 4 of source lanes t / 4, 4 + t / 4, 8 + t / 4, 12 + t / 4 - so source
 //                 lane 4 e + q points at V[key 4 kb + e][16 c + 4 q ..+3] and lane t receives
 //                 column 16 c + t of four keys.  No transposed copy of V or P is ever stored.
-// Ranges of keys (splits) write fp32 partial outputs with their max and sum; a second kernel
-// merges them (the reference's second pass).
+// Ranges of keys (splits) write partial outputs in the input dtype (kernels.py:556-558) with their
+// fp32 max and sum; a second kernel merges them (the reference's second pass).
 #include "dflash_common.h"
 
 #include <cmath>
@@ -54,7 +54,7 @@ struct SdpaArgs {
   const uint16_t* v;
   const uint16_t* mask;  // [B, Hq, 16, N] additive, in the input dtype, or null
   uint16_t* out;         // [B, Hq, 16, D]
-  float* part_o;         // [splits, B * Hq, 16, D]
+  uint16_t* part_o;      // [splits, B * Hq, 16, D] in the input dtype, as the reference keeps them
   float* part_ml;        // [splits, B * Hq, 16, 2]  (max, sum)
   long long k_batch_stride, k_head_stride, k_seq_stride;
   long long v_batch_stride, v_head_stride, v_seq_stride;
@@ -88,7 +88,7 @@ __device__ __forceinline__ float elem_to_f32(uint16_t h) {
 // columns [slice * D / CS, (slice + 1) * D / CS) of the output, slice = w / G: with few query
 // heads per key/value head the output columns are split over CS waves (each repeats the cheap
 // K Q^T) so that a SIMD has more than one wave to switch between.  blockDim.x = 64 * max(G * CS, 4).
-template <int D, bool FP16, int CS>
+template <int D, bool FP16, int CS, bool MASK>
 __global__ __launch_bounds__(512) void sdpa_q16_kernel(SdpaArgs a) {
   constexpr int kCols = D / 16 / CS;          // 16-column chunks of the output per wave
   constexpr int P = D + kPadElems;            // row pitch of a tile in LDS, elements
@@ -169,15 +169,17 @@ __global__ __launch_bounds__(512) void sdpa_q16_kernel(SdpaArgs a) {
       const uint16_t* sk = lds + buf * 2 * kTileElems;
       const uint16_t* sv = sk + kTileElems;
       // S^T = K Q^T for the two 16-key halves of the tile
+      // (all reads of the tile are issued before the first product: one LDS latency, not sixteen)
+      uint4 kf[2][D / 32];
+#pragma unroll
+      for (int s = 0; s < D / 32; ++s)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) kf[t][s] = *reinterpret_cast<const uint4*>(sk + (16 * t + j) * P + 32 * s + 8 * kb);
       f32x4_t st[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-      for (int s = 0; s < D / 32; ++s) {
+      for (int s = 0; s < D / 32; ++s)
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          const uint4 kf = *reinterpret_cast<const uint4*>(sk + (16 * t + j) * P + 32 * s + 8 * kb);
-          st[t] = mfma32<FP16>(kf, qreg[s], st[t]);
-        }
-      }
+        for (int t = 0; t < 2; ++t) st[t] = mfma32<FP16>(kf[t][s], qreg[s], st[t]);
       // scores of query j for keys n0 + 16 t + 4 kb + r
       float x[8];
       bool use[8];
@@ -189,7 +191,7 @@ __global__ __launch_bounds__(512) void sdpa_q16_kernel(SdpaArgs a) {
           const int n = n0 + 16 * t + 4 * kb + r;
           bool ok = n < n_end && n <= a.N - 16 + j;
           float s = st[t][r] * a.scale;
-          if (a.mask != nullptr && ok) {
+          if (MASK && ok) {
             const float mv = elem_to_f32<FP16>(a.mask[qrow * a.N + n]);
             ok = mv >= a.lowest;
             s += mv;
@@ -220,12 +222,16 @@ __global__ __launch_bounds__(512) void sdpa_q16_kernel(SdpaArgs a) {
       // O^T += V^T P^T, 16 columns of V at a time
       const int src = lane & 15;  // source lane inside the group of 16: key 4 kb + src / 4, columns 4 (src % 4) ..+3
       const uint16_t* vrow = sv + (4 * kb + (src >> 2)) * P + 4 * (src & 3) + 16 * kCols * slice;
+      typedef __attribute__((address_space(3))) s16x4_t lds_s16x4;
+      s16x4_t lo[kCols], hi[kCols];
 #pragma unroll
       for (int c = 0; c < kCols; ++c) {
-        typedef __attribute__((address_space(3))) s16x4_t lds_s16x4;
-        const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vrow + 16 * c));
-        const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vrow + 16 * P + 16 * c));
-        const uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
+        lo[c] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vrow + 16 * c));
+        hi[c] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vrow + 16 * P + 16 * c));
+      }
+#pragma unroll
+      for (int c = 0; c < kCols; ++c) {
+        const uint2 lo2 = __builtin_bit_cast(uint2, lo[c]), hi2 = __builtin_bit_cast(uint2, hi[c]);
         O[c] = mfma32<FP16>(uint4{lo2.x, lo2.y, hi2.x, hi2.y}, pb, O[c]);
       }
     }
@@ -263,7 +269,9 @@ __global__ __launch_bounds__(512) void sdpa_q16_kernel(SdpaArgs a) {
   } else {
     const size_t prow = (size_t)split * a.B * a.Hq * 16 + qrow;
 #pragma unroll
-    for (int c = 0; c < kCols; ++c) *reinterpret_cast<f32x4_t*>(a.part_o + prow * D + col0 + 16 * c) = O[c];
+    for (int c = 0; c < kCols; ++c)
+      *reinterpret_cast<uint2*>(a.part_o + prow * D + col0 + 16 * c) =
+          uint2{pack2<FP16>(O[c][0], O[c][1]), pack2<FP16>(O[c][2], O[c][3])};
     if (kb == 0 && slice == 0) *reinterpret_cast<f32x2_t*>(a.part_ml + prow * 2) = f32x2_t{m_run, l_run};
   }
 }
@@ -300,7 +308,12 @@ __global__ __launch_bounds__(256) void sdpa_q16_merge_kernel(SdpaArgs a, int D) 
   f32x4_t o = {0.f, 0.f, 0.f, 0.f};
   if (4 * c4 < D) {
     for (int s = g; s < a.splits; s += 4)
-      o += *reinterpret_cast<const f32x4_t*>(a.part_o + ((size_t)s * rows + row) * D + 4 * c4) * weight[s];
+    {
+      const uint2 h = *reinterpret_cast<const uint2*>(a.part_o + ((size_t)s * rows + row) * D + 4 * c4);
+      const f32x4_t v = {elem_to_f32<FP16>((uint16_t)h.x), elem_to_f32<FP16>((uint16_t)(h.x >> 16)),
+                         elem_to_f32<FP16>((uint16_t)h.y), elem_to_f32<FP16>((uint16_t)(h.y >> 16))};
+      o += v * weight[s];
+    }
   }
   acc[g][c4] = o;
   __syncthreads();
@@ -314,7 +327,7 @@ __global__ __launch_bounds__(256) void sdpa_q16_merge_kernel(SdpaArgs a, int D) 
 
 int pick_splits(int B, int Hk, int N, int* keys_per_split) {
   // About one workgroup per compute unit, and never less than 128 keys per split: every split
-  // adds B * Hq * 16 * (D + 2) * 4 bytes of partial results, written once and read once.
+  // adds B * Hq * 16 * (2 D + 8) bytes of partial results, written once and read once.
   // DFLASH_SDPA_SPLITS=n asks for n ranges instead (read per call: experiments and tests)
   const char* env = getenv("DFLASH_SDPA_SPLITS");
   const int forced = env ? atoi(env) : 0;
@@ -338,7 +351,7 @@ extern "C" size_t dflash_sdpa_q16_workspace_bytes(int B, int Hq, int Hk, int N, 
   int per = 0;
   const int splits = pick_splits(B, Hk, N, &per);
   if (splits == 1) return 0;
-  return (size_t)splits * B * Hq * 16 * (D + 2) * sizeof(float);
+  return (size_t)splits * B * Hq * 16 * (D * sizeof(uint16_t) + 2 * sizeof(float));
 }
 
 extern "C" int dflash_sdpa_q16(const void* q, const void* k, const void* v, const void* mask, void* out,
@@ -375,12 +388,12 @@ extern "C" int dflash_sdpa_q16(const void* q, const void* k, const void* v, cons
   a.part_o = nullptr;
   a.part_ml = nullptr;
   if (a.splits > 1) {
-    const size_t need = (size_t)a.splits * B * Hq * 16 * (D + 2) * sizeof(float);
+    const size_t need = (size_t)a.splits * B * Hq * 16 * (D * sizeof(uint16_t) + 2 * sizeof(float));
     DFLASH_REQUIRE(workspace && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0, DFLASH_ERR_WORKSPACE,
                    "dflash_sdpa_q16: workspace of %zu bytes needed, %zu given", need,
                    workspace ? workspace_bytes : (size_t)0);
-    a.part_o = (float*)workspace;
-    a.part_ml = a.part_o + (size_t)a.splits * B * Hq * 16 * D;
+    a.part_ml = (float*)workspace;   // [splits, rows, 2] fp32 first: keeps both arrays 16-byte aligned
+    a.part_o = (uint16_t*)(a.part_ml + (size_t)a.splits * B * Hq * 16 * 2);
   }
 
   hipStream_t s = (hipStream_t)stream;
@@ -389,19 +402,20 @@ extern "C" int dflash_sdpa_q16(const void* q, const void* k, const void* v, cons
   const int waves = a.G * cs < 4 ? 4 : a.G * cs;
   const size_t lds_bytes = (size_t)2 * 2 * kTileKeys * (D + kPadElems) * sizeof(uint16_t);
   const bool f16 = dtype == DFLASH_FP16;
-  const void* table[2][2][3] = {
-      {{(const void*)sdpa_q16_kernel<128, false, 1>, (const void*)sdpa_q16_kernel<128, false, 2>,
-        (const void*)sdpa_q16_kernel<128, false, 4>},
-       {(const void*)sdpa_q16_kernel<128, true, 1>, (const void*)sdpa_q16_kernel<128, true, 2>,
-        (const void*)sdpa_q16_kernel<128, true, 4>}},
-      {{(const void*)sdpa_q16_kernel<256, false, 1>, (const void*)sdpa_q16_kernel<256, false, 2>,
-        (const void*)sdpa_q16_kernel<256, false, 4>},
-       {(const void*)sdpa_q16_kernel<256, true, 1>, (const void*)sdpa_q16_kernel<256, true, 2>,
-        (const void*)sdpa_q16_kernel<256, true, 4>}}};
+#define DFLASH_SDPA_ROW(D_, F_, M_)                                                                      \
+  {(const void*)sdpa_q16_kernel<D_, F_, 1, M_>, (const void*)sdpa_q16_kernel<D_, F_, 2, M_>, \
+   (const void*)sdpa_q16_kernel<D_, F_, 4, M_>}
+  const void* table[2][2][2][3] = {
+      {{DFLASH_SDPA_ROW(128, false, false), DFLASH_SDPA_ROW(128, false, true)},
+       {DFLASH_SDPA_ROW(128, true, false), DFLASH_SDPA_ROW(128, true, true)}},
+      {{DFLASH_SDPA_ROW(256, false, false), DFLASH_SDPA_ROW(256, false, true)},
+       {DFLASH_SDPA_ROW(256, true, false), DFLASH_SDPA_ROW(256, true, true)}}};
+#undef DFLASH_SDPA_ROW
+  const bool masked = mask != nullptr;
   const int ics = cs == 1 ? 0 : cs == 2 ? 1 : 2;
-  const void* fn = table[D == 256][f16][ics];
-  static bool attr_set[12] = {};
-  const int idx = ((D == 256) * 2 + f16) * 3 + ics;
+  const void* fn = table[D == 256][f16][masked][ics];
+  static bool attr_set[24] = {};
+  const int idx = (((D == 256) * 2 + f16) * 2 + masked) * 3 + ics;
   if (!attr_set[idx]) {
     DFLASH_HIP_OK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
     attr_set[idx] = true;
