@@ -544,7 +544,16 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
   for (int t2 = 0; t2 < 2; ++t2) {
     const int row0 = 32 * wave + 16 * t2 + 4 * kq;
     *reinterpret_cast<f32x4_t*>(sD + li * 128 + row0) = D[t2];
-    if (li < T) *reinterpret_cast<f32x4_t*>(a.tape + obase + row0) = D[t2];
+  }
+  {
+    // the tape leaves from LDS in full 128-byte lines: lane (t, q) stores this wave's rows
+    // 32 wave + 8 q ..+7 of step t (the matrix-core layout would give 64-byte pieces)
+    const int t = lane >> 2, dv0 = 32 * wave + 8 * (lane & 3);
+    if (t < T) {
+      float* dst = a.tape + ((slotT + t) * a.Hv + hv) * 128 + dv0;
+      *reinterpret_cast<f32x4_t*>(dst) = *reinterpret_cast<const f32x4_t*>(sD + t * 128 + dv0);
+      *reinterpret_cast<f32x4_t*>(dst + 4) = *reinterpret_cast<const f32x4_t*>(sD + t * 128 + dv0 + 4);
+    }
   }
   __syncthreads();
 
