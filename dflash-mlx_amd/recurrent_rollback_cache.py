@@ -17,12 +17,12 @@ launch whose accepted length may live on the device.
 """
 from __future__ import annotations
 
-from typing import Any, List, Optional, Sequence, Union
+from typing import Any, List, Optional, Union
 
 import torch
 
 from . import _native
-from .kernels import _DTYPE_CODE, _tape_replay_ops, replay_launch, tape_replay_kernel
+from .kernels import replay_launch, tape_replay_kernel
 
 
 def conv_state_rebuild(conv_prev: Optional[torch.Tensor], qkv: torch.Tensor,

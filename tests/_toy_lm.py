@@ -5,7 +5,6 @@ import torch
 import torch.nn as nn
 
 from dflash_mlx_amd import gdn_layer as G
-from dflash_mlx_amd.cache import KVCache
 from dflash_mlx_amd.quantized import QuantizedLinear
 
 
@@ -24,29 +23,18 @@ class RMSNorm(nn.Module):
         return G.rms_norm_ops(x, self.weight, 1e-6)
 
 
-class Attention(nn.Module):
-    def __init__(self, hidden, heads, head_dim, gen, dtype):
-        super().__init__()
-        self.heads, self.head_dim = heads, head_dim
-        self.q_proj = _qlinear(hidden, heads * head_dim, gen, dtype)
-        self.k_proj = _qlinear(hidden, heads * head_dim, gen, dtype)
-        self.v_proj = _qlinear(hidden, heads * head_dim, gen, dtype)
-        self.o_proj = _qlinear(heads * head_dim, hidden, gen, dtype)
+def _attention(hidden, heads, kv_heads, head_dim, gen, dtype):
+    """The package's gated attention layer over 4-bit projections."""
+    from dflash_mlx_amd.attention_layer import GatedAttention
 
-    def forward(self, x, mask=None, cache=None):
-        B, S, _ = x.shape
-        split = lambda t: t.reshape(B, S, self.heads, self.head_dim).transpose(1, 2)
-        q, k, v = split(self.q_proj(x)), split(self.k_proj(x)), split(self.v_proj(x))
-        past = cache.offset if cache is not None else 0
-        if cache is not None:
-            k, v = cache.update_and_fetch(k, v)
-        T = k.shape[2]
-        pos_q = torch.arange(past, past + S, device=x.device)[:, None]
-        allowed = torch.arange(T, device=x.device)[None, :] <= pos_q
-        scores = (q.float() @ k.float().transpose(-1, -2)) * self.head_dim ** -0.5
-        scores = scores.masked_fill(~allowed, float("-inf"))
-        out = (torch.softmax(scores, dim=-1) @ v.float()).to(x.dtype)
-        return self.o_proj(out.transpose(1, 2).reshape(B, S, -1))
+    attn = GatedAttention(num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=head_dim,
+                          q_proj=_qlinear(hidden, 2 * heads * head_dim, gen, dtype),
+                          k_proj=_qlinear(hidden, kv_heads * head_dim, gen, dtype),
+                          v_proj=_qlinear(hidden, kv_heads * head_dim, gen, dtype),
+                          o_proj=_qlinear(heads * head_dim, hidden, gen, dtype), dtype=dtype)
+    attn.q_norm.weight.data = (1 + 0.1 * torch.randn(head_dim, generator=gen)).to(dtype)
+    attn.k_norm.weight.data = (1 + 0.1 * torch.randn(head_dim, generator=gen)).to(dtype)
+    return attn
 
 
 class MLP(nn.Module):
@@ -78,12 +66,15 @@ class Block(nn.Module):
             la.A_log.data = torch.log(torch.rand(Hv, generator=gen) * 2 + 0.2).to(dtype)
             la.dt_bias.data = (torch.randn(Hv, generator=gen) * 0.3).to(dtype)
         else:
-            self.self_attn = Attention(hidden, Hv, D, gen, dtype)
+            self.self_attn = _attention(hidden, Hv, max(1, Hv // 2), D, gen, dtype)
         self.mlp = MLP(hidden, 2 * hidden, gen, dtype)
 
     def forward(self, x, cache):
-        mixer = self.linear_attn if self.is_linear else self.self_attn
-        x = x + mixer(self.input_layernorm(x), mask=None, cache=cache).to(x.dtype)
+        if self.is_linear:
+            mixed = self.linear_attn(self.input_layernorm(x), mask=None, cache=cache)
+        else:
+            mixed = self.self_attn(self.input_layernorm(x), mask="causal", cache=cache)
+        x = x + mixed.to(x.dtype)
         return x + self.mlp(self.post_attention_layernorm(x))
 
 
@@ -117,11 +108,20 @@ class ToyHybridLM(nn.Module):
             x = layer(x, c)
         return self.lm_head(self.norm(x)).float()
 
-    def install_hooks(self):
+    def install_hooks(self, *, exact_attention_over=None):
+        """The reference's per-layer hooks (dflash_mlx/runtime.py:620-652); the exact attention
+        path starts at ``exact_attention_over`` cached positions (1024 if None)."""
+        from dflash_mlx_amd.attention_layer import configure_full_attention_split
+
         for layer in self.layers:
             if layer.is_linear:
                 G._install_exact_small_proj_hooks(layer.linear_attn)
                 G._install_speculative_linear_cache_hook(layer.linear_attn)
+        configure_full_attention_split(self.layers, enabled=True)
+        if exact_attention_over is not None:
+            for layer in self.layers:
+                if not layer.is_linear:
+                    layer.self_attn._dflash_split_sdpa_exact_kv_threshold = int(exact_attention_over)
         return self
 
 

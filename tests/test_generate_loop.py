@@ -44,6 +44,9 @@ def test_checkpoint_round_trip(tmp_path):
             for n in ("A_log", "dt_bias"):
                 getattr(b.linear_attn, n).data = getattr(a.linear_attn, n).data
             b.linear_attn.conv1d.weight.data = a.linear_attn.conv1d.weight.data
+        else:
+            b.self_attn.q_norm.weight.data = a.self_attn.q_norm.weight.data
+            b.self_attn.k_norm.weight.data = a.self_attn.k_norm.weight.data
     ids = torch.randint(0, 384, (1, 9))
     cache = lambda m: make_target_cache(m.pattern)
     assert torch.equal(model(ids, cache(model)), blank(ids, cache(blank)))
@@ -68,8 +71,10 @@ def test_loader_rejects_malformed_triples(tmp_path):
 
 
 @pytest.mark.parametrize("kind", ["perfect", "random", "partly"])
-def test_speculative_cycle_commits_the_targets_greedy_tokens(kind):
-    model = ToyHybridLM(seed=3).install_hooks()
+@pytest.mark.parametrize("exact_attention_over", [None, 4])
+def test_speculative_cycle_commits_the_targets_greedy_tokens(kind, exact_attention_over):
+    # exact_attention_over = 4: the attention layers take their query-by-query path in every verify block
+    model = ToyHybridLM(seed=3).install_hooks(exact_attention_over=exact_attention_over)
     target = lambda ids, cache: model(ids, cache)
     prompt = torch.randint(0, 384, (11,), generator=torch.Generator().manual_seed(5))
     n_new = 45

@@ -83,3 +83,27 @@ def test_speculative_decoding_on_the_device(native_lib, monkeypatch, fp32_state)
     assert 0 < sum(histories["partly"]) < n_new
     # against 1-row decoding through the stock matmul
     _same_or_parting_at_a_near_tie(model, prompt, spec, greedy, fp32_state)
+
+
+def test_long_prompt_takes_the_attention_kernel(native_lib, monkeypatch):
+    """1100 cached positions: every 16-token verify block of the attention layer goes through the
+    16-query kernel (shorter tail blocks and the prefill through the general attention)."""
+    from dflash_mlx_amd import attention_layer as A
+    from dflash_mlx_amd import kernels as K
+
+    monkeypatch.setenv("DFLASH_VERIFY_QMM", "1")
+    model = _model(13)
+    seen = []
+    real = K.batched_sdpa_2pass_exact
+    monkeypatch.setattr(A, "batched_sdpa_2pass_exact", lambda **kw: seen.append(int(kw["keys"].shape[2])) or real(**kw))
+    target = lambda ids, cache: model(ids, cache)
+    prompt = torch.randint(0, 384, (1100,), generator=torch.Generator().manual_seed(8)).to(DEV)
+    n_new = 40
+    greedy = generate_greedy(target, _cache(model, True), prompt, n_new)
+    seen.clear()
+    history = []
+    spec = generate_speculative(target, drafts(greedy.cpu(), 384, seed=4)["partly"], _cache(model, True), prompt, n_new,
+                                block_tokens=16, acceptance_history=history)
+    torch.cuda.synchronize()
+    assert len(seen) >= 2 and all(n >= 1116 for n in seen)
+    _same_or_parting_at_a_near_tie(model, prompt, spec, greedy, True)

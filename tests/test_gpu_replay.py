@@ -7,7 +7,6 @@ import numpy as np
 import pytest
 import torch
 
-import dflash_mlx_amd._native as nat
 from dflash_mlx_amd import runtime as R
 from dflash_mlx_amd.cache import KVCache
 from dflash_mlx_amd.kernels import _tape_replay_ops, replay_launch, tape_replay_kernel
