@@ -367,6 +367,15 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
   using A = Act<ACT_FP16>;
   constexpr int SBROW = 8 * CHUNK;              // bytes of scales per row and chunk
   constexpr int kChunkLoads = CHUNK == 4 ? 2 : 1;  // loads per loader and chunk
+  // The first unit is what a launch waits for longest, and its scales and biases (256 pieces
+  // of 32 bytes, one DRAM access each) are the last of it to land.  The worker waves, which
+  // have nothing to do until that unit is in LDS, ask for it as their first instructions -
+  // about a microsecond before the loader waves have their pointers set up - and the loaders
+  // start with the second unit.  CHUNK = 4: per worker lane one 16-byte load of scales or biases
+  // (wave w < 4 the scales of rows 32 w .., the others the biases), one of x (instruction w of
+  // the loaders' scheme) and two of codes (instructions 2 w, 2 w + 1).
+  constexpr bool kWorkersFetchFirstChunk = CHUNK == 4;
+  constexpr int kFirst = kWorkersFetchFirstChunk ? 1 : 0;  // units at the head of the range the loaders skip
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
   const int tid = threadIdx.x;
@@ -527,15 +536,19 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
     };
 
     int rb_i = rb0, st_i = st0;  // next unit to issue
-    int issued = u0;
-    int slot_i = 0;     // ring slot of the next unit to issue
-    int sb_slot_i = 0;  // scale/bias slot of the next chunk to issue
-    set_row_block(rb_i);
+    int issued = u0 + kFirst;
+    int slot_i = kFirst;  // ring slot of the next unit to issue
+    if (kFirst && ++st_i == p.stages) {
+      st_i = 0;
+      ++rb_i;
+    }
+    int sb_slot_i = kFirst;  // scale/bias slot of the next chunk to issue
+    if (issued < u1 || !kFirst) set_row_block(rb_i);
     // Issues one unit: 6 loads (2 for x, 4 for codes), plus kChunkLoads with the first unit
     // of every scale/bias chunk and with the first unit of the range.
     auto issue_next = [&]() __attribute__((always_inline)) {
       char* slot = lds + slot_i * kSlotBytes;
-      if ((st_i % CHUNK) == 0 || issued == u0) {
+      if ((st_i % CHUNK) == 0 || (!kFirst && issued == u0)) {
         char* sb = lds + kSbOffset + sb_slot_i * kSbSlotBytes;
         const size_t off = (size_t)(st_i / CHUNK) * (CHUNK * kGroups * 2);
         if (CHUNK == 4) {
@@ -563,15 +576,15 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
     // Loads this loader has issued for units u0..v.  Unit indices are global and the number
     // of stages is a multiple of CHUNK, so a unit starts a chunk iff its index is one.
     auto loads_through = [&](int v) __attribute__((always_inline)) -> int {
-      return 6 * (v - u0 + 1) + kChunkLoads * (1 + (v / CHUNK) - (u0 / CHUNK));
+      return 6 * (v - u0 + 1 - kFirst) + kChunkLoads * (1 - kFirst + (v / CHUNK) - (u0 / CHUNK));
     };
     // Waits until this loader's part of unit v has landed (loads retire in issue order).
     auto wait_unit = [&](int v) __attribute__((always_inline)) {
       wait_loads(loads_through(issued - 1) - loads_through(v));
     };
 
-    for (int i = 0; i < kAhead && issued < u1; ++i) issue_next();
-    wait_unit(u0);
+    for (int i = kFirst; i < kAhead && issued < u1; ++i) issue_next();
+    if (!kFirst) wait_unit(u0);
     asm volatile("s_barrier" ::: "memory");
     int rb_left = p.stages - st0;  // units of the current row block from unit u on
     int in_rb = 0;                 // units of the current row block this workgroup has done
@@ -603,6 +616,39 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
   }
 
   // ================================== worker waves ====================================
+  if (kWorkersFetchFirstChunk) {
+    const Where wh = locate(rb0);
+    const int G = p.K / kGS;
+    const int part = wave & 3;
+    int row = wh.rb * kRows + 32 * part + (lane >> 1);
+    row = row < p.N ? row : p.N - 1;
+    const uint16_t* mat = (wave < 4 ? p.scales : p.biases) + (size_t)wh.expert * p.N * G;
+    const char* src = (const char*)(mat + (size_t)row * G) + (lane & 1) * 16 +
+                      (size_t)(st0 / CHUNK) * (CHUNK * kGroups * 2);
+    load16_to_lds(src, lds + kSbOffset + (wave < 4 ? 0 : kSbArrayBytes) + part * 1024);
+    // x: instruction `wave` of the loaders' scheme; codes: instructions 2 wave and 2 wave + 1
+    int xrow = lane & 15;
+    if (GATHER) {
+      const int m = xrow < wh.rows ? xrow : 0;
+      xrow = (int)lds_read_u16(lds0 + kTabOffset + kTabRows + 2 * (wh.entry * 16 + m));
+    }
+    const char* xsrc = (const char*)(p.x + (size_t)xrow * p.K + (wave >> 1) * kGS +
+                                     (2 * (wave & 1) + (lane >> 5)) * 16 + ((lane >> 4) & 1) * 8) +
+                       (size_t)st0 * (kUnitK * 2);
+    load16_to_lds(xsrc, lds + kXOffset + wave * 1024);
+    const size_t row_bytes = (size_t)p.K >> 1;
+    const uint32_t* wmat = p.w + (size_t)wh.expert * p.N * (row_bytes >> 2);
+    const int w_r = lane >> 3;
+    const int w_c = (lane & 7) ^ (((w_r >> 1) & 3) << 1);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int q = 2 * wave + i;
+      int wrow = wh.rb * kRows + 8 * q + w_r;
+      wrow = wrow < p.N ? wrow : p.N - 1;
+      load16_to_lds_stream((const char*)wmat + (size_t)wrow * row_bytes + w_c * 16 + (size_t)st0 * (kUnitK / 2),
+                           lds + q * 1024);
+    }
+  }
   const int col = lane & 15;
   const int kblk = lane >> 4;
   const uint4 ones = make_uint4(A::kOnes, A::kOnes, A::kOnes, A::kOnes);
@@ -667,6 +713,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
     }
   };
 
+  if (kWorkersFetchFirstChunk) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   asm volatile("s_barrier" ::: "memory");
   next_addresses();
   operands_issue_piece<0, SBROW>(rd_x, rd_w, rd_s, op[0], acc4[0]);
