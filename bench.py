@@ -41,17 +41,25 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def build_stack(stack: str, device: str):
-    """All operands of one pass over the stack, generated on the device."""
+def build_stack(stack: str, device: str, join_gate_up: bool = False):
+    """All operands of one pass over the stack, generated on the device.  ``join_gate_up``:
+    the rows of gate_proj and up_proj (same values as in the separate form) laid end to end
+    and served by one call on gate_proj's input, as ``fuse_shared_input_linears`` arranges
+    them for projections that read the same activations."""
     import torch
 
-    from dflash_mlx_amd.workloads import make_qmm_case, seed_for, stack_linears
+    from dflash_mlx_amd.workloads import QmmCase, make_qmm_case, seed_for, stack_linears
 
     linears, layers, cfg = stack_linears(stack)
     calls = []
     for layer in range(layers):
-        for i, (_, K, N) in enumerate(linears):
-            calls.append(make_qmm_case(K, N, seed_for(cfg, layer) * 8 + i, device=device))
+        for i, (name, K, N) in enumerate(linears):
+            case = make_qmm_case(K, N, seed_for(cfg, layer) * 8 + i, device=device)
+            if join_gate_up and name == "up_proj":
+                gate = calls.pop()
+                case = QmmCase(gate.x, torch.cat([gate.w, case.w]), torch.cat([gate.scales, case.scales]),
+                               torch.cat([gate.biases, case.biases]), case.group_size)
+            calls.append(case)
     torch.cuda.synchronize()
     return calls
 
@@ -96,13 +104,15 @@ def capture(fn):
     return graph, out
 
 
-def bench_qmm_stack(stack: str, steps: int, warmup: int, device: str):
+def bench_qmm_stack(stack: str, steps: int, warmup: int, device: str, join_gate_up: bool = False):
     import torch
 
-    from dflash_mlx_amd.workloads import stack_bytes
+    from dflash_mlx_amd.workloads import qmm_algorithmic_bytes, stack_bytes
 
-    calls = build_stack(stack, device)
+    calls = build_stack(stack, device, join_gate_up)
     weight_bytes, total_bytes = stack_bytes(stack)
+    if join_gate_up:  # x and the launch are shared: count what the calls made here move
+        total_bytes = sum(qmm_algorithmic_bytes(c.K, c.N)[1] for c in calls)
     log(f"[bench] {stack} stack: {len(calls)} qmm calls/step, {weight_bytes / 1e9:.3f} GB weights")
 
     eager = run_pass(calls)  # also creates the split-K workspace outside of graph capture
@@ -511,6 +521,11 @@ def main() -> int:
         extra[f"stack_{other}"] = dict(ms_per_step=round(o["ms_per_step"], 4),
                                        weight_gbps=round(o["weight_gbps"], 1),
                                        frac_hbm=round(o["total_bytes"] / (o["event_ms_per_step"] * 1e-3) / HBM_PEAK, 4))
+        j = bench_qmm_stack(args.workload, args.steps, args.warmup, device, join_gate_up=True)
+        extra[f"stack_{args.workload}_gate_up_in_one_launch"] = dict(
+            calls_per_step=j["calls_per_step"], ms_per_step=round(j["ms_per_step"], 4),
+            weight_gbps=round(j["weight_gbps"], 1), avg_launch_us=round(j["avg_launch_us"], 3),
+            frac_hbm=round(j["total_bytes"] / (j["event_ms_per_step"] * 1e-3) / HBM_PEAK, 4))
         extra["single_call_16x4096x4096"] = {k: {kk: round(vv, 4) for kk, vv in v.items()}
                                              for k, v in bench_single_call(device).items()}
         mo = bench_moe(device, args.steps, args.warmup)

@@ -41,15 +41,20 @@ def _verify_enabled_for(config: Any) -> bool:
 
 def enable_verify_linears(model: torch.nn.Module, config: Any, meta: Optional[dict] = None) -> int:
     """Load-time step of dflash_mlx/runtime.py:714-721: when the target qualifies, default
-    ``DFLASH_VERIFY_QMM`` to "1" (an explicit user setting wins) and swap the linears."""
+    ``DFLASH_VERIFY_QMM`` to "1" (an explicit user setting wins) and swap the linears.
+    Beyond the reference: swapped projections that read the same input (gate/up, q/k/v, the
+    input projections of a linear-attention layer) are then joined so that one launch serves
+    them (``fuse_shared_input_linears``; ``DFLASH_VERIFY_FUSE_SHARED_INPUT=0`` keeps them apart)."""
     if not _verify_enabled_for(config):
         return 0
     os.environ.setdefault("DFLASH_VERIFY_QMM", "1")
-    from .verify_linear import install_verify_linears
+    from .verify_linear import fuse_shared_input_linears, install_verify_linears
 
     n_swapped = install_verify_linears(model)
+    n_groups = fuse_shared_input_linears(model) if n_swapped else 0
     if meta is not None:
         meta["verify_linear_swapped"] = n_swapped
+        meta["verify_shared_input_groups"] = n_groups
     return n_swapped
 
 

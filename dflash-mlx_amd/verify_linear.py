@@ -5,17 +5,25 @@ eligibility rules (:47-75), the same per-call dispatch - ``M == 16`` goes to
 ``verify_matmul``, everything else to the stock operator (:103-143) - and the
 same install / uninstall entry points (:146-196).  A swapped module shares the
 packed weight, scales and biases tensors with the module it replaces.
+
+``fuse_shared_input_linears`` has no counterpart in the reference.  A verify call of
+16 x K against N rows costs about 8 us on this part before and after its weights stream
+(first-access latency, split-K hand-over, the gap to the next launch), whatever N is, so
+projections that read the same activations - gate/up of an MLP, q/k/v of an attention
+layer, the input projections of a linear-attention layer - are cheaper as one launch over
+their rows laid end to end than as one launch each: the module tree, every module's own
+tensors (now views into the shared storage) and all results stay as they were.
 """
 from __future__ import annotations
 
 import os
-from typing import Callable, Optional
+from typing import Callable, List, Optional, Sequence, Tuple
 
 import torch
 import torch.nn as nn
 
 from .quantized import QuantizedLinear, quantized_matmul
-from .verify_qmm import verify_matmul
+from .verify_qmm import _should_use_verify, verify_matmul
 
 _VERIFY_MAX_N_DEFAULT = 100_000
 
@@ -79,6 +87,60 @@ def is_verify_eligible(ql, path: str = "") -> bool:
     return True
 
 
+# Sibling projections that read the same input in the decoder layers the reference serves.
+SHARED_INPUT_GROUPS: Tuple[Tuple[str, ...], ...] = (
+    ("gate_proj", "up_proj"),
+    ("q_proj", "k_proj", "v_proj"),
+    ("in_proj_qkv", "in_proj_z", "in_proj_b", "in_proj_a"),
+    ("in_proj_qkvz", "in_proj_ba"),
+)
+
+
+class SharedInputGroup:
+    """Rows of several projections laid end to end: one verify launch serves them all.
+
+    The first member asked about an input computes ``x @ [W_0; W_1; ...]^T`` and every member
+    takes its columns of that product, once; a member asking twice, or about another input,
+    starts a new product.  An input is recognised by storage address, shape, strides, dtype and
+    version counter, and the group holds on to it until every member has been served, so that
+    no other live tensor can take its place in between."""
+
+    def __init__(self, members: Sequence["VerifyQuantizedLinear"]):
+        first = members[0]
+        self.group_size, self.bits = first.group_size, first.bits
+        self.weight = torch.cat([m.weight for m in members], dim=0).contiguous()
+        self.scales = torch.cat([m.scales for m in members], dim=0).contiguous()
+        self.biases = torch.cat([m.biases for m in members], dim=0).contiguous()
+        self.bounds: List[Tuple[int, int]] = []
+        row = 0
+        for m in members:
+            n = int(m.weight.shape[0])
+            self.bounds.append((row, row + n))
+            row += n
+        self._key = None
+        self._input: Optional[torch.Tensor] = None
+        self._product: Optional[torch.Tensor] = None
+        self._pending = 0
+
+    @staticmethod
+    def _key_of(x: torch.Tensor):
+        return (x.data_ptr(), tuple(x.shape), tuple(x.stride()), x.dtype, x._version)
+
+    def member_output(self, index: int, x: torch.Tensor) -> torch.Tensor:
+        bit = 1 << index
+        if self._product is None or not (self._pending & bit) or self._key != self._key_of(x):
+            self._product = verify_matmul(x, self.weight, self.scales, self.biases, transpose=True,
+                                          group_size=self.group_size, bits=self.bits)
+            self._key, self._input = self._key_of(x), x
+            self._pending = (1 << len(self.bounds)) - 1
+        lo, hi = self.bounds[index]
+        out = self._product[..., lo:hi]
+        self._pending &= ~bit
+        if not self._pending:
+            self._key = self._input = self._product = None
+        return out
+
+
 def _build_dispatch(obj: "VerifyQuantizedLinear"):
     w = obj.weight
     s = obj.scales
@@ -87,12 +149,15 @@ def _build_dispatch(obj: "VerifyQuantizedLinear"):
     bits = obj.bits
     mode = obj.mode
     bias = obj.bias
+    shared = getattr(obj, "_shared_input", None)
 
     def call(x: torch.Tensor) -> torch.Tensor:
         m = 1
         for d in x.shape[:-1]:
             m *= d
-        if m == 16:
+        if m == 16 and shared is not None and _should_use_verify(x, gs, bits, True):
+            y = shared[0].member_output(shared[1], x)
+        elif m == 16:
             y = verify_matmul(x, w, s, b, transpose=True, group_size=gs, bits=bits)
         else:
             y = quantized_matmul(x, w, s, b, transpose=True, group_size=gs, bits=bits, mode=mode)
@@ -108,6 +173,7 @@ class VerifyQuantizedLinear(QuantizedLinear):
     def from_quantized(cls, ql: QuantizedLinear) -> "VerifyQuantizedLinear":
         obj = cls(ql.weight, ql.scales, getattr(ql, "biases", None), getattr(ql, "bias", None),
                   group_size=ql.group_size, bits=ql.bits, mode=getattr(ql, "mode", "affine"))
+        object.__setattr__(obj, "_shared_input", None)
         object.__setattr__(obj, "_call_fn", _build_dispatch(obj))
         obj.requires_grad_(False)
         return obj
@@ -116,8 +182,10 @@ class VerifyQuantizedLinear(QuantizedLinear):
         return self._call_fn(x)
 
     def _apply(self, fn, *args, **kwargs):
-        # .to()/.cuda() replace the buffers; re-bind the dispatch closure to the new ones
+        # .to()/.cuda() replace the buffers; re-bind the dispatch closure to the new ones.
+        # The new buffers are no longer views into a shared-input group's storage: leave it.
         out = super()._apply(fn, *args, **kwargs)
+        object.__setattr__(self, "_shared_input", None)
         object.__setattr__(self, "_call_fn", _build_dispatch(self))
         return out
 
@@ -149,6 +217,45 @@ def install_verify_linears(model: nn.Module, *,
 
     _swap_modules(model, _maybe_swap)
     return count
+
+
+def fuse_shared_input_linears(model: nn.Module, *,
+                              groups: Sequence[Sequence[str]] = SHARED_INPUT_GROUPS) -> int:
+    """Joins, under every parent module, the swapped projections named by one of ``groups``
+    (those present, when at least two of them are and they agree in K, group size, dtype and
+    device, K is a multiple of 512 and none adds a bias vector) into a ``SharedInputGroup``.  Call it after
+    ``install_verify_linears`` and after the model sits on its device.  Returns the number of
+    groups formed.  ``DFLASH_VERIFY_FUSE_SHARED_INPUT=0`` turns it into a no-op."""
+    if os.environ.get("DFLASH_VERIFY_FUSE_SHARED_INPUT", "1").strip() == "0":
+        return 0
+    formed = 0
+    for parent in model.modules():
+        for names in groups:
+            members = [getattr(parent, n, None) for n in names]
+            members = [m for m in members if isinstance(m, VerifyQuantizedLinear)
+                       and getattr(m, "_shared_input", None) is None and m.bias is None]
+            if len(members) < 2 or len({id(m) for m in members}) != len(members):
+                continue
+            ref = members[0]
+            same = all(m.weight.shape[1] == ref.weight.shape[1] and m.group_size == ref.group_size and
+                       m.bits == ref.bits and m.mode == ref.mode and m.scales.dtype == ref.scales.dtype and
+                       m.weight.dtype == ref.weight.dtype and m.weight.device == ref.weight.device
+                       for m in members)
+            rows = sum(int(m.weight.shape[0]) for m in members)
+            # K a multiple of 512: no variant's divisibility guard can send the joint product
+            # to the stock operator, whose rounding differs between one matrix and several
+            k = int(ref.weight.shape[1]) * (32 // ref.bits)
+            if not same or k % 512 != 0 or rows >= _env_int("DFLASH_VERIFY_MAX_N", _VERIFY_MAX_N_DEFAULT):
+                continue
+            group = SharedInputGroup(members)
+            for index, (m, (lo, hi)) in enumerate(zip(members, group.bounds)):
+                # the module's own tensors become views: the stock path and state_dict see the
+                # same values, and the separate copies are released
+                m.weight, m.scales, m.biases = group.weight[lo:hi], group.scales[lo:hi], group.biases[lo:hi]
+                object.__setattr__(m, "_shared_input", (group, index))
+                object.__setattr__(m, "_call_fn", _build_dispatch(m))
+            formed += 1
+    return formed
 
 
 def uninstall_verify_linears(model: nn.Module) -> int:

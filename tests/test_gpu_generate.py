@@ -11,17 +11,21 @@ import torch
 
 from dflash_mlx_amd.generate import generate_greedy, generate_speculative
 from dflash_mlx_amd.runtime import make_target_cache
-from dflash_mlx_amd.verify_linear import VerifyQuantizedLinear, install_verify_linears
+from dflash_mlx_amd.verify_linear import (VerifyQuantizedLinear, fuse_shared_input_linears,
+                                          install_verify_linears)
 from _toy_lm import ToyHybridLM, drafts
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def _model(seed):
+def _model(seed, join_shared_input=False):
     model = ToyHybridLM(seed=seed, hidden=512, Hk=2, Hv=4, D=128, dtype=torch.bfloat16).to(DEV)
     swapped = install_verify_linears(model)
     assert swapped == sum(isinstance(m, VerifyQuantizedLinear) for m in model.modules()) > 0
+    if join_shared_input:
+        # gate/up of every MLP, q/k/v of every attention layer, qkv/z of every linear-attention layer
+        assert fuse_shared_input_linears(model) == 2 * len(model.layers)
     return model.install_hooks()
 
 
@@ -51,10 +55,10 @@ def _same_or_parting_at_a_near_tie(model, prompt, a, b, fp32_state):
     return False
 
 
-@pytest.mark.parametrize("fp32_state", [True, False])
-def test_speculative_decoding_on_the_device(native_lib, monkeypatch, fp32_state):
+@pytest.mark.parametrize("fp32_state,join_shared_input", [(True, False), (False, False), (True, True)])
+def test_speculative_decoding_on_the_device(native_lib, monkeypatch, fp32_state, join_shared_input):
     monkeypatch.setenv("DFLASH_VERIFY_QMM", "1")
-    model = _model(11)
+    model = _model(11, join_shared_input)
     target = lambda ids, cache: model(ids, cache)
     prompt = torch.randint(0, 384, (11,), generator=torch.Generator().manual_seed(5)).to(DEV)
     n_new = 64

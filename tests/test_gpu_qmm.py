@@ -13,7 +13,8 @@ import torch
 import dflash_mlx_amd._native as nat
 from dflash_mlx_amd import verify_qmm as VQ
 from dflash_mlx_amd.quantized import QuantizedLinear, quantize, quantized_matmul
-from dflash_mlx_amd.verify_linear import VerifyQuantizedLinear
+from dflash_mlx_amd.verify_linear import (VerifyQuantizedLinear, fuse_shared_input_linears,
+                                          install_verify_linears)
 from dflash_mlx_amd.workloads import make_qmm_case, seed_for
 from oracle import dflash_oracle as O
 
@@ -236,6 +237,41 @@ def test_verify_linear_on_device(verify_env, native_lib):
     # a module moved after construction still dispatches on its current buffers
     v2 = VerifyQuantizedLinear.from_quantized(QuantizedLinear.from_linear(lin.to(torch.bfloat16), 64, 4)).to(DEV)
     assert torch.equal(v2(x), direct)
+
+
+def test_shared_input_projections_in_one_launch(verify_env, native_lib, c_oracle, monkeypatch):
+    """gate/up of an MLP joined into one launch: every member's output meets the bar against
+    the exact product of its own rows, equals the columns of a direct call on the joint matrix,
+    and M != 16 still takes the stock operator on the member's rows."""
+    import dflash_mlx_amd.verify_linear as VL
+
+    K = 1024
+    cases = {"gate_proj": make_qmm_case(K, 1536, seed_for(0, 71)), "up_proj": make_qmm_case(K, 2048 + 32, seed_for(0, 72))}
+    mlp = torch.nn.Module()
+    for name, c in cases.items():
+        setattr(mlp, name, QuantizedLinear(c.w.clone(), c.scales.clone(), c.biases.clone(), group_size=64, bits=4))
+    model = torch.nn.Module()
+    model.mlp = mlp.to(DEV)
+    assert install_verify_linears(model) == 2 and fuse_shared_input_linears(model) == 1
+    launches = []
+    direct = VL.verify_matmul
+    monkeypatch.setattr(VL, "verify_matmul", lambda x, w, *a, **k: (launches.append(int(w.shape[0])), direct(x, w, *a, **k))[1])
+    for mod in (model.mlp.gate_proj, model.mlp.up_proj):
+        object.__setattr__(mod, "_call_fn", VL._build_dispatch(mod))
+    x = cases["gate_proj"].x.to(DEV)
+    out = {n: getattr(model.mlp, n)(x) for n in cases}
+    torch.cuda.synchronize()
+    assert launches == [1536 + 2080]
+    group = model.mlp.gate_proj._shared_input[0]
+    joint = VQ.verify_matmul(x, group.weight, group.scales, group.biases, group_size=64, bits=4)
+    assert torch.equal(torch.cat([out["gate_proj"], out["up_proj"]], dim=-1), joint)
+    for name, c in cases.items():
+        exact, _ = c_oracle.qmm_m16(_bits(x), c.w.numpy().view(np.uint32), _bits(c.scales), _bits(c.biases), 64, flavour=0)
+        _check_north_star(_f32(out[name]).astype(np.float64), exact.astype(np.float64))
+    x3 = (torch.randn(3, K, device=DEV)).to(torch.bfloat16)
+    c = cases["up_proj"].to(DEV)
+    assert torch.equal(model.mlp.up_proj(x3), quantized_matmul(x3, c.w, c.scales, c.biases))
+    assert launches == [1536 + 2080]
 
 
 def test_c_abi_direct_n16_and_errors(native_lib):

@@ -16,13 +16,14 @@ from dflash_mlx_amd.quantized import (QuantizedLinear, dequantize, pack_codes, q
                                       quantized_matmul, unpack_codes)
 from dflash_mlx_amd.recurrent_rollback_cache import RecurrentRollbackCache
 from dflash_mlx_amd.verify_linear import (VerifyQuantizedLinear, install_verify_linears,
-                                          is_verify_eligible, uninstall_verify_linears)
+                                          is_verify_eligible, uninstall_verify_linears,
+                                          fuse_shared_input_linears)
 from dflash_mlx_amd.workloads import make_qmm_case
 from oracle import dflash_oracle as O
 
 
-def _mk_linear(i, o):
-    lin = nn.Linear(i, o, bias=False)
+def _mk_linear(i, o, bias=False):
+    lin = nn.Linear(i, o, bias=bias)
     with torch.no_grad():
         lin.weight.copy_(torch.randn(o, i) * 0.1)
     return lin.to(torch.bfloat16)
@@ -322,3 +323,89 @@ def test_array_op_forms_match_the_oracle(g_per_dk):
         r = _tape_replay_ops(t(to), t(k), t(g), t(S0), tm)
         np.testing.assert_allclose(r.numpy(), ro, rtol=1e-12, atol=1e-13)
         np.testing.assert_allclose(r.numpy(), so, rtol=1e-9, atol=1e-10)     # replay of the full tape
+
+
+class _SharedInputToy(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.mlp = nn.Module()
+        self.mlp.gate_proj = QuantizedLinear.from_linear(_mk_linear(512, 256), 64, 4)
+        self.mlp.up_proj = QuantizedLinear.from_linear(_mk_linear(512, 384), 64, 4)
+        self.mlp.down_proj = QuantizedLinear.from_linear(_mk_linear(384, 512), 64, 4)
+        self.attn = nn.Module()
+        self.attn.q_proj = QuantizedLinear.from_linear(_mk_linear(512, 256), 64, 4)
+        self.attn.k_proj = QuantizedLinear.from_linear(_mk_linear(512, 64), 64, 4)
+        self.attn.v_proj = QuantizedLinear.from_linear(_mk_linear(512, 64, bias=True), 64, 4)   # adds a bias: stays out
+        self.odd = nn.Module()
+        self.odd.gate_proj = QuantizedLinear.from_linear(_mk_linear(384, 256), 64, 4)     # K % 512 != 0: not joined
+        self.odd.up_proj = QuantizedLinear.from_linear(_mk_linear(384, 256), 64, 4)
+
+
+def test_fuse_shared_input_groups_keep_every_result(monkeypatch):
+    """Joined projections: the modules keep their values (as views of one storage), the stock
+    path is untouched, and with the verify gate open one product serves all members once."""
+    import dflash_mlx_amd.verify_linear as VL
+
+    monkeypatch.delenv("DFLASH_VERIFY_QMM", raising=False)
+    m = _SharedInputToy()
+    assert install_verify_linears(m) == 8
+    before = {k: v.clone() for k, v in m.state_dict().items()}
+    x = torch.randn(16, 512).to(torch.bfloat16)
+    stock = {n: getattr(m.mlp, n)(x) for n in ("gate_proj", "up_proj")}
+    assert fuse_shared_input_linears(m) == 2            # gate/up of mlp, q/k of attn
+    assert fuse_shared_input_linears(m) == 0            # idempotent
+    after = m.state_dict()
+    assert before.keys() == after.keys() and all(torch.equal(before[k], after[k]) for k in before)
+    group = m.mlp.gate_proj._shared_input[0]
+    assert m.mlp.up_proj._shared_input == (group, 1) and group.bounds == [(0, 256), (256, 640)]
+    assert m.mlp.up_proj.weight.data_ptr() == group.weight[256:].data_ptr()
+    assert m.attn.v_proj._shared_input is None and m.odd.gate_proj._shared_input is None
+    assert m.attn.q_proj._shared_input[0].bounds == [(0, 256), (256, 320)]
+    # gate closed (no DFLASH_VERIFY_QMM): every member runs the stock operator on its own rows
+    for n in ("gate_proj", "up_proj"):
+        assert torch.equal(getattr(m.mlp, n)(x), stock[n])
+    x5 = torch.randn(5, 512).to(torch.bfloat16)
+    assert torch.equal(m.mlp.up_proj(x5), quantized_matmul(x5, before["mlp.up_proj.weight"], before["mlp.up_proj.scales"],
+                                                           before["mlp.up_proj.biases"]))
+
+    # gate open, device product replaced by the stock operator: count the joint products
+    calls = []
+
+    def product(x, w, s, b, **kw):
+        calls.append(int(w.shape[0]))
+        return quantized_matmul(x, w, s, b, **kw)
+
+    monkeypatch.setattr(VL, "verify_matmul", product)
+    monkeypatch.setattr(VL, "_should_use_verify", lambda x, gs, bits, tr: True)
+    for mod in (m.mlp.gate_proj, m.mlp.up_proj):
+        object.__setattr__(mod, "_call_fn", VL._build_dispatch(mod))
+    full = quantized_matmul(x, group.weight, group.scales, group.biases)
+    g1, u1 = m.mlp.gate_proj(x), m.mlp.up_proj(x)
+    assert calls == [640] and torch.equal(g1, full[:, :256]) and torch.equal(u1, full[:, 256:])
+    assert group._input is None and group._product is None           # all served: nothing held
+    # same member twice, then another input with one member left waiting
+    m.mlp.gate_proj(x)
+    m.mlp.gate_proj(x)
+    assert calls == [640, 640, 640] and group._input is x
+    x2 = torch.randn(16, 512).to(torch.bfloat16)
+    u2 = m.mlp.up_proj(x2)
+    assert calls == [640] * 4 and torch.equal(u2, quantized_matmul(x2, group.weight, group.scales, group.biases)[:, 256:])
+    # an input changed in place is a new input
+    g3 = m.mlp.gate_proj(x2)
+    assert calls == [640] * 4                      # gate of x2 was still pending
+    m.mlp.gate_proj(x2)
+    x2.add_(1.0)
+    u4 = m.mlp.up_proj(x2)
+    assert calls == [640] * 6 and torch.equal(u4, quantized_matmul(x2, group.weight, group.scales, group.biases)[:, 256:])
+    assert g3.shape == (16, 256)
+    # moving the module gives it buffers of its own: it leaves the group
+    m.mlp.up_proj._apply(lambda t: t.clone())
+    assert m.mlp.up_proj._shared_input is None
+    assert uninstall_verify_linears(m) == 8
+
+
+def test_fuse_shared_input_switch(monkeypatch):
+    m = _SharedInputToy()
+    install_verify_linears(m)
+    monkeypatch.setenv("DFLASH_VERIFY_FUSE_SHARED_INPUT", "0")
+    assert fuse_shared_input_linears(m) == 0 and m.mlp.gate_proj._shared_input is None
