@@ -295,49 +295,6 @@ constexpr int kOffBeta = kOffC + 16;   // 0 for masked and missing steps
 constexpr int kOffGate = kOffBeta + 16;  // 1 for masked and missing steps
 constexpr int kChunkLdsFloats = kOffGate + 16;
 
-// Eight consecutive elements of q, k or v as loaded: 16 bytes for the 16-bit types (WIDE = false),
-// 32 bytes for fp32.
-template <bool WIDE>
-struct Raw8 {
-  uint4 w[WIDE ? 2 : 1];
-};
-// Eight consecutive elements from element i (a multiple of 8) of a 16-byte aligned array.
-template <bool WIDE>
-__device__ __forceinline__ Raw8<WIDE> load8_raw(const void* p, size_t i) {
-  Raw8<WIDE> r;
-  if (WIDE) {
-    const uint4* src = reinterpret_cast<const uint4*>((const float*)p + i);
-    r.w[0] = src[0];
-    r.w[WIDE ? 1 : 0] = src[1];
-  } else {
-    r.w[0] = *reinterpret_cast<const uint4*>((const uint16_t*)p + i);
-  }
-  return r;
-}
-template <bool WIDE>
-__device__ __forceinline__ void raw8_to_lds(const Raw8<WIDE>& r, int dt, float* dst) {
-  const uint4 hi = r.w[WIDE ? 1 : 0];
-  const uint32_t w[8] = {r.w[0].x, r.w[0].y, r.w[0].z, r.w[0].w, hi.x, hi.y, hi.z, hi.w};
-  float o[8];
-  if (WIDE) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) o[j] = __uint_as_float(w[j]);
-  } else if (dt == DFLASH_BF16) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      o[2 * j] = __uint_as_float(w[j] << 16);
-      o[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      o[2 * j] = f16_bits_to_f32(w[j] & 0xffffu);
-      o[2 * j + 1] = f16_bits_to_f32(w[j] >> 16);
-    }
-  }
-  reinterpret_cast<float4*>(dst)[0] = float4{o[0], o[1], o[2], o[3]};
-  reinterpret_cast<float4*>(dst)[1] = float4{o[4], o[5], o[6], o[7]};
-}
 // Four consecutive elements at element i (a multiple of 4) of a 16-byte aligned array.
 __device__ __forceinline__ void store4_from_f32(void* p, size_t i, f32x4_t v, int dt) {
   if (dt == DFLASH_FP32) {
@@ -350,29 +307,6 @@ __device__ __forceinline__ void store4_from_f32(void* p, size_t i, f32x4_t v, in
                                                         f32_to_f16_bits(v.z) | (f32_to_f16_bits(v.w) << 16)};
   }
 }
-__device__ __forceinline__ f32x4_t mfma4(float x, float y, f32x4_t acc) {
-  return __builtin_amdgcn_mfma_f32_16x16x4f32(x, y, acc, 0, 0, 0);
-}
-
-// The matrix-core layout puts 4 lanes (kq) on a row of S per 16-byte access: 64 contiguous
-// bytes per row, which the memory system moves at about half the rate of full 128-byte lines
-// (stores above all).  Memory is therefore accessed with 8 lanes per row - register (t2, c) of
-// lane (li, kq) is row 16 t2 + 8 (c & 1) + li % 8, 16-byte column 8 (c / 2) + 4 (li / 8) + kq -
-// and swap_row_bit() exchanges lane bit 3 with the low bit of c between the two layouts:
-// the odd register of lanes li < 8 trades places with the even register of lanes li >= 8
-// (DPP row_ror:8 reads lane li ^ 8; the bank mask picks the half row that is written).
-__device__ __forceinline__ int memory_index(int wave, int li, int kq, int t2, int c) {
-  return (32 * wave + 16 * t2 + 8 * (c & 1) + (li & 7)) * 32 + 8 * (c >> 1) + 4 * (li >> 3) + kq;
-}
-__device__ __forceinline__ void swap_row_bit(f32x4_t& even, f32x4_t& odd) {
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const int x = __float_as_int(even[e]), y = __float_as_int(odd[e]);
-    even[e] = __int_as_float(__builtin_amdgcn_update_dpp(x, y, 0x128, 0xF, 0xC, false));
-    odd[e] = __int_as_float(__builtin_amdgcn_update_dpp(y, x, 0x128, 0xF, 0x3, false));
-  }
-}
-
 // What one (slot, head) item brings in from memory, as it sits in registers while in flight.
 template <bool WIDE>
 struct Incoming {

@@ -117,91 +117,190 @@ __device__ __forceinline__ int slot_steps(const ReplayArgs& a, int slot) {
 }
 
 // ---------------------------------------------------------------------------
-// fp32 state, Dk = Dv = 128, T <= 16: register-resident single sweep.
-// Thread (row0 = tid/32, c4 = tid%32) owns float4 column c4 of rows row0 + 8*i.
+// fp32 state, Dk = Dv = 128, T <= 16: the folded sweep as a rank-16 update on the matrix cores.
+//   S_out^T = diag(prod g) S_in^T + K'^T Delta,   K'[t][dk] = c_t[dk] k_t[dk]  (16 steps = 4 MFMAs
+// of 16 x 16 x 4 fp32 per 16 x 16 tile).  As scalar FMAs the update costs a wave 1024
+// instructions (4400 cycles) per head; with every workgroup of a CU reaching that phase at the
+// same time the memory pipes idle meanwhile.  The state sits in registers in accumulator layout
+// (see swap_row_bit) and goes in and out in full 128-byte lines.
+// LDS (floats): sK[16][kPad] | sD[16][kPad] | sG[16][128] or [16] | sGt[128]
 // ---------------------------------------------------------------------------
+constexpr int kPad = 132;  // row stride of the staged tables: step rows fall on different banks
+constexpr size_t replay_f32_128_lds_floats(bool g_per_dk) {
+  return 2 * 16 * kPad + (g_per_dk ? 16 * 128 : 16) + 128;
+}
+
+// st (accumulator layout) <- diag(sGt) st + K'^T Delta over the first 4 NB steps; MFMA j of a tile
+// covers steps 4 j + kq.
+template <int NB>
+__device__ __forceinline__ void rank_update(f32x4_t (&st)[2][8], const float* sK, const float* sD, const float* sGt,
+                                            int wave, int li, int kq) {
+  float dB[2][NB > 0 ? NB : 1];  // delta[step][32 wave + 16 t2 + li]
+#pragma unroll
+  for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+    for (int j = 0; j < NB; ++j) dB[t2][j] = sD[(4 * j + kq) * kPad + 32 * wave + 16 * t2 + li];
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    float kA[NB > 0 ? NB : 1];  // K'[step][16 c + li]
+#pragma unroll
+    for (int j = 0; j < NB; ++j) kA[j] = sK[(4 * j + kq) * kPad + 16 * c + li];
+    const float4 gt4 = *reinterpret_cast<const float4*>(sGt + 16 * c + 4 * kq);
+    const f32x4_t gt = {gt4.x, gt4.y, gt4.z, gt4.w};
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      f32x4_t acc = st[t2][c] * gt;
+#pragma unroll
+      for (int j = 0; j < NB; ++j) acc = mfma4(kA[j], dB[t2][j], acc);
+      st[t2][c] = acc;
+    }
+  }
+}
+
+template <bool TAPE_WIDE, bool K_WIDE>
 __global__ __launch_bounds__(kThreads) void replay_f32_128(ReplayArgs a) {
   extern __shared__ float smem[];
-  constexpr int Tl = 16;
-  const Smem s = carve(smem, a, Tl);
+  float* sK = smem;
+  float* sD = sK + 16 * kPad;
+  float* sG = sD + 16 * kPad;
+  float* sGt = sG + (a.g_per_dk ? 16 * 128 : 16);
   const int slot = blockIdx.x / a.Hv, hv = blockIdx.x % a.Hv;
   const int n = slot_steps(a, slot);
-  const int tid = threadIdx.x, c4 = tid & 31, row0 = tid >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kq = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
   const f32x4_t* in = reinterpret_cast<const f32x4_t*>(a.state_in) + (size_t)blockIdx.x * (128 * 32);
   f32x4_t* out = reinterpret_cast<f32x4_t*>(a.state_out) + (size_t)blockIdx.x * (128 * 32);
 
   // The tape is asked for first and the state right behind it: loads return in issue order,
   // so the tape is in LDS and the gates are folded while the 64 KiB of state are still on
-  // their way, instead of the state waiting in registers for the tape.
-  float td[8], tk[8], tg[8];
-  float tg1 = 1.f;
+  // their way, instead of the state waiting in registers for the tape.  Every request goes out
+  // before anything is awaited: thread (t = tid / 16, seg = tid % 16) fetches eight elements of
+  // step t as raw bits, and what the bits mean (dtype, mask) is sorted out afterwards.
+  const int t = tid >> 4, seg = tid & 15;
+  const bool live = t < n;
+  const bool g_wide = a.g_dtype == DFLASH_FP32;
+  // raw bytes and bits in plain registers; nothing is computed from them until the state has
+  // been asked for (see the fence below)
+  typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
+  u32x4_t rd0 = {0u, 0u, 0u, 0u}, rd1 = rd0, rk0 = rd0, rk1 = rd0, rg0 = rd0, rg1 = rd0;
+  uint32_t mask_t = 1u, mask_g = 1u, g1_bits = 0u;
   {
     const int hk = hv / (a.Hv / a.Hk);
     const size_t slotT = (size_t)slot * a.T;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int i = tid + kThreads * j, t = i >> 7, d = i & 127;  // step, element
-      const bool on = t < n && (a.mask == nullptr || a.mask[slotT + t] != 0);
-      td[j] = 0.f, tk[j] = 0.f, tg[j] = 1.f;
-      if (on) {
-        td[j] = load_as_f32(a.tape, ((slotT + t) * a.Hv + hv) * 128 + d, a.tape_dtype);
-        tk[j] = load_as_f32(a.k, ((slotT + t) * a.Hk + hk) * 128 + d, a.k_dtype);
-        if (a.g_per_dk) tg[j] = load_as_f32(a.g, ((slotT + t) * a.Hv + hv) * 128 + d, a.g_dtype);
+    if (live) {
+      const size_t d_at = ((slotT + t) * a.Hv + hv) * 128 + 8 * seg;
+      const size_t k_at = ((slotT + t) * a.Hk + hk) * 128 + 8 * seg;
+      if (TAPE_WIDE) {
+        rd0 = reinterpret_cast<const u32x4_t*>((const float*)a.tape + d_at)[0];
+        rd1 = reinterpret_cast<const u32x4_t*>((const float*)a.tape + d_at)[1];
+      } else {
+        rd0 = *reinterpret_cast<const u32x4_t*>((const uint16_t*)a.tape + d_at);
+      }
+      if (K_WIDE) {
+        rk0 = reinterpret_cast<const u32x4_t*>((const float*)a.k + k_at)[0];
+        rk1 = reinterpret_cast<const u32x4_t*>((const float*)a.k + k_at)[1];
+      } else {
+        rk0 = *reinterpret_cast<const u32x4_t*>((const uint16_t*)a.k + k_at);
+      }
+      if (a.mask != nullptr) mask_t = a.mask[slotT + t];
+      if (a.g_per_dk) {
+        if (g_wide) {
+          rg0 = reinterpret_cast<const u32x4_t*>((const float*)a.g + d_at)[0];
+          rg1 = reinterpret_cast<const u32x4_t*>((const float*)a.g + d_at)[1];
+        } else {
+          rg0 = *reinterpret_cast<const u32x4_t*>((const uint16_t*)a.g + d_at);
+        }
       }
     }
-    if (!a.g_per_dk && tid < Tl) {
-      if (tid < n && (a.mask == nullptr || a.mask[slotT + tid] != 0))
-        tg1 = load_as_f32(a.g, (slotT + tid) * a.Hv + hv, a.g_dtype);
-    }
-  }
-
-  f32x4_t st[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) st[i] = __builtin_nontemporal_load(&in[(row0 + 8 * i) * 32 + c4]);
-
-  // same tables as stage_tape(): masked and missing steps are (delta = 0, k = 0, g = 1)
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int i = tid + kThreads * j, t = i >> 7, d = i & 127;
-    s.sA[(size_t)d * Tl + t] = td[j];
-    s.sK[i] = tk[j];
-    if (a.g_per_dk) s.sG[i] = tg[j];
-  }
-  if (!a.g_per_dk && tid < Tl) s.sG[tid] = tg1;
-  __syncthreads();
-  fold_gates(a, s, n);
-  __syncthreads();
-
-  float4 bk[16];
-#pragma unroll
-  for (int t = 0; t < 16; ++t) bk[t] = reinterpret_cast<const float4*>(s.sK + (size_t)t * 128)[c4];
-  const float4 gt = reinterpret_cast<const float4*>(s.sGt)[c4];
-
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int row = row0 + 8 * i;
-    f32x4_t v = st[i];
-    v.x *= gt.x;
-    v.y *= gt.y;
-    v.z *= gt.z;
-    v.w *= gt.w;
-    const float4* dl = reinterpret_cast<const float4*>(s.sA + (size_t)row * Tl);
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const float4 d4 = dl[q];
-      const float d[4] = {d4.x, d4.y, d4.z, d4.w};
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const float4 b = bk[4 * q + u];
-        v.x += d[u] * b.x;
-        v.y += d[u] * b.y;
-        v.z += d[u] * b.z;
-        v.w += d[u] * b.w;
+    if (!a.g_per_dk && tid < n) {  // thread t < 16 also fetches the gate of step t
+      const size_t at = (slotT + tid) * a.Hv + hv;
+      if (g_wide) {
+        g1_bits = ((const uint32_t*)a.g)[at];
+      } else {
+        g1_bits = ((const uint16_t*)a.g)[at];
       }
+      if (a.mask != nullptr) mask_g = a.mask[slotT + tid];
     }
-    __builtin_nontemporal_store(v, &out[row * 32 + c4]);
   }
+
+  f32x4_t st[2][8];
+#pragma unroll
+  for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+    for (int c = 0; c < 8; ++c) st[t2][c] = __builtin_nontemporal_load(&in[memory_index(wave, li, kq, t2, c)]);
+
+  // Fence: the state's loads are out before any of the tape's values is looked at, so the
+  // wait that the first use brings covers the tape only (loads return in issue order).
+  asm volatile("" : "+v"(rd0), "+v"(rd1), "+v"(rk0), "+v"(rk1), "+v"(rg0), "+v"(rg1), "+v"(mask_t), "+v"(mask_g),
+               "+v"(g1_bits)::"memory");
+
+  // masked and missing steps are (delta = 0, k = 0, g = 1): no-op steps
+  {
+    const bool keep = live && mask_t != 0;
+    Raw8<TAPE_WIDE> rd;
+    Raw8<K_WIDE> rk;
+    const u32x4_t zero = {0u, 0u, 0u, 0u};
+    auto as_uint4 = [](u32x4_t v) { return uint4{v.x, v.y, v.z, v.w}; };
+    rd.w[0] = as_uint4(keep ? rd0 : zero);
+    rd.w[TAPE_WIDE ? 1 : 0] = as_uint4(keep ? (TAPE_WIDE ? rd1 : rd0) : zero);
+    rk.w[0] = as_uint4(keep ? rk0 : zero);
+    rk.w[K_WIDE ? 1 : 0] = as_uint4(keep ? (K_WIDE ? rk1 : rk0) : zero);
+    raw8_to_lds<TAPE_WIDE>(rd, a.tape_dtype, sD + t * kPad + 8 * seg);
+    raw8_to_lds<K_WIDE>(rk, a.k_dtype, sK + t * kPad + 8 * seg);
+    if (a.g_per_dk) {
+      float* dst = sG + t * 128 + 8 * seg;
+      if (!keep) {
+        reinterpret_cast<float4*>(dst)[0] = reinterpret_cast<float4*>(dst)[1] = float4{1.f, 1.f, 1.f, 1.f};
+      } else if (g_wide) {
+        Raw8<true> rg;
+        rg.w[0] = as_uint4(rg0), rg.w[1] = as_uint4(rg1);
+        raw8_to_lds<true>(rg, a.g_dtype, dst);
+      } else {
+        Raw8<false> rg;
+        rg.w[0] = as_uint4(rg0);
+        raw8_to_lds<false>(rg, a.g_dtype, dst);
+      }
+    } else if (tid < 16) {
+      const bool on = tid < n && mask_g != 0;
+      sG[tid] = !on ? 1.f : a.g_dtype == DFLASH_BF16 ? bf16_bits_to_f32(g1_bits)
+                          : a.g_dtype == DFLASH_FP16 ? f16_bits_to_f32(g1_bits) : __uint_as_float(g1_bits);
+    }
+  }
+  __syncthreads();
+  // suffix products of the gates into the k rows; their total into sGt
+  if (tid < 128) {
+    float c = 1.f;
+    for (int t = n - 1; t >= 0; --t) {
+      sK[t * kPad + tid] *= c;
+      c *= a.g_per_dk ? sG[t * 128 + tid] : sG[t];
+    }
+    sGt[tid] = c;
+  }
+  __syncthreads();
+
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    swap_row_bit(st[0][2 * m], st[0][2 * m + 1]);
+    swap_row_bit(st[1][2 * m], st[1][2 * m + 1]);
+  }
+  // n is uniform over the workgroup: blocks of four steps beyond it are skipped
+  switch ((n + 3) >> 2) {
+    case 0: rank_update<0>(st, sK, sD, sGt, wave, li, kq); break;
+    case 1: rank_update<1>(st, sK, sD, sGt, wave, li, kq); break;
+    case 2: rank_update<2>(st, sK, sD, sGt, wave, li, kq); break;
+    case 3: rank_update<3>(st, sK, sD, sGt, wave, li, kq); break;
+    default: rank_update<4>(st, sK, sD, sGt, wave, li, kq); break;
+  }
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    swap_row_bit(st[0][2 * m], st[0][2 * m + 1]);
+    swap_row_bit(st[1][2 * m], st[1][2 * m + 1]);
+  }
+#pragma unroll
+  for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+    for (int c = 0; c < 8; ++c) __builtin_nontemporal_store(st[t2][c], &out[memory_index(wave, li, kq, t2, c)]);
 }
 
 // ---------------------------------------------------------------------------
@@ -296,9 +395,12 @@ extern "C" int dflash_tape_replay(const void* tape, const void* k, const void* g
   DFLASH_REQUIRE(T == 0 || (tape && k && g), DFLASH_ERR_ARG, "dflash_tape_replay: null tape");
   if (slots == 0) return DFLASH_OK;
   const bool exact = exact_order != 0 || state_dtype != DFLASH_FP32;
-  const bool fast = !exact && Dk == 128 && Dv == 128 && T <= 16;
+  // the 128 x 128 kernel fetches tape, k and per-element gates 16 bytes at a time
+  const bool aligned16 = (((uintptr_t)tape | (uintptr_t)k | (g_per_dk ? (uintptr_t)g : 0)) % 16) == 0;
+  const bool fast = !exact && Dk == 128 && Dv == 128 && T <= 16 && aligned16;
   const size_t Tl = fast ? 16 : (size_t)T;
-  const size_t smem_floats = (size_t)Dv * Tl + Tl * Dk + Tl * (g_per_dk ? Dk : 1) + (size_t)Dk;
+  const size_t smem_floats = fast ? replay_f32_128_lds_floats(g_per_dk != 0)
+                                  : (size_t)Dv * Tl + Tl * Dk + Tl * (g_per_dk ? Dk : 1) + (size_t)Dk;
   const size_t smem = smem_floats * sizeof(float);
   DFLASH_REQUIRE(state_dtype != DFLASH_FP32 ||
                      (((uintptr_t)state_in % 16) == 0 && ((uintptr_t)state_out % 16) == 0),
@@ -321,7 +423,11 @@ extern "C" int dflash_tape_replay(const void* tape, const void* k, const void* g
   if (exact) {
     hipLaunchKernelGGL(replay_generic<true>, grid, block, smem, s, a);
   } else if (fast) {
-    hipLaunchKernelGGL(replay_f32_128, grid, block, smem, s, a);
+    const bool tw = tape_dtype == DFLASH_FP32, kw = k_dtype == DFLASH_FP32;
+    if (tw && kw) hipLaunchKernelGGL((replay_f32_128<true, true>), grid, block, smem, s, a);
+    else if (tw) hipLaunchKernelGGL((replay_f32_128<true, false>), grid, block, smem, s, a);
+    else if (kw) hipLaunchKernelGGL((replay_f32_128<false, true>), grid, block, smem, s, a);
+    else hipLaunchKernelGGL((replay_f32_128<false, false>), grid, block, smem, s, a);
   } else {
     hipLaunchKernelGGL(replay_generic<false>, grid, block, smem, s, a);
   }
