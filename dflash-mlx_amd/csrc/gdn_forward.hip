@@ -293,7 +293,8 @@ constexpr int kOffM = kOffLq + 256;  // (I + L)^-1
 constexpr int kOffC = kOffM + 256;
 constexpr int kOffBeta = kOffC + 16;   // 0 for masked and missing steps
 constexpr int kOffGate = kOffBeta + 16;  // 1 for masked and missing steps
-constexpr int kChunkLdsFloats = kOffGate + 16;
+constexpr int kOffOn = kOffGate + 16;    // 1 for steps that count, 0 for masked and missing ones
+constexpr int kChunkLdsFloats = kOffOn + 16;
 
 // Four consecutive elements at element i (a multiple of 4) of a 16-byte aligned array.
 __device__ __forceinline__ void store4_from_f32(void* p, size_t i, f32x4_t v, int dt) {
@@ -311,7 +312,7 @@ __device__ __forceinline__ void store4_from_f32(void* p, size_t i, f32x4_t v, in
 template <bool WIDE>
 struct Incoming {
   Raw8<WIDE> k, q, v;
-  float gate, beta;
+  uint32_t gate_bits, beta_bits, mask_byte;  // of step tid (threads below 16), as loaded
   f32x4_t st[2][8];
 };
 template <bool WIDE>
@@ -331,11 +332,23 @@ __device__ __forceinline__ void issue_item_loads(const GdnArgs& a, int item, int
     in.q = load8_raw<WIDE>(a.q, kq_at);
     in.v = load8_raw<WIDE>(a.v, v_at);
   }
-  in.gate = 1.f;
-  in.beta = 0.f;
-  if (tid < T && (a.mask == nullptr || a.mask[slotT + tid] != 0)) {
-    in.gate = load_as_f32(a.g, (slotT + tid) * a.Hv + hv, a.g_dtype);
-    in.beta = load_as_f32(a.beta, (slotT + tid) * a.Hv + hv, a.beta_dtype);
+  // gate, beta and mask of step tid as raw bits: whether the step counts is decided once the
+  // state has been asked for, so that no request waits for another one's answer
+  in.gate_bits = in.beta_bits = 0u;
+  in.mask_byte = 1u;
+  if (tid < T && tid < 16) {
+    const size_t at = (slotT + tid) * a.Hv + hv;
+    if (a.g_dtype == DFLASH_FP32) {
+      in.gate_bits = ((const uint32_t*)a.g)[at];
+    } else {
+      in.gate_bits = ((const uint16_t*)a.g)[at];
+    }
+    if (a.beta_dtype == DFLASH_FP32) {
+      in.beta_bits = ((const uint32_t*)a.beta)[at];
+    } else {
+      in.beta_bits = ((const uint16_t*)a.beta)[at];
+    }
+    if (a.mask != nullptr) in.mask_byte = a.mask[slotT + tid];
   }
   const f32x4_t* src = reinterpret_cast<const f32x4_t*>((const float*)a.state_in + (size_t)item * 128 * 128);
 #pragma unroll
@@ -343,6 +356,11 @@ __device__ __forceinline__ void issue_item_loads(const GdnArgs& a, int item, int
 #pragma unroll
     for (int c = 0; c < 8; ++c)
       in.st[t2][c] = __builtin_nontemporal_load(&src[memory_index(wave, li, kq, t2, c)]);
+  // Fence: everything above is on its way before the first of these values is looked at.
+  asm volatile("" : "+v"(in.gate_bits), "+v"(in.beta_bits), "+v"(in.mask_byte)::"memory");
+}
+__device__ __forceinline__ float bits_as_f32(uint32_t bits, int dt) {
+  return dt == DFLASH_BF16 ? bf16_bits_to_f32(bits) : dt == DFLASH_FP16 ? f16_bits_to_f32(bits) : __uint_as_float(bits);
 }
 
 // One workgroup per (slot, head); the register cap keeps at least three on a compute unit.
@@ -360,6 +378,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
   float* sC = smem + kOffC;
   float* sBeta = smem + kOffBeta;
   float* sGate = smem + kOffGate;
+  float* sOn = smem + kOffOn;
 
   const int T = a.T;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -380,8 +399,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
     raw8_to_lds(cur.v, a.in_dtype, sV + t * 128 + 8 * seg);
   }
   if (tid < 16) {
-    sGate[tid] = cur.gate;
-    sBeta[tid] = cur.beta;
+    const bool on = tid < T && cur.mask_byte != 0;  // masked and missing steps: gate 1, beta 0
+    sGate[tid] = on ? bits_as_f32(cur.gate_bits, a.g_dtype) : 1.f;
+    sBeta[tid] = on ? bits_as_f32(cur.beta_bits, a.beta_dtype) : 0.f;
+    sOn[tid] = on ? 1.f : 0.f;
   }
   __syncthreads();
   {  // c_t / c_s = prod_{s < u <= t} g_u for s <= t, and c_t itself
@@ -499,7 +520,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
     for (int j = 0; j < 4; ++j) dA[t2][j] = sD[(4 * j + kq) * 128 + 32 * wave + 16 * t2 + li];
   {
     const float ct = sC[li];
-    const bool on = li < T && (a.mask == nullptr || a.mask[slotT + li] != 0);
+    const bool on = sOn[li] != 0.f;
 #pragma unroll
     for (int t2 = 0; t2 < 2; ++t2) {
       f32x4_t Y = W[t2] * ct;

@@ -158,7 +158,7 @@ __device__ __forceinline__ void rank_update(f32x4_t (&st)[2][8], const float* sK
 }
 
 template <bool TAPE_WIDE, bool K_WIDE>
-__global__ __launch_bounds__(kThreads) void replay_f32_128(ReplayArgs a) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void replay_f32_128(ReplayArgs a) {
   extern __shared__ float smem[];
   float* sK = smem;
   float* sD = sK + 16 * kPad;
@@ -177,8 +177,10 @@ __global__ __launch_bounds__(kThreads) void replay_f32_128(ReplayArgs a) {
   // their way, instead of the state waiting in registers for the tape.  Every request goes out
   // before anything is awaited: thread (t = tid / 16, seg = tid % 16) fetches eight elements of
   // step t as raw bits, and what the bits mean (dtype, mask) is sorted out afterwards.
+  // Rows are fetched whether accepted or not (every row below T exists): the accepted length
+  // may itself still be on its way from device memory, and nothing here waits for it.
   const int t = tid >> 4, seg = tid & 15;
-  const bool live = t < n;
+  const bool row = t < a.T;
   const bool g_wide = a.g_dtype == DFLASH_FP32;
   // raw bytes and bits in plain registers; nothing is computed from them until the state has
   // been asked for (see the fence below)
@@ -188,7 +190,7 @@ __global__ __launch_bounds__(kThreads) void replay_f32_128(ReplayArgs a) {
   {
     const int hk = hv / (a.Hv / a.Hk);
     const size_t slotT = (size_t)slot * a.T;
-    if (live) {
+    if (row) {
       const size_t d_at = ((slotT + t) * a.Hv + hv) * 128 + 8 * seg;
       const size_t k_at = ((slotT + t) * a.Hk + hk) * 128 + 8 * seg;
       if (TAPE_WIDE) {
@@ -213,7 +215,7 @@ __global__ __launch_bounds__(kThreads) void replay_f32_128(ReplayArgs a) {
         }
       }
     }
-    if (!a.g_per_dk && tid < n) {  // thread t < 16 also fetches the gate of step t
+    if (!a.g_per_dk && tid < a.T && tid < 16) {  // thread t < 16 also fetches the gate of step t
       const size_t at = (slotT + tid) * a.Hv + hv;
       if (g_wide) {
         g1_bits = ((const uint32_t*)a.g)[at];
@@ -237,7 +239,7 @@ __global__ __launch_bounds__(kThreads) void replay_f32_128(ReplayArgs a) {
 
   // masked and missing steps are (delta = 0, k = 0, g = 1): no-op steps
   {
-    const bool keep = live && mask_t != 0;
+    const bool keep = t < n && mask_t != 0;
     Raw8<TAPE_WIDE> rd;
     Raw8<K_WIDE> rk;
     const u32x4_t zero = {0u, 0u, 0u, 0u};
