@@ -288,17 +288,43 @@ __global__ __launch_bounds__(256) void sdpa_q16_merge_kernel(SdpaArgs a, int D) 
   const size_t row = blockIdx.x;  // (b * Hq + hq) * 16 + i
   const size_t rows = (size_t)a.B * a.Hq * 16;
   const int tid = threadIdx.x, c4 = tid & 63, g = tid >> 6;
+  const bool col = 4 * c4 < D;
+  // Group g adds up splits g, g + 4, ...; eight of them per round.  The first round's partial
+  // outputs are asked for before anything else, and every round asks for all eight before it
+  // uses one: a split's answer takes a microsecond, and there are up to 64 per group.
+  constexpr int kRound = 8;
+  uint2 h[kRound];
+  auto issue_round = [&](int s0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < kRound; ++j) {
+      const int s = s0 + 4 * j;
+      h[j] = uint2{0u, 0u};
+      if (col && s < a.splits) h[j] = *reinterpret_cast<const uint2*>(a.part_o + ((size_t)s * rows + row) * D + 4 * c4);
+    }
+  };
+  issue_round(g);
   if (tid < 64) {
+    f32x2_t ml[kMaxSplits / 64];
+#pragma unroll
+    for (int j = 0; j < kMaxSplits / 64; ++j) {
+      const int s = tid + 64 * j;
+      ml[j] = f32x2_t{kMasked, 0.f};
+      if (s < a.splits) ml[j] = *reinterpret_cast<const f32x2_t*>(a.part_ml + ((size_t)s * rows + row) * 2);
+    }
     float m = kMasked;
-    for (int s = tid; s < a.splits; s += 64) m = fmaxf(m, a.part_ml[((size_t)s * rows + row) * 2]);
+#pragma unroll
+    for (int j = 0; j < kMaxSplits / 64; ++j) m = fmaxf(m, ml[j][0]);
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
     float l = 0.f;
-    for (int s = tid; s < a.splits; s += 64) {
-      const f32x2_t ml = *reinterpret_cast<const f32x2_t*>(a.part_ml + ((size_t)s * rows + row) * 2);
-      const float w = __expf(ml[0] - m);
-      weight[s] = w;
-      l += w * ml[1];
+#pragma unroll
+    for (int j = 0; j < kMaxSplits / 64; ++j) {
+      const int s = tid + 64 * j;
+      if (s < a.splits) {
+        const float w = __expf(ml[j][0] - m);
+        weight[s] = w;
+        l += w * ml[j][1];
+      }
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) l += __shfl_xor(l, off, 64);
@@ -306,18 +332,21 @@ __global__ __launch_bounds__(256) void sdpa_q16_merge_kernel(SdpaArgs a, int D) 
   }
   __syncthreads();
   f32x4_t o = {0.f, 0.f, 0.f, 0.f};
-  if (4 * c4 < D) {
-    for (int s = g; s < a.splits; s += 4)
-    {
-      const uint2 h = *reinterpret_cast<const uint2*>(a.part_o + ((size_t)s * rows + row) * D + 4 * c4);
-      const f32x4_t v = {elem_to_f32<FP16>((uint16_t)h.x), elem_to_f32<FP16>((uint16_t)(h.x >> 16)),
-                         elem_to_f32<FP16>((uint16_t)h.y), elem_to_f32<FP16>((uint16_t)(h.y >> 16))};
-      o += v * weight[s];
+  for (int s0 = g; s0 < a.splits; s0 += 4 * kRound) {
+    if (s0 != g) issue_round(s0);
+#pragma unroll
+    for (int j = 0; j < kRound; ++j) {
+      const int s = s0 + 4 * j;
+      if (s < a.splits) {
+        const f32x4_t v = {elem_to_f32<FP16>((uint16_t)h[j].x), elem_to_f32<FP16>((uint16_t)(h[j].x >> 16)),
+                           elem_to_f32<FP16>((uint16_t)h[j].y), elem_to_f32<FP16>((uint16_t)(h[j].y >> 16))};
+        o += v * weight[s];
+      }
     }
   }
   acc[g][c4] = o;
   __syncthreads();
-  if (g == 0 && 4 * c4 < D) {
+  if (g == 0 && col) {
     o = acc[0][c4] + acc[1][c4] + acc[2][c4] + acc[3][c4];
     const float inv = total > 0.f ? 1.f / total : 1.f;
     const uint2 packed = {pack2<FP16>(o[0] * inv, o[1] * inv), pack2<FP16>(o[2] * inv, o[3] * inv)};
