@@ -7,18 +7,17 @@
 //     S[dv][dk] <- g_t * S[dv][dk] + k_t[dk] * delta_t[dv].
 //
 // The operation moves 2*Dv*Dk*4 bytes of state per head and almost nothing
-// else, so it is laid out for HBM streaming, not for the matrix cores:
-//  * one workgroup per (slot, value head); a thread owns one float4 column of
-//    Dk and walks the rows, so every wave load/store is 512 contiguous bytes
-//    and the whole 64 KiB tile of a 128x128 head is in flight at once;
+// else, so it is laid out for HBM streaming:
+//  * one workgroup per (slot, value head); the whole 64 KiB tile of a 128x128
+//    head is in flight at once, in and out in full 128-byte lines;
 //  * the tape (k, delta, g of <= T steps) is staged once into LDS as fp32;
-//  * for an fp32 state the T sequential sweeps are folded into a single sweep
-//    using  S_a = (prod g) S0 + sum_t delta_t (x) (c_t k_t),  c_t = prod_{u>t} g_u
-//    (c_t folded into the staged k rows, per-Dk gates included), which halves
-//    the VALU work - at 16 steps the step-by-step form would be VALU-bound
-//    before it is HBM-bound on this part.  bf16/fp16 states, which the
-//    reference rounds after every step (kernels.py:281-283), and callers that
-//    ask for it keep the step-by-step order;
+//  * for an fp32 state the T sequential sweeps are folded into a single one,
+//      S_a = (prod g) S0 + sum_t delta_t (x) (c_t k_t),  c_t = prod_{u>t} g_u
+//    (c_t folded into the staged k rows, per-Dk gates included).  For 128x128
+//    that is a rank-16 update which runs on the fp32 matrix cores; as scalar
+//    FMAs it costs more time than the memory traffic of the head.  bf16/fp16
+//    states, which the reference rounds after every step (kernels.py:281-283),
+//    and callers that ask for it keep the step-by-step order;
 //  * the accepted length is read per slot from device memory, so a rollback
 //    does not need the host to know it, and one launch covers all layers.
 #include "dflash_common.h"
