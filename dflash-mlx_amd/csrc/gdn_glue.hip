@@ -53,33 +53,80 @@ __device__ __forceinline__ float silu_rounded(float x, int dt) {
   return round_through(x * round_through(sigmoid_f32(x), dt), dt);
 }
 
-// PER adjacent elements of an array of dtype dt, starting at element i (a multiple of PER):
-// 2-byte types in 64-bit accesses when PER is a multiple of 4, one 32-bit access for a pair.
+// PER adjacent elements of an array, starting at element i (a multiple of PER), as raw bits
+// (16-bit types zero-extended): 2-byte types in 64-bit accesses when PER is a multiple of 4, one
+// 32-bit access for a pair.  Loading and interpreting are separate steps so that a wave can have
+// all of its requests out before it waits for the first answer: with the dtype switch inside, every
+// load sits in a branch of its own together with its conversion and is awaited there.
 template <int PER>
-__device__ __forceinline__ void load_adjacent(const void* p, size_t i, int dt, float (&out)[PER]) {
-  if (dt == DFLASH_FP32) {
-    const float* src = (const float*)p + i;
+__device__ __forceinline__ void load_adjacent_raw(const void* p, size_t i, bool wide, uint32_t (&raw)[PER]) {
+  // no arithmetic on what comes back: the words stay as loaded (two elements per word for an even
+  // number of 16-bit elements) until unpack_adjacent()
+  if (wide) {
+    const uint32_t* src = (const uint32_t*)p + i;
 #pragma unroll
-    for (int e = 0; e < PER; ++e) out[e] = src[e];
-    return;
-  }
-  uint16_t h[PER];
-  if (PER % 4 == 0) {
+    for (int e = 0; e < PER; ++e) raw[e] = src[e];
+  } else if (PER % 4 == 0) {
 #pragma unroll
     for (int e = 0; e < PER; e += 4) {
       const uint2 w = *reinterpret_cast<const uint2*>((const uint16_t*)p + i + e);
-      h[e] = (uint16_t)w.x, h[e + 1 < PER ? e + 1 : 0] = (uint16_t)(w.x >> 16);
-      h[e + 2 < PER ? e + 2 : 0] = (uint16_t)w.y, h[e + 3 < PER ? e + 3 : 0] = (uint16_t)(w.y >> 16);
+      raw[e / 2] = w.x, raw[e / 2 + 1 < PER ? e / 2 + 1 : 0] = w.y;
     }
   } else if (PER == 2) {
-    const uint32_t w = *reinterpret_cast<const uint32_t*>((const uint16_t*)p + i);
-    h[0] = (uint16_t)w, h[PER > 1 ? 1 : 0] = (uint16_t)(w >> 16);
+    raw[0] = *reinterpret_cast<const uint32_t*>((const uint16_t*)p + i);
   } else {
 #pragma unroll
-    for (int e = 0; e < PER; ++e) h[e] = ((const uint16_t*)p)[i + e];
+    for (int e = 0; e < PER; ++e) raw[e] = ((const uint16_t*)p)[i + e];
   }
+}
+__device__ __forceinline__ float bits_as_f32(uint32_t bits, int dt) {
+  return dt == DFLASH_BF16 ? bf16_bits_to_f32(bits) : dt == DFLASH_FP16 ? f16_bits_to_f32(bits) : __uint_as_float(bits);
+}
+template <int PER>
+__device__ __forceinline__ void unpack_adjacent(const uint32_t (&raw)[PER], int dt, float (&out)[PER]) {
 #pragma unroll
-  for (int e = 0; e < PER; ++e) out[e] = dt == DFLASH_BF16 ? bf16_bits_to_f32(h[e]) : f16_bits_to_f32(h[e]);
+  for (int e = 0; e < PER; ++e) {
+    constexpr bool kPacked = PER % 4 == 0 || PER == 2;  // as load_adjacent_raw() packs 16-bit elements
+    if (dt == DFLASH_FP32 || !kPacked) {
+      out[e] = bits_as_f32(raw[e], dt);
+    } else {
+      out[e] = bits_as_f32((e & 1) ? raw[e / 2] >> 16 : raw[e / 2] & 0xFFFFu, dt);
+    }
+  }
+}
+__device__ __forceinline__ uint32_t load_bits(const void* p, size_t i, bool wide) {
+  if (wide) return ((const uint32_t*)p)[i];
+  return ((const uint16_t*)p)[i];
+}
+template <int PER>
+__device__ __forceinline__ void load_adjacent(const void* p, size_t i, int dt, float (&out)[PER]) {
+  uint32_t raw[PER];
+  load_adjacent_raw<PER>(p, i, dt == DFLASH_FP32, raw);
+  unpack_adjacent<PER>(raw, dt, out);
+}
+// PER adjacent elements stored from fp32 (round to nearest even), packed like the loads.
+template <int PER>
+__device__ __forceinline__ void store_adjacent(void* p, size_t i, int dt, const float (&v)[PER]) {
+  if (dt == DFLASH_FP32) {
+    float* dst = (float*)p + i;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) dst[e] = v[e];
+    return;
+  }
+  uint32_t h[PER];
+#pragma unroll
+  for (int e = 0; e < PER; ++e) h[e] = dt == DFLASH_BF16 ? f32_to_bf16_bits(v[e]) : f32_to_f16_bits(v[e]);
+  if (PER % 4 == 0) {
+#pragma unroll
+    for (int e = 0; e < PER; e += 4)
+      *reinterpret_cast<uint2*>((uint16_t*)p + i + e) =
+          uint2{h[e] | (h[e + 1 < PER ? e + 1 : 0] << 16), h[e + 2 < PER ? e + 2 : 0] | (h[e + 3 < PER ? e + 3 : 0] << 16)};
+  } else if (PER == 2) {
+    *reinterpret_cast<uint32_t*>((uint16_t*)p + i) = h[0] | (h[PER > 1 ? 1 : 0] << 16);
+  } else {
+#pragma unroll
+    for (int e = 0; e < PER; ++e) ((uint16_t*)p)[i + e] = (uint16_t)h[e];
+  }
 }
 
 // One wave per (batch, step, head); heads 0..Hk-1 are q, Hk..2Hk-1 are k, the rest v.  A lane
@@ -96,43 +143,52 @@ __device__ __forceinline__ void prepare_head(const PrepareArgs& p, int b, int s,
   const int cb = is_v ? 2 * key_dim + (h - 2 * p.Hk) * p.Dv : h * p.Dk;  // q and k heads are contiguous
   const int c = cb + PER * lane;
 
-  float x[K][PER], w[PER * K];
+  const bool wide = p.dt == DFLASH_FP32, pwide = p.param_dt == DFLASH_FP32;
+  uint32_t xr[K][PER], wr[PER * K], on[K];
 #pragma unroll
   for (int j = 0; j < K; ++j) {
     const int r = s + j;  // row of [conv_state | qkv]
 #pragma unroll
-    for (int e = 0; e < PER; ++e) x[j][e] = 0.f;
+    for (int e = 0; e < PER; ++e) xr[j][e] = 0u;
+    on[j] = 1u;
     if (r < keep) {
-      if (p.conv_state) load_adjacent<PER>(p.conv_state, ((size_t)b * keep + r) * C + c, p.dt, x[j]);
-    } else if (p.mask == nullptr || p.mask[(size_t)b * p.S + (r - keep)]) {
-      load_adjacent<PER>(p.qkv, ((size_t)b * p.S + (r - keep)) * C + c, p.dt, x[j]);
+      if (p.conv_state) load_adjacent_raw<PER>(p.conv_state, ((size_t)b * keep + r) * C + c, wide, xr[j]);
+    } else {
+      load_adjacent_raw<PER>(p.qkv, ((size_t)b * p.S + (r - keep)) * C + c, wide, xr[j]);
+      if (p.mask != nullptr) on[j] = p.mask[(size_t)b * p.S + (r - keep)];
     }
   }
-  load_adjacent<PER * K>(p.conv_w, (size_t)c * K, p.dt, w);
-  float gate_a = 0.f, gate_b = 0.f, a_log = 0.f, bias = 0.f;
+  load_adjacent_raw<PER * K>(p.conv_w, (size_t)c * K, wide, wr);
+  uint32_t a_bits = 0u, b_bits = 0u, a_log_bits = 0u, bias_bits = 0u;
   const int hv = h - 2 * p.Hk;
   const size_t vrow = ((size_t)b * p.S + s) * p.Hv + (is_v ? hv : 0);
   if (is_v && lane == 0) {
-    gate_a = load_as_f32(p.a, vrow, p.dt);
-    gate_b = load_as_f32(p.b, vrow, p.dt);
-    a_log = load_as_f32(p.A_log, hv, p.param_dt);
-    bias = load_as_f32(p.dt_bias, hv, p.param_dt);
+    a_bits = load_bits(p.a, vrow, wide);
+    b_bits = load_bits(p.b, vrow, wide);
+    a_log_bits = load_bits(p.A_log, hv, pwide);
+    bias_bits = load_bits(p.dt_bias, hv, pwide);
   }
+  asm volatile("" ::: "memory");  // every request above is out before the first value is interpreted
+  float x[K][PER], w[PER * K];
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    unpack_adjacent<PER>(xr[j], p.dt, x[j]);  // zero bits are 0.0 in every dtype
+#pragma unroll
+    for (int e = 0; e < PER; ++e) x[j][e] = on[j] ? x[j][e] : 0.f;
+  }
+  unpack_adjacent<PER * K>(wr, p.dt, w);
+  const float gate_a = bits_as_f32(a_bits, p.dt), gate_b = bits_as_f32(b_bits, p.dt);
+  const float a_log = bits_as_f32(a_log_bits, p.param_dt), bias = bits_as_f32(bias_bits, p.param_dt);
 
   // the last `keep` rows of [conv_state | qkv] are the next conv state
-  if (s + keep >= p.S) {
-#pragma unroll
-    for (int e = 0; e < PER; ++e)
-      store_from_f32(p.conv_next, ((size_t)b * keep + (s + keep - p.S)) * C + c + e, x[K - 1][e], p.dt);
-  }
+  if (s + keep >= p.S) store_adjacent<PER>(p.conv_next, ((size_t)b * keep + (s + keep - p.S)) * C + c, p.dt, x[K - 1]);
   if (s == 0) {
     for (int r = p.S; r < keep; ++r) {  // blocks shorter than the state: old rows move up
       float old[PER];
 #pragma unroll
       for (int e = 0; e < PER; ++e) old[e] = 0.f;
       if (p.conv_state) load_adjacent<PER>(p.conv_state, ((size_t)b * keep + r) * C + c, p.dt, old);
-#pragma unroll
-      for (int e = 0; e < PER; ++e) store_from_f32(p.conv_next, ((size_t)b * keep + (r - p.S)) * C + c + e, old[e], p.dt);
+      store_adjacent<PER>(p.conv_next, ((size_t)b * keep + (r - p.S)) * C + c, p.dt, old);
     }
   }
 
@@ -148,8 +204,7 @@ __device__ __forceinline__ void prepare_head(const PrepareArgs& p, int b, int s,
   }
 
   if (is_v) {
-#pragma unroll
-    for (int e = 0; e < PER; ++e) store_from_f32(p.v, vrow * p.Dv + PER * lane + e, act[e], p.dt);
+    store_adjacent<PER>(p.v, vrow * p.Dv + PER * lane, p.dt, act);
     if (lane == 0) {
       // a + dt_bias and the softplus live in the promoted dtype of the two operands
       const int sum_dt = p.param_dt == DFLASH_FP32 ? DFLASH_FP32 : p.dt;
@@ -166,9 +221,10 @@ __device__ __forceinline__ void prepare_head(const PrepareArgs& p, int b, int s,
   const float scale = is_q ? p.scale_q : p.scale_k;
   void* out = is_q ? p.q : p.k;
   const size_t row = ((size_t)b * p.S + s) * p.Hk + (is_q ? h : h - p.Hk);
+  float scaled[PER];
 #pragma unroll
-  for (int e = 0; e < PER; ++e)
-    store_from_f32(out, row * p.Dk + PER * lane + e, scale * round_through(act[e] * inv_rms, p.dt), p.dt);
+  for (int e = 0; e < PER; ++e) scaled[e] = scale * round_through(act[e] * inv_rms, p.dt);
+  store_adjacent<PER>(out, row * p.Dk + PER * lane, p.dt, scaled);
 }
 
 template <int K>
@@ -198,27 +254,42 @@ struct NormArgs {
   float eps;
 };
 
-// One wave per row: rms_norm(x, weight) * silu(z).
+// One wave per row: rms_norm(x, weight) * silu(z); a lane holds PER = D / 64 adjacent elements.
+template <int PER>
+__device__ __forceinline__ void gated_norm_row(const NormArgs& p, long long row, int lane) {
+  const bool wide = p.dt == DFLASH_FP32;
+  const size_t at = (size_t)row * p.D + PER * lane;
+  uint32_t xr[PER], zr[PER], wr[PER];
+  load_adjacent_raw<PER>(p.x, at, wide, xr);
+  load_adjacent_raw<PER>(p.z, at, wide, zr);
+  load_adjacent_raw<PER>(p.weight, PER * lane, p.weight_dt == DFLASH_FP32, wr);
+  asm volatile("" ::: "memory");  // all three requests are out before the first value is interpreted
+  float x[PER], z[PER], wt[PER];
+  unpack_adjacent<PER>(xr, p.dt, x);
+  unpack_adjacent<PER>(zr, p.dt, z);
+  unpack_adjacent<PER>(wr, p.weight_dt, wt);
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) ss += x[e] * x[e];
+  const float inv_rms = 1.0f / sqrtf(wave_sum(ss) / (float)p.D + p.eps);
+  float y[PER];
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    const float normed = round_through(x[e] * inv_rms * wt[e], p.dt);
+    y[e] = silu_rounded(z[e], p.dt) * normed;
+  }
+  store_adjacent<PER>(p.y, at, p.dt, y);
+}
+
 __global__ __launch_bounds__(kWavesPerGroup * 64) void gdn_gated_norm_kernel(NormArgs p) {
   const int lane = threadIdx.x & 63;
   const long long row = (long long)blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
   if (row >= p.rows) return;
-  const int per_lane = p.D / 64;
-  float x[kMaxPerLane];
-  float ss = 0.f;
-#pragma unroll
-  for (int i = 0; i < kMaxPerLane; ++i) {
-    x[i] = i < per_lane ? load_as_f32(p.x, (size_t)row * p.D + lane + 64 * i, p.dt) : 0.f;
-    ss += x[i] * x[i];
-  }
-  const float inv_rms = 1.0f / sqrtf(wave_sum(ss) / (float)p.D + p.eps);
-#pragma unroll
-  for (int i = 0; i < kMaxPerLane; ++i) {
-    if (i >= per_lane) continue;
-    const int c = lane + 64 * i;
-    const float normed = round_through(x[i] * inv_rms * load_as_f32(p.weight, c, p.weight_dt), p.dt);
-    const float gate = silu_rounded(load_as_f32(p.z, (size_t)row * p.D + c, p.dt), p.dt);
-    store_from_f32(p.y, (size_t)row * p.D + c, gate * normed, p.dt);
+  switch (p.D / 64) {
+    case 1: gated_norm_row<1>(p, row, lane); break;
+    case 2: gated_norm_row<2>(p, row, lane); break;
+    case 3: gated_norm_row<3>(p, row, lane); break;
+    default: gated_norm_row<4>(p, row, lane); break;
   }
 }
 
