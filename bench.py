@@ -174,14 +174,17 @@ def bench_single_call(device: str, launches: int = 200):
     return out
 
 
-def bench_moe(device: str, steps: int, warmup: int, layers: int = 40):
+def bench_moe(device: str, steps: int, warmup: int, layers: int = 40, join_gate_up: bool = False):
     """config[4]: MoE-shaped verify step at M=16 - 256 experts of intermediate 512 (gate/up
     2048->512, down 512->2048), top-8 routing, gathered per-expert qmm, plus a shared expert
     through verify_matmul; `layers` layers replayed from a HIP graph.  Algorithmic bytes
-    count the weights of the experts the seeded routing actually touches."""
+    count the weights of the experts the seeded routing actually touches.  ``join_gate_up``:
+    gate and up, which read the same rows, laid end to end per expert (and for the shared
+    expert) and served by one launch each - four launches per layer instead of six."""
     import torch
 
-    from dflash_mlx_amd.verify_qmm import gather_qmm, verify_matmul
+    from dflash_mlx_amd.verify_qmm import gather_qmm, join_expert_projections, verify_matmul
+    from dflash_mlx_amd.workloads import MoeCase, QmmCase
     from dflash_mlx_amd.workloads import make_moe_case, make_qmm_case, qmm_algorithmic_bytes, seed_for
 
     per_expert = 3 * qmm_algorithmic_bytes(2048, 512)[0]
@@ -195,19 +198,29 @@ def bench_moe(device: str, steps: int, warmup: int, layers: int = 40):
         shared = [make_qmm_case(2048, 512, seed_for(4, layer) * 8 + 3, device=device),
                   make_qmm_case(2048, 512, seed_for(4, layer) * 8 + 4, device=device),
                   make_qmm_case(512, 2048, seed_for(4, layer) * 8 + 5, device=device)]
-        calls.append((gate, up, down, shared))
-        total += (int(torch.unique(gate.expert_ids).numel()) + 1) * per_expert
+        if join_gate_up:
+            (w, sc, bi), _ = join_expert_projections((gate.w, gate.scales, gate.biases), (up.w, up.scales, up.biases))
+            gate_up = MoeCase(gate.x, gate.expert_ids, w, sc, bi, 64)
+            sg, su, sd = shared
+            shared_gu = QmmCase(sg.x, torch.cat([sg.w, su.w]), torch.cat([sg.scales, su.scales]),
+                                torch.cat([sg.biases, su.biases]), 64)
+            calls.append(((gate_up, down), (shared_gu, sd)))
+            del gate, up, sg, su
+        else:
+            calls.append(((gate, up, down), tuple(shared)))
+        total += (int(torch.unique(down.expert_ids).numel()) + 1) * per_expert
     torch.cuda.synchronize()
 
     def one_pass():
         out = []
-        for gate, up, down, shared in calls:
-            for c in (gate, up, down):
+        for gathered, shared in calls:
+            for c in gathered:
                 out.append(gather_qmm(c.x, c.w, c.scales, c.biases, c.expert_ids, group_size=64))
             for c in shared:
                 out.append(verify_matmul(c.x, c.w, c.scales, c.biases))
         return out
 
+    launches_per_layer = len(calls[0][0]) + len(calls[0][1])
     g, _ = capture(one_pass)
     for _ in range(max(1, warmup)):
         g.replay()
@@ -215,7 +228,8 @@ def bench_moe(device: str, steps: int, warmup: int, layers: int = 40):
     ms = wall_ms / steps
     del g, calls
     torch.cuda.empty_cache()
-    return dict(layers=layers, ms_per_step=ms, weight_bytes=total, weight_gbps=total / (ms * 1e-3) / 1e9,
+    return dict(layers=layers, launches_per_layer=launches_per_layer,
+                ms_per_step=ms, weight_bytes=total, weight_gbps=total / (ms * 1e-3) / 1e9,
                 frac_hbm=total / (ms * 1e-3) / HBM_PEAK)
 
 
@@ -531,6 +545,9 @@ def main() -> int:
         mo = bench_moe(device, args.steps, args.warmup)
         extra["moe_35b_a3b_stack"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in mo.items()}
         log(f"[bench] moe: {mo['ms_per_step']:.3f} ms/step, {mo['weight_gbps']:.0f} GB/s")
+        mj = bench_moe(device, args.steps, args.warmup, join_gate_up=True)
+        extra["moe_35b_a3b_stack_gate_up_in_one_launch"] = {k: (round(v, 4) if isinstance(v, float) else v)
+                                                            for k, v in mj.items()}
         rp = bench_replay(device, args.steps, args.warmup)
         extra["gdn_tape_replay"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in rp.items()}
         fw = bench_gdn_forward(device, args.steps, args.warmup)

@@ -182,3 +182,21 @@ def gather_qmm(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: t
                                    group_size, _DTYPE_CODE[x2.dtype], _DTYPE_CODE[scales.dtype], stream)
     _native.check(rc, "dflash_qmm_m16_gather")
     return y.reshape(*x.shape[:-1], N)
+
+
+def join_expert_projections(*projections):
+    """Lays the rows of several per-expert projections that read the same rows of x (gate and up
+    of a switch MLP) end to end per expert: from ``(w [E, N_i, K/8], scales, biases)`` triples to
+    one ``(w [E, sum N_i, K/8], scales, biases)`` and the column bounds of each in the joint output,
+    so that one ``gather_qmm`` launch serves them all (a launch costs the same ~8 us around its
+    weight stream whether it covers one projection or two)."""
+    if len(projections) < 2:
+        raise ValueError("at least two (w, scales, biases) triples are needed")
+    w = torch.cat([p[0] for p in projections], dim=1).contiguous()
+    scales = torch.cat([p[1] for p in projections], dim=1).contiguous()
+    biases = torch.cat([p[2] for p in projections], dim=1).contiguous()
+    bounds, row = [], 0
+    for p in projections:
+        bounds.append((row, row + int(p[0].shape[1])))
+        row += int(p[0].shape[1])
+    return (w, scales, biases), bounds

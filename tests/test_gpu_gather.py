@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import dflash_mlx_amd._native as nat
-from dflash_mlx_amd.verify_qmm import gather_qmm
+from dflash_mlx_amd.verify_qmm import gather_qmm, join_expert_projections
 from dflash_mlx_amd.workloads import make_moe_case, seed_for
 from oracle import dflash_oracle as O
 
@@ -42,6 +42,27 @@ def test_config4_expert_shapes(native_lib, K, N):
     _check(case, y)
     # deterministic
     assert torch.equal(y, gather_qmm(d.x, d.w, d.scales, d.biases, d.expert_ids, group_size=64))
+
+
+def test_gate_and_up_of_the_experts_in_one_launch(native_lib):
+    """Two projections that read the same rows, laid end to end per expert: the joint launch gives
+    each of them its own product (to the same bar; the K split of the streaming kernel depends on
+    the row count, so single output roundings may differ from the separate launches)."""
+    gate = make_moe_case(1024, 384, seed_for(4, 31), experts=24)
+    up = make_moe_case(1024, 256, seed_for(4, 32), experts=24)
+    up.x, up.expert_ids = gate.x, gate.expert_ids
+    g, u = gate.to(DEV), up.to(DEV)
+    (w, sc, bi), bounds = join_expert_projections((g.w, g.scales, g.biases), (u.w, u.scales, u.biases))
+    assert bounds == [(0, 384), (384, 640)] and w.shape == (24, 640, 128)
+    y = gather_qmm(g.x, w, sc, bi, g.expert_ids, group_size=64)
+    torch.cuda.synchronize()
+    _check(gate, y[:, :384])
+    _check(up, y[:, 384:])
+    sep = torch.cat([gather_qmm(c.x, c.w, c.scales, c.biases, c.expert_ids, group_size=64) for c in (g, u)], dim=-1)
+    close = (y.float() - sep.float()).abs() <= 2 ** -7 * sep.float().abs().amax(dim=-1, keepdim=True)
+    assert bool(close.all())
+    with pytest.raises(ValueError):
+        join_expert_projections((g.w, g.scales, g.biases))
 
 
 def test_more_than_sixteen_rows_per_expert_and_unused_experts(native_lib):
