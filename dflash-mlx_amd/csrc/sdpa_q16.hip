@@ -38,6 +38,7 @@ namespace dflash {
 namespace {
 
 constexpr int kTileKeys = 32;
+constexpr int kThreads = 512;   // eight waves
 constexpr int kPadElems = 8;      // 16 bytes: rows of a tile start 16 bytes apart modulo 128
 // Score of a key that is not used: below every score a used key can have (a used key may carry
 // the dtype's lowest finite value as its mask, -3.39e38 for bf16).
@@ -87,26 +88,26 @@ __device__ __forceinline__ float elem_to_f32(uint16_t h) {
 // One workgroup per (batch, key/value head, split).  Wave w serves query head w % G and the
 // columns [slice * D / CS, (slice + 1) * D / CS) of the output, slice = w / G: with few query
 // heads per key/value head the output columns are split over CS waves (each repeats the cheap
-// K Q^T) so that a SIMD has more than one wave to switch between.  blockDim.x = 64 * max(G * CS, 4).
+// K Q^T) so that a SIMD has more than one wave to switch between.  Every launch has kThreads
+// threads: waves beyond G * CS move tiles only.
 template <int D, bool FP16, int CS, bool MASK>
-__global__ __launch_bounds__(512) void sdpa_q16_kernel(SdpaArgs a) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_q16_kernel(SdpaArgs a) {
   constexpr int kCols = D / 16 / CS;          // 16-column chunks of the output per wave
   constexpr int P = D + kPadElems;            // row pitch of a tile in LDS, elements
   constexpr int kTileElems = kTileKeys * P;   // one K or V tile
   constexpr int kChunks = kTileKeys * D / 8;  // 16-byte pieces of a tile
-  constexpr int kLoads = kChunks / 256;       // per thread with the smallest workgroup
+  constexpr int kLoads = kChunks / kThreads;  // per thread: every launch has kThreads threads
   extern __shared__ __align__(16) uint16_t lds[];  // [2][K tile | V tile]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int threads = blockDim.x;
   const int split = blockIdx.x % a.splits;
   const int bh = blockIdx.x / a.splits;
   const int b = bh / a.Hk, hk = bh % a.Hk;
   const int n_begin = split * a.keys_per_split;
   const int n_end = n_begin + a.keys_per_split < a.N ? n_begin + a.keys_per_split : a.N;
   const int j = lane & 15, kb = lane >> 4;
-  const bool computes = wave < a.G * CS;
+  const bool computes = wave < a.G * CS;  // the other waves only move tiles
   const int slice = computes ? wave / a.G : 0;
   const int hq = hk * a.G + (computes ? wave % a.G : 0);
   const size_t qrow = ((size_t)b * a.Hq + hq) * 16 + j;  // this lane's query
@@ -116,48 +117,46 @@ __global__ __launch_bounds__(512) void sdpa_q16_kernel(SdpaArgs a) {
 
   // ---- tile movement: global -> registers -> LDS.  Two register stages: the loads of tile i + 2
   // are issued before the arithmetic of tile i, and tile i + 1 goes from its registers to LDS
-  // after it, a full tile after its loads were issued. -----------------------------------------
-  uint4 kr[2][kLoads], vr[2][kLoads];
-  using Stage0 = std::integral_constant<int, 0>;
-  using Stage1 = std::integral_constant<int, 1>;
-  auto fetch = [&](auto stage, int n0) __attribute__((always_inline)) {
-    constexpr int S = decltype(stage)::value;
+  // after it, a full tile after its loads were issued.  Nothing here is conditional: rows past
+  // the end of the range repeat its last row (their scores are masked, their weights zero) and a
+  // tile past the end is fetched and dropped, so that the number of loads in flight at every wait
+  // is known when the kernel is compiled and a wait covers the older tile only. -----------------
+  typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;  // a native vector: plain loads and stores
+  struct Stage {
+    u32x4_t k[kLoads], v[kLoads];
+  };
+  Stage stage0, stage1;
+  auto fetch = [&](Stage& st, int n0) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
-      const int c = tid + i * threads;
+      const int c = tid + i * kThreads;
       const int key = c / (D / 8), piece = c % (D / 8);
-      const int n = n0 + key;
-      kr[S][i] = uint4{0u, 0u, 0u, 0u};
-      vr[S][i] = uint4{0u, 0u, 0u, 0u};
-      if (c < kChunks && n < n_end) {
-        kr[S][i] = *reinterpret_cast<const uint4*>(kbase + (size_t)n * a.k_seq_stride + 8 * piece);
-        vr[S][i] = *reinterpret_cast<const uint4*>(vbase + (size_t)n * a.v_seq_stride + 8 * piece);
-      }
+      const int n = n0 + key < n_end ? n0 + key : n_end - 1;
+      st.k[i] = *reinterpret_cast<const u32x4_t*>(kbase + (size_t)n * a.k_seq_stride + 8 * piece);
+      st.v[i] = *reinterpret_cast<const u32x4_t*>(vbase + (size_t)n * a.v_seq_stride + 8 * piece);
     }
   };
-  auto stash = [&](auto stage, int buf) __attribute__((always_inline)) {
-    constexpr int S = decltype(stage)::value;
+  auto stash = [&](const Stage& st, int buf) __attribute__((always_inline)) {
     uint16_t* sk = lds + buf * 2 * kTileElems;
     uint16_t* sv = sk + kTileElems;
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
-      const int c = tid + i * threads;
-      if (c < kChunks) {
-        const int key = c / (D / 8), piece = c % (D / 8);
-        *reinterpret_cast<uint4*>(sk + key * P + 8 * piece) = kr[S][i];
-        *reinterpret_cast<uint4*>(sv + key * P + 8 * piece) = vr[S][i];
-      }
+      const int c = tid + i * kThreads;
+      const int key = c / (D / 8), piece = c % (D / 8);
+      *reinterpret_cast<u32x4_t*>(sk + key * P + 8 * piece) = st.k[i];
+      *reinterpret_cast<u32x4_t*>(sv + key * P + 8 * piece) = st.v[i];
     }
   };
-
-  fetch(Stage0{}, n_begin);
-  fetch(Stage1{}, n_begin + kTileKeys);
 
   // ---- this wave's queries, as the B operand of K Q^T -----------------------------------------
   uint4 qreg[D / 32];
 #pragma unroll
   for (int s = 0; s < D / 32; ++s)
     qreg[s] = computes ? *reinterpret_cast<const uint4*>(a.q + qrow * D + 32 * s + 8 * kb) : uint4{0u, 0u, 0u, 0u};
+  // (asked for ahead of the tiles: loads return in order, and the first product needs these)
+
+  fetch(stage0, n_begin);
+  fetch(stage1, n_begin + kTileKeys);
 
   f32x4_t O[kCols];
 #pragma unroll
@@ -238,19 +237,19 @@ __global__ __launch_bounds__(512) void sdpa_q16_kernel(SdpaArgs a) {
 
   };
 
-  stash(Stage0{}, 0);
+  stash(stage0, 0);
   __syncthreads();
   for (int n0 = n_begin; n0 < n_end; n0 += 2 * kTileKeys) {
     // even tile in buffer 0; stage 1 holds the next tile, stage 0 is free
-    if (n0 + 2 * kTileKeys < n_end) fetch(Stage0{}, n0 + 2 * kTileKeys);
+    fetch(stage0, n0 + 2 * kTileKeys);
     compute_tile(0, n0);
-    if (n0 + kTileKeys < n_end) stash(Stage1{}, 1);
+    stash(stage1, 1);
     __syncthreads();
     if (n0 + kTileKeys >= n_end) break;
     // odd tile in buffer 1; stage 0 holds the next tile, stage 1 is free
-    if (n0 + 3 * kTileKeys < n_end) fetch(Stage1{}, n0 + 3 * kTileKeys);
+    fetch(stage1, n0 + 3 * kTileKeys);
     compute_tile(1, n0 + kTileKeys);
-    if (n0 + 2 * kTileKeys < n_end) stash(Stage0{}, 0);
+    stash(stage0, 0);
     __syncthreads();
   }
 
@@ -428,7 +427,6 @@ extern "C" int dflash_sdpa_q16(const void* q, const void* k, const void* v, cons
   hipStream_t s = (hipStream_t)stream;
   // column split: as many waves as fit eight, in powers of two
   const int cs = a.G <= 2 ? 4 : a.G <= 4 ? 2 : 1;
-  const int waves = a.G * cs < 4 ? 4 : a.G * cs;
   const size_t lds_bytes = (size_t)2 * 2 * kTileKeys * (D + kPadElems) * sizeof(uint16_t);
   const bool f16 = dtype == DFLASH_FP16;
 #define DFLASH_SDPA_ROW(D_, F_, M_)                                                                      \
@@ -450,7 +448,7 @@ extern "C" int dflash_sdpa_q16(const void* q, const void* k, const void* v, cons
     attr_set[idx] = true;
   }
   void* args[] = {&a};
-  DFLASH_HIP_OK(hipLaunchKernel(fn, dim3((unsigned)(B * Hk * a.splits)), dim3(64 * waves), args, lds_bytes, s));
+  DFLASH_HIP_OK(hipLaunchKernel(fn, dim3((unsigned)(B * Hk * a.splits)), dim3(kThreads), args, lds_bytes, s));
   if (a.splits > 1) {
     if (dtype == DFLASH_FP16) {
       hipLaunchKernelGGL(sdpa_q16_merge_kernel<true>, dim3((unsigned)(B * Hq * 16)), dim3(256), 0, s, a, D);
