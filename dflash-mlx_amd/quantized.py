@@ -12,6 +12,8 @@ holding elements ``8*(k>>3) .. +7`` of row n, element k in bits ``4*(k&7) .. +3`
 """
 from __future__ import annotations
 
+import os
+
 from typing import Optional, Tuple
 
 import torch
@@ -66,6 +68,22 @@ def quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, bia
         raise NotImplementedError(f"quantisation mode {mode!r}")
     wd = dequantize(w, scales, biases, group_size, bits, dtype=x.dtype)
     return x @ (wd.transpose(-1, -2) if transpose else wd)
+
+
+def stock_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
+                 *, transpose: bool = True, group_size: int = 64, bits: int = 4, mode: str = "affine") -> torch.Tensor:
+    """What a quantized module computes outside the verify switch: ``quantized_matmul``, except
+    that at most 16 rows of device activations take the M=16 kernel on zero-padded rows
+    (``verify_qmm.small_m_matmul``) instead of dequantising the whole matrix - one-token steps
+    and the narrow projections that the verify gate does not admit.  ``DFLASH_STOCK_KERNEL=0``
+    keeps every such call on the array-op form."""
+    if transpose and mode == "affine" and x.is_cuda and os.environ.get("DFLASH_STOCK_KERNEL", "1") != "0":
+        from .verify_qmm import small_m_matmul
+
+        y = small_m_matmul(x, w, scales, biases, group_size=group_size, bits=bits)
+        if y is not None:
+            return y
+    return quantized_matmul(x, w, scales, biases, transpose=transpose, group_size=group_size, bits=bits, mode=mode)
 
 
 def quantize(w: torch.Tensor, group_size: int = 64, bits: int = 4) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
@@ -125,8 +143,8 @@ class QuantizedLinear(nn.Module):
         return cls(w, s, b, bias, group_size=group_size, bits=bits)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        y = quantized_matmul(x, self.weight, self.scales, self.biases, transpose=True,
-                             group_size=self.group_size, bits=self.bits, mode=self.mode)
+        y = stock_matmul(x, self.weight, self.scales, self.biases, transpose=True,
+                         group_size=self.group_size, bits=self.bits, mode=self.mode)
         if self.bias is not None:
             y = y + self.bias
         return y

@@ -22,7 +22,7 @@ from typing import Callable, List, Optional, Sequence, Tuple
 import torch
 import torch.nn as nn
 
-from .quantized import QuantizedLinear, quantized_matmul
+from .quantized import QuantizedLinear, stock_matmul
 from .verify_qmm import _should_use_verify, verify_matmul
 
 _VERIFY_MAX_N_DEFAULT = 100_000
@@ -160,7 +160,7 @@ def _build_dispatch(obj: "VerifyQuantizedLinear"):
         elif m == 16:
             y = verify_matmul(x, w, s, b, transpose=True, group_size=gs, bits=bits)
         else:
-            y = quantized_matmul(x, w, s, b, transpose=True, group_size=gs, bits=bits, mode=mode)
+            y = stock_matmul(x, w, s, b, transpose=True, group_size=gs, bits=bits, mode=mode)
         return y if bias is None else y + bias
 
     return call

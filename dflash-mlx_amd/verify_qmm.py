@@ -149,6 +149,35 @@ def verify_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases
 verify_qmm = verify_matmul
 
 
+def small_m_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
+                   *, group_size: int = 64, bits: int = 4) -> "torch.Tensor | None":
+    """``x @ dequant(w).T`` for at most 16 rows of device activations through the M=16 kernel:
+    the rows are padded with zeros to 16 (a row of the product depends on its own row of x only,
+    so a row comes out the same whatever shares the block with it).  Covers what the C ABI covers
+    (N a multiple of 16, K a multiple of the group size, bf16/fp16), which is more than the
+    Python gate of ``verify_matmul`` lets through; returns None for anything else.  No
+    counterpart in the reference, whose stock operator is a fused kernel of its own: here the
+    stock operator dequantises the whole matrix with array ops, which for a one-token step or a
+    48-row projection costs far more than the product itself."""
+    if (not x.is_cuda or bits != 4 or group_size not in (32, 64, 128) or x.dtype not in _DTYPE_CODE or
+            scales.dtype not in _DTYPE_CODE or biases.dtype != scales.dtype or w.ndim != 2 or not _native.is_built()):
+        return None
+    K, N = int(x.shape[-1]), int(w.shape[0])
+    m = 1
+    for d in x.shape[:-1]:
+        m *= int(d)
+    if m < 1 or m > 16 or N % 16 != 0 or K % group_size != 0 or K % 32 != 0 or int(w.shape[1]) * 8 != K:
+        return None
+    x2 = x.reshape(m, K)
+    if m < 16:
+        x16 = torch.zeros((16, K), dtype=x.dtype, device=x.device)
+        x16[:m] = x2
+    else:
+        x16 = x2.contiguous()
+    y = _launch(x16, w.contiguous(), scales.contiguous(), biases.contiguous(), K, N, group_size, "mma2big", 1)
+    return y[:m].reshape(*x.shape[:-1], N)
+
+
 def gather_qmm(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
                expert_ids: torch.Tensor, *, group_size: int = 64, bits: int = 4) -> torch.Tensor:
     """Per-row expert selection for MoE layers: ``y[p] = x[p] @ dequant(w[expert_ids[p]]).T``.

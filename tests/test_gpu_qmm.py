@@ -12,7 +12,7 @@ import torch
 
 import dflash_mlx_amd._native as nat
 from dflash_mlx_amd import verify_qmm as VQ
-from dflash_mlx_amd.quantized import QuantizedLinear, quantize, quantized_matmul
+from dflash_mlx_amd.quantized import QuantizedLinear, quantize, quantized_matmul, stock_matmul
 from dflash_mlx_amd.verify_linear import (VerifyQuantizedLinear, fuse_shared_input_linears,
                                           install_verify_linears)
 from dflash_mlx_amd.workloads import make_qmm_case, seed_for
@@ -270,8 +270,38 @@ def test_shared_input_projections_in_one_launch(verify_env, native_lib, c_oracle
         _check_north_star(_f32(out[name]).astype(np.float64), exact.astype(np.float64))
     x3 = (torch.randn(3, K, device=DEV)).to(torch.bfloat16)
     c = cases["up_proj"].to(DEV)
-    assert torch.equal(model.mlp.up_proj(x3), quantized_matmul(x3, c.w, c.scales, c.biases))
+    assert torch.equal(model.mlp.up_proj(x3), stock_matmul(x3, c.w, c.scales, c.biases))
     assert launches == [1536 + 2080]
+
+
+def test_stock_operator_takes_the_kernel_for_few_rows(verify_env, native_lib, c_oracle):
+    """Outside the verify switch a module with at most 16 rows of device activations runs the
+    M=16 kernel on zero-padded rows: a row's result does not depend on what shares its block, a
+    48-row projection (which the Python gate of verify_matmul does not admit) is served, and
+    DFLASH_STOCK_KERNEL=0 or more than 16 rows give the array-op form."""
+    case = make_qmm_case(1024, 48, seed_for(0, 91))
+    d = case.to(DEV)
+    full = stock_matmul(d.x, d.w, d.scales, d.biases)
+    exact, _ = c_oracle.qmm_m16(_bits(case.x), case.w.numpy().view(np.uint32), _bits(case.scales), _bits(case.biases), 64,
+                                flavour=0)
+    _check_north_star(_f32(full).astype(np.float64), exact.astype(np.float64))
+    for rows in (slice(0, 1), slice(5, 6), slice(3, 12)):
+        part = stock_matmul(d.x[rows], d.w, d.scales, d.biases)
+        assert torch.equal(part, full[rows])
+    assert torch.equal(stock_matmul(d.x[:4].reshape(2, 2, 1024), d.w, d.scales, d.biases), full[:4].reshape(2, 2, 48))
+    ql = QuantizedLinear(d.w, d.scales, d.biases, group_size=64, bits=4)
+    assert torch.equal(ql(d.x[2:3]), full[2:3])
+    # the array-op form: asked for, or too many rows
+    x20 = torch.cat([d.x, d.x[:4]])
+    assert torch.equal(stock_matmul(x20, d.w, d.scales, d.biases), quantized_matmul(x20, d.w, d.scales, d.biases))
+    verify_env.setenv("DFLASH_STOCK_KERNEL", "0")
+    assert torch.equal(stock_matmul(d.x[:1], d.w, d.scales, d.biases), quantized_matmul(d.x[:1], d.w, d.scales, d.biases))
+    # and verify_matmul's own fallback stays the array-op form (the reference's A/B switch)
+    verify_env.delenv("DFLASH_STOCK_KERNEL")
+    verify_env.setenv("DFLASH_VERIFY_QMM", "0")
+    big = make_qmm_case(512, 64, 41).to(DEV)
+    assert torch.equal(VQ.verify_matmul(big.x, big.w, big.scales, big.biases),
+                       quantized_matmul(big.x, big.w, big.scales, big.biases))
 
 
 def test_c_abi_direct_n16_and_errors(native_lib):
