@@ -444,9 +444,17 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
   // Workgroups beyond the number of units leave; the others divide the units among
   // themselves, so every one of them has work and every contributor of a row block arrives.
   const int grid = (int)gridDim.x < units ? (int)gridDim.x : units;
-  if ((int)blockIdx.x >= grid) return;
-  const int u0 = range_begin(units, blockIdx.x, grid);
-  const int u1 = range_begin(units, blockIdx.x + 1, grid);
+  // Workgroups are handed to the eight XCDs in turn (b % 8), each with an L2 of its own, while
+  // neighbours in unit order share the scale/bias lines and the partial tiles of the row block
+  // they split: with a full grid, unit ranges follow the XCD-major order b % 8, b / 8, so that
+  // neighbours mostly sit behind the same L2.
+  const int xcds = 8;
+  const int wg = (grid == (int)gridDim.x && grid % xcds == 0)
+                     ? (int)(blockIdx.x % xcds) * (grid / xcds) + (int)(blockIdx.x / xcds)
+                     : (int)blockIdx.x;
+  if (wg >= grid) return;
+  const int u0 = range_begin(units, wg, grid);
+  const int u1 = range_begin(units, wg + 1, grid);
   const int rb0 = u0 / p.stages, st0 = u0 - rb0 * p.stages;  // (virtual) row block, stage
 
   // Where a virtual row block lives: entry, row block inside the matrix, expert, rows.
@@ -758,7 +766,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
           // (slot 1); partial tiles are kept in accumulator layout.  The store is not awaited
           // here: arrival is announced once, after the last unit.
           const int which = rb == rb0 ? 0 : 1;
-          store_partial(p.partials + ((size_t)blockIdx.x * 2 + which) * kPartialFloats + tid * 4, acc);
+          store_partial(p.partials + ((size_t)wg * 2 + which) * kPartialFloats + tid * 4, acc);
           shared_rb[which] = rb;
         }
         ++rb;
