@@ -297,6 +297,43 @@ __device__ __forceinline__ void load_partials8(const float* const (&p)[8], f32x4
       : "memory");
 }
 
+// The same loads for two row blocks at once: issue_partials8() only asks, and join_partials8()
+// asks for the second block's tiles and waits for both; it names the first block's registers
+// as operands of its own, so that nothing can be placed between the two that touches them
+// while they are being written.
+__device__ __forceinline__ void issue_partials8(const float* const (&p)[8], f32x4_t (&v)[8]) {
+  asm volatile(
+      "global_load_dwordx4 %0, %8, off sc1\n"
+      "global_load_dwordx4 %1, %9, off sc1\n"
+      "global_load_dwordx4 %2, %10, off sc1\n"
+      "global_load_dwordx4 %3, %11, off sc1\n"
+      "global_load_dwordx4 %4, %12, off sc1\n"
+      "global_load_dwordx4 %5, %13, off sc1\n"
+      "global_load_dwordx4 %6, %14, off sc1\n"
+      "global_load_dwordx4 %7, %15, off sc1\n"
+      : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]),
+        "=&v"(v[7])
+      : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7])
+      : "memory");
+}
+__device__ __forceinline__ void join_partials8(const float* const (&p)[8], f32x4_t (&v)[8], f32x4_t (&first)[8]) {
+  asm volatile(
+      "global_load_dwordx4 %0, %16, off sc1\n"
+      "global_load_dwordx4 %1, %17, off sc1\n"
+      "global_load_dwordx4 %2, %18, off sc1\n"
+      "global_load_dwordx4 %3, %19, off sc1\n"
+      "global_load_dwordx4 %4, %20, off sc1\n"
+      "global_load_dwordx4 %5, %21, off sc1\n"
+      "global_load_dwordx4 %6, %22, off sc1\n"
+      "global_load_dwordx4 %7, %23, off sc1\n"
+      "s_waitcnt vmcnt(0)\n"
+      : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]),
+        "=&v"(v[7]), "+v"(first[0]), "+v"(first[1]), "+v"(first[2]), "+v"(first[3]), "+v"(first[4]),
+        "+v"(first[5]), "+v"(first[6]), "+v"(first[7])
+      : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7])
+      : "memory");
+}
+
 struct Params {
   const uint16_t* x;
   const uint32_t* w;
@@ -817,31 +854,57 @@ arrive:
                : "memory");
   const bool is_last[2] = {__builtin_amdgcn_readfirstlane(last0) != 0,
                            __builtin_amdgcn_readfirstlane(last1) != 0};
+  // The last contributor to arrive adds the partial tiles in contributor order.  Only the
+  // first contributor can have started before a row block (then the block is the one its range
+  // ends in, slot 1); every later one starts inside it (slot 0).  A workgroup that is last at
+  // both of its row blocks asks for the tiles of both before it adds any: the two answers take
+  // as long as one.
+  auto sources = [&](int i, int wg0, const float* (&src)[8]) __attribute__((always_inline)) {
+    const int lo = shared_rb[i] * p.stages;
+    const int which_first = range_begin(units, wg_lo[i], grid) < lo ? 1 : 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int w = wg0 + j <= wg_hi[i] ? wg0 + j : wg_hi[i];  // surplus slots re-read the last tile
+      src[j] = p.partials + ((size_t)w * 2 + (w == wg_lo[i] ? which_first : 0)) * kPartialFloats + tid * 4;
+    }
+  };
+  auto add_round = [&](int i, int wg0, const f32x4_t (&v)[8], f32x4_t& acc) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (wg0 + j <= wg_hi[i]) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] += v[j][r];
+      }
+    }
+  };
+  f32x4_t first[2][8];
+  if (is_last[0] && is_last[1]) {
+    const float* src0[8];
+    const float* src1[8];
+    sources(0, wg_lo[0], src0);
+    sources(1, wg_lo[1], src1);
+    issue_partials8(src0, first[0]);
+    join_partials8(src1, first[1], first[0]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      if (!is_last[i]) continue;
+      const float* src[8];
+      sources(i, wg_lo[i], src);
+      load_partials8(src, first[i]);
+    }
+  }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     if (!is_last[i]) continue;
-    // The last contributor to arrive adds the partial tiles in contributor order.  Only the
-    // first contributor can have started before this row block (then the block is the one
-    // its range ends in, slot 1); every later one starts inside it (slot 0).
-    const int lo = shared_rb[i] * p.stages;
-    const int which_first = range_begin(units, wg_lo[i], grid) < lo ? 1 : 0;
     f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    for (int wg = wg_lo[i]; wg <= wg_hi[i]; wg += 8) {
+    add_round(i, wg_lo[i], first[i], acc);
+    for (int wg0 = wg_lo[i] + 8; wg0 <= wg_hi[i]; wg0 += 8) {  // more than eight contributors: long K, few rows
       const float* src[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int w = wg + j <= wg_hi[i] ? wg + j : wg_hi[i];  // surplus slots re-read the last tile
-        src[j] = p.partials + ((size_t)w * 2 + (w == wg_lo[i] ? which_first : 0)) * kPartialFloats + tid * 4;
-      }
+      sources(i, wg0, src);
       f32x4_t v[8];
       load_partials8(src, v);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        if (wg + j <= wg_hi[i]) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r) acc[r] += v[j][r];
-        }
-      }
+      add_round(i, wg0, v, acc);
     }
     emit(shared_rb[i], acc);
   }
