@@ -331,10 +331,29 @@ def bench_gdn_forward(device: str, steps: int, warmup: int):
     us = start.elapsed_time(stop) / n * 1e3
     per_head = 2 * D * D * 4 + T * (D * 2 + D * 2 + D * 4 + (Hk * 2 * D * 2) // Hv + 4 + 2)
     total = per_head * L * Hv
-    del sets
+
+    # A model's forward reaches this kernel one layer at a time (the rollback, not the forward,
+    # covers all layers at once): a launch over the 32 heads of a single layer, replayed from a
+    # HIP graph that walks the 48 layers of a state set.
+    def one_layer(i):
+        q, k, v, g, beta, state, state_out, y, tape = sets[(i // L) % 4]
+        l = i % L
+        rc = lib.dflash_gdn_forward_tape(
+            q[l].data_ptr(), k[l].data_ptr(), v[l].data_ptr(), g[l].data_ptr(), beta[l].data_ptr(),
+            state[l].data_ptr(), state_out[l].data_ptr(), y[l].data_ptr(), tape[l].data_ptr(), None,
+            1, T, Hk, Hv, D, D, _DTYPE_CODE[q.dtype], _DTYPE_CODE[g.dtype], _DTYPE_CODE[beta.dtype],
+            _DTYPE_CODE[state.dtype], 0, torch.cuda.current_stream(device).cuda_stream)
+        _native.check(rc, "dflash_gdn_forward_tape")
+
+    graph, _ = capture(lambda: [one_layer(i) for i in range(4 * L)])
+    graph.replay()
+    _, ev_ms = time_region(graph.replay, 3)
+    us_single = ev_ms / 3 / (4 * L) * 1e3
+    del sets, graph
     torch.cuda.empty_cache()
     return dict(us_per_forward=us, us_per_layer=us / L, gbps=total / us / 1e3,
-                frac_hbm=total / (us * 1e-6) / HBM_PEAK, bytes=total, layers=L, heads=Hv, steps=T)
+                frac_hbm=total / (us * 1e-6) / HBM_PEAK, bytes=total, layers=L, heads=Hv, steps=T,
+                us_per_single_layer_launch=us_single)
 
 
 def bench_gdn_glue(device: str, steps: int, warmup: int):

@@ -223,30 +223,52 @@ def fuse_shared_input_linears(model: nn.Module, *,
                               groups: Sequence[Sequence[str]] = SHARED_INPUT_GROUPS) -> int:
     """Joins, under every parent module, the swapped projections named by one of ``groups``
     (those present, when at least two of them are and they agree in K, group size, dtype and
-    device, K is a multiple of 512 and none adds a bias vector) into a ``SharedInputGroup``.  Call it after
+    device, K is a multiple of 512, the rows add up to a multiple of 32 and none adds a bias vector)
+    into a ``SharedInputGroup``; narrow projections left out of the swap (N a multiple of 16) join too.  Call it after
     ``install_verify_linears`` and after the model sits on its device.  Returns the number of
     groups formed.  ``DFLASH_VERIFY_FUSE_SHARED_INPUT=0`` turns it into a no-op."""
     if os.environ.get("DFLASH_VERIFY_FUSE_SHARED_INPUT", "1").strip() == "0":
         return 0
     formed = 0
-    for parent in model.modules():
+
+    def candidate(parent: nn.Module, name: str):
+        """(holder, attribute, module) of the projection ``parent.name`` if it can be a group
+        member, else None.  A narrow projection that the N % 32 rule kept out of the swap (the
+        48-row gates of a linear-attention layer) may still join - the joint product is what has
+        to pass the gate; a pad-to-16 wrapper around it is looked through."""
+        holder, attr, m = parent, name, getattr(parent, name, None)
+        if m is not None and getattr(m, "_dflash_exact_small_proj_wrapped", False) and hasattr(m, "linear"):
+            holder, attr, m = m, "linear", m.linear
+        narrow = (type(m) is QuantizedLinear and m.bits == 4 and m.mode == "affine" and m.group_size in (32, 64, 128)
+                  and int(m.weight.shape[0]) % 16 == 0 and m.biases is not None)
+        if (narrow or (isinstance(m, VerifyQuantizedLinear) and getattr(m, "_shared_input", None) is None)) \
+                and m.bias is None:
+            return holder, attr, m
+        return None
+
+    for parent in list(model.modules()):
         for names in groups:
-            members = [getattr(parent, n, None) for n in names]
-            members = [m for m in members if isinstance(m, VerifyQuantizedLinear)
-                       and getattr(m, "_shared_input", None) is None and m.bias is None]
-            if len(members) < 2 or len({id(m) for m in members}) != len(members):
+            found = [c for c in (candidate(parent, n) for n in names) if c is not None]
+            if len(found) < 2 or len({id(c[2]) for c in found}) != len(found):
                 continue
-            ref = members[0]
+            ref = found[0][2]
             same = all(m.weight.shape[1] == ref.weight.shape[1] and m.group_size == ref.group_size and
                        m.bits == ref.bits and m.mode == ref.mode and m.scales.dtype == ref.scales.dtype and
                        m.weight.dtype == ref.weight.dtype and m.weight.device == ref.weight.device
-                       for m in members)
-            rows = sum(int(m.weight.shape[0]) for m in members)
+                       for _, _, m in found)
+            rows = sum(int(m.weight.shape[0]) for _, _, m in found)
             # K a multiple of 512: no variant's divisibility guard can send the joint product
             # to the stock operator, whose rounding differs between one matrix and several
             k = int(ref.weight.shape[1]) * (32 // ref.bits)
-            if not same or k % 512 != 0 or rows >= _env_int("DFLASH_VERIFY_MAX_N", _VERIFY_MAX_N_DEFAULT):
+            if not same or k % 512 != 0 or rows % 32 != 0 or \
+                    rows >= _env_int("DFLASH_VERIFY_MAX_N", _VERIFY_MAX_N_DEFAULT):
                 continue
+            members = []
+            for holder, attr, m in found:
+                if not isinstance(m, VerifyQuantizedLinear):  # a narrow projection: swapped now that it has a group
+                    m = VerifyQuantizedLinear.from_quantized(m)
+                    setattr(holder, attr, m)
+                members.append(m)
             group = SharedInputGroup(members)
             for index, (m, (lo, hi)) in enumerate(zip(members, group.bounds)):
                 # the module's own tensors become views: the stock path and state_dict see the

@@ -274,6 +274,50 @@ def test_shared_input_projections_in_one_launch(verify_env, native_lib, c_oracle
     assert launches == [1536 + 2080]
 
 
+def test_input_projections_of_a_linear_attention_layer_in_one_launch(verify_env, native_lib, c_oracle, monkeypatch):
+    """qkv, z and the two 48-row gates (behind their pad-to-16 wrappers) read the same input: a
+    16-token block takes one launch for the four of them, a shorter block (padded by the wrappers
+    only) goes member by member, and every result meets the bar against its own exact product."""
+    import dflash_mlx_amd.verify_linear as VL
+    from dflash_mlx_amd.gdn_layer import _install_exact_small_proj_hooks
+
+    K = 1024
+    cases = {"in_proj_qkv": make_qmm_case(K, 1024, seed_for(0, 95)), "in_proj_z": make_qmm_case(K, 512, seed_for(0, 96)),
+             "in_proj_b": make_qmm_case(K, 48, seed_for(0, 97)), "in_proj_a": make_qmm_case(K, 48, seed_for(0, 98))}
+    la = torch.nn.Module()
+    for name, c in cases.items():
+        setattr(la, name, QuantizedLinear(c.w.clone(), c.scales.clone(), c.biases.clone(), group_size=64, bits=4))
+    model = torch.nn.Module()
+    model.linear_attn = la.to(DEV)
+    assert install_verify_linears(model) == 2
+    _install_exact_small_proj_hooks(model.linear_attn)
+    assert fuse_shared_input_linears(model) == 1
+    launches = []
+    direct = VL.verify_matmul
+    monkeypatch.setattr(VL, "verify_matmul", lambda x, w, *a, **k: (launches.append(int(w.shape[0])), direct(x, w, *a, **k))[1])
+    for name in cases:
+        mod = getattr(model.linear_attn, name)
+        mod = getattr(mod, "linear", mod)
+        object.__setattr__(mod, "_call_fn", VL._build_dispatch(mod))
+    x = cases["in_proj_qkv"].x.to(DEV).reshape(1, 16, K)
+    out = {n: getattr(model.linear_attn, n)(x) for n in cases}
+    torch.cuda.synchronize()
+    assert launches == [1024 + 512 + 48 + 48]
+    for name, c in cases.items():
+        exact, _ = c_oracle.qmm_m16(_bits(x.reshape(16, K)), c.w.numpy().view(np.uint32), _bits(c.scales), _bits(c.biases), 64,
+                                    flavour=0)
+        assert out[name].shape == (1, 16, c.N)
+        _check_north_star(_f32(out[name].reshape(16, c.N)).astype(np.float64), exact.astype(np.float64))
+    # a 3-token block: the wrappers pad the gates' input to 16 (a tensor of their own each), qkv and z see 3 rows
+    x3 = x[:, :3]
+    short = {n: getattr(model.linear_attn, n)(x3) for n in cases}
+    torch.cuda.synchronize()
+    for name, c in cases.items():
+        assert short[name].shape == (1, 3, c.N)
+        ref = out[name][:, :3].float()
+        assert (short[name].float() - ref).abs().max() <= 2 ** -6 * ref.abs().max()
+
+
 def test_stock_operator_takes_the_kernel_for_few_rows(verify_env, native_lib, c_oracle):
     """Outside the verify switch a module with at most 16 rows of device activations runs the
     M=16 kernel on zero-padded rows: a row's result does not depend on what shares its block, a

@@ -409,3 +409,43 @@ def test_fuse_shared_input_switch(monkeypatch):
     install_verify_linears(m)
     monkeypatch.setenv("DFLASH_VERIFY_FUSE_SHARED_INPUT", "0")
     assert fuse_shared_input_linears(m) == 0 and m.mlp.gate_proj._shared_input is None
+
+
+def test_narrow_projections_join_a_shared_input_group(monkeypatch):
+    """The 48-row gates of a linear-attention layer are kept out of the swap by the N % 32 rule,
+    but join the group of the layer's input projections (behind their pad-to-16 wrappers too);
+    without a group they stay what they were."""
+    from dflash_mlx_amd.gdn_layer import _install_exact_small_proj_hooks
+
+    monkeypatch.delenv("DFLASH_VERIFY_QMM", raising=False)
+
+    def layer():
+        la = nn.Module()
+        la.in_proj_qkv = QuantizedLinear.from_linear(_mk_linear(512, 256), 64, 4)
+        la.in_proj_z = QuantizedLinear.from_linear(_mk_linear(512, 128), 64, 4)
+        la.in_proj_b = QuantizedLinear.from_linear(_mk_linear(512, 48), 64, 4)
+        la.in_proj_a = QuantizedLinear.from_linear(_mk_linear(512, 48), 64, 4)
+        m = nn.Module()
+        m.linear_attn = la
+        return m
+
+    for wrap_first in (False, True):
+        m = layer()
+        x = torch.randn(16, 512).to(torch.bfloat16)
+        want = {n: getattr(m.linear_attn, n)(x) for n in ("in_proj_qkv", "in_proj_z", "in_proj_b", "in_proj_a")}
+        assert install_verify_linears(m) == 2                       # qkv and z only
+        if wrap_first:
+            _install_exact_small_proj_hooks(m.linear_attn)
+        assert fuse_shared_input_linears(m) == 1
+        if not wrap_first:
+            _install_exact_small_proj_hooks(m.linear_attn)
+        inner = m.linear_attn.in_proj_a.linear
+        assert isinstance(inner, VerifyQuantizedLinear) and inner._shared_input[0].bounds == [
+            (0, 256), (256, 384), (384, 432), (432, 480)] and inner._shared_input[1] == 3
+        for n, w in want.items():
+            assert torch.equal(getattr(m.linear_attn, n)(x), w)
+    # 256 + 48 rows are not a multiple of 32: no group, and the narrow projection is left alone
+    m = layer()
+    del m.linear_attn.in_proj_z, m.linear_attn.in_proj_a
+    install_verify_linears(m)
+    assert fuse_shared_input_linears(m) == 0 and type(m.linear_attn.in_proj_b) is QuantizedLinear
