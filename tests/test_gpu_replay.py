@@ -138,6 +138,30 @@ def test_fp32_tape_and_bf16_gate(native_lib):
     assert _rel_l2(out, _oracle_slots(case, np.full(2, 16))) <= TOL
 
 
+@pytest.mark.parametrize("g_per_dk", [False, True])
+@pytest.mark.parametrize("tape_dt,k_dt,g_dt", [(torch.bfloat16, torch.bfloat16, torch.float32),
+                                               (torch.float16, torch.float16, torch.float16),
+                                               (torch.float32, torch.bfloat16, torch.bfloat16),
+                                               (torch.bfloat16, torch.float32, torch.float32),
+                                               (torch.float32, torch.float32, torch.float32)])
+def test_matrix_core_kernel_dtypes_masks_and_short_tapes(native_lib, tape_dt, k_dt, g_dt, g_per_dk):
+    """The 128 x 128 kernel fetches the tape as raw 16-byte pieces and sorts out dtype, mask and
+    accepted length afterwards: every combination of 2- and 4-byte tape, k and gate, per-head
+    and per-element gates, with a mask, per-slot lengths and a tape of fewer than 16 steps."""
+    for T in (16, 5):
+        case = make_replay_case(3, batch=2, T=T, Hk=2, Hv=4, steps=T, g_per_dk=g_per_dk, seed=90 + T, tape_dtype=tape_dt)
+        case.k = case.k.to(k_dt)
+        case.g = case.g.to(g_dt)
+        rng = np.random.default_rng(T)
+        mask = rng.integers(0, 4, (6, T)) > 0
+        steps = torch.tensor([0, 1, T // 2, T - 1, T, T], dtype=torch.int32)
+        for m in (None, mask):
+            out = _np(_launch(case, steps, mask=m))
+            want = _oracle_slots(case, steps.numpy(), m)
+            for s in range(6):
+                assert _rel_l2(out.reshape(6, -1)[s], want.reshape(6, -1)[s]) <= TOL, (T, s, m is not None)
+
+
 @pytest.mark.parametrize("name,dt", [("bf16", torch.bfloat16), ("fp16", torch.float16)])
 def test_low_precision_state_rounds_every_step(native_lib, name, dt):
     """kernels.py:281-283: a bf16/fp16 state is rounded after every step."""
