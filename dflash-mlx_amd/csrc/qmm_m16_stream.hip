@@ -58,7 +58,10 @@ constexpr int kDepth = 5;                      // ring slots of (codes + x)
 // Units a loader keeps issued beyond the one being consumed.  A CU holds about 64 KiB of
 // loads in flight (what HBM latency times its share of the bandwidth comes to); a loader
 // that tries to issue more only sits in its issue stage and is late for the next barrier.
+// Short ranges (fewer than four units per workgroup) keep two: most of such a launch is its
+// start, where every request that is not for the first unit delays the first unit.
 constexpr int kAhead = 3;
+constexpr int kAheadShort = 2;
 constexpr int kWBytes = kRows * (kUnitK / 2);  // 16 KiB: 128 B per row
 constexpr int kXBytes = 16 * kUnitK * 2;       // 8 KiB
 constexpr int kXOffset = kWBytes;
@@ -628,7 +631,8 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       wait_loads(loads_through(issued - 1) - loads_through(v));
     };
 
-    for (int i = kFirst; i < kAhead && issued < u1; ++i) issue_next();
+    const int ahead = units < 4 * grid ? kAheadShort : kAhead;
+    for (int i = kFirst; i < ahead && issued < u1; ++i) issue_next();
     if (!kFirst) wait_unit(u0);
     asm volatile("s_barrier" ::: "memory");
     int rb_left = p.stages - st0;  // units of the current row block from unit u on
@@ -642,7 +646,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       // keep kAhead units issued beyond unit u; their slots are free: the ring has kDepth > kAhead
       // slots, and the slot of unit u itself (which may carry a cross-wave sum below) is only
       // refilled kDepth - kAhead units later
-      const int limit = u + kAhead;
+      const int limit = u + ahead;
       while (issued <= limit && issued < u1) issue_next();
       ++in_rb;
       --rb_left;
