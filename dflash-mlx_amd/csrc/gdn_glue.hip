@@ -144,37 +144,45 @@ __device__ __forceinline__ void prepare_head(const PrepareArgs& p, int b, int s,
   const int c = cb + PER * lane;
 
   const bool wide = p.dt == DFLASH_FP32, pwide = p.param_dt == DFLASH_FP32;
-  uint32_t xr[K][PER], wr[PER * K], on[K];
+  // Every load below is unconditional: which row of which array a tap comes from, and whether it
+  // counts at all, is decided by selecting the address (a tap that does not count reads some
+  // readable row and is zeroed afterwards).  Loads inside branches, with the registers they
+  // write preset to zero, make the compiler wait for earlier loads that used the same registers.
+  uint32_t xr[K][PER], wr[PER * K], mask_byte[K];
+  bool counts[K];
 #pragma unroll
   for (int j = 0; j < K; ++j) {
     const int r = s + j;  // row of [conv_state | qkv]
-#pragma unroll
-    for (int e = 0; e < PER; ++e) xr[j][e] = 0u;
-    on[j] = 1u;
-    if (r < keep) {
-      if (p.conv_state) load_adjacent_raw<PER>(p.conv_state, ((size_t)b * keep + r) * C + c, wide, xr[j]);
-    } else {
-      load_adjacent_raw<PER>(p.qkv, ((size_t)b * p.S + (r - keep)) * C + c, wide, xr[j]);
-      if (p.mask != nullptr) on[j] = p.mask[(size_t)b * p.S + (r - keep)];
-    }
+    const bool from_state = r < keep;
+    counts[j] = !from_state || p.conv_state != nullptr;
+    const void* base = (from_state && p.conv_state != nullptr) ? p.conv_state : p.qkv;
+    const size_t row = !counts[j] ? (size_t)b * p.S
+                                  : from_state ? (size_t)b * keep + r : (size_t)b * p.S + (r - keep);
+    load_adjacent_raw<PER>(base, row * C + c, wide, xr[j]);
+    // the mask byte of a qkv row; without a mask (or for a state row) some byte that is not looked at
+    const uint8_t* mp = (p.mask != nullptr && !from_state) ? p.mask + (size_t)b * p.S + (r - keep)
+                                                           : (const uint8_t*)p.qkv;
+    mask_byte[j] = *mp;
   }
   load_adjacent_raw<PER * K>(p.conv_w, (size_t)c * K, wide, wr);
-  uint32_t a_bits = 0u, b_bits = 0u, a_log_bits = 0u, bias_bits = 0u;
   const int hv = h - 2 * p.Hk;
   const size_t vrow = ((size_t)b * p.S + s) * p.Hv + (is_v ? hv : 0);
-  if (is_v && lane == 0) {
-    a_bits = load_bits(p.a, vrow, wide);
-    b_bits = load_bits(p.b, vrow, wide);
-    a_log_bits = load_bits(p.A_log, hv, pwide);
-    bias_bits = load_bits(p.dt_bias, hv, pwide);
-  }
+  // gates of the value head (key heads read head 0's and do not use them)
+  const uint32_t a_bits = load_bits(p.a, vrow, wide);
+  const uint32_t b_bits = load_bits(p.b, vrow, wide);
+  const uint32_t a_log_bits = load_bits(p.A_log, is_v ? hv : 0, pwide);
+  const uint32_t bias_bits = load_bits(p.dt_bias, is_v ? hv : 0, pwide);
   asm volatile("" ::: "memory");  // every request above is out before the first value is interpreted
   float x[K][PER], w[PER * K];
 #pragma unroll
   for (int j = 0; j < K; ++j) {
-    unpack_adjacent<PER>(xr[j], p.dt, x[j]);  // zero bits are 0.0 in every dtype
+    unpack_adjacent<PER>(xr[j], p.dt, x[j]);
+    {
+      const bool from_state = s + j < keep;
+      const bool on = counts[j] && (p.mask == nullptr || from_state || mask_byte[j] != 0);
 #pragma unroll
-    for (int e = 0; e < PER; ++e) x[j][e] = on[j] ? x[j][e] : 0.f;
+      for (int e = 0; e < PER; ++e) x[j][e] = on ? x[j][e] : 0.f;
+    }
   }
   unpack_adjacent<PER * K>(wr, p.dt, w);
   const float gate_a = bits_as_f32(a_bits, p.dt), gate_b = bits_as_f32(b_bits, p.dt);
