@@ -349,11 +349,48 @@ def bench_gdn_forward(device: str, steps: int, warmup: int):
     graph.replay()
     _, ev_ms = time_region(graph.replay, 3)
     us_single = ev_ms / 3 / (4 * L) * 1e3
-    del sets, graph
+    del graph
+
+    # ... and with the layer's gated output norm: as a launch of its own behind the forward, and
+    # computed by the forward's launch (dflash_gdn_forward_tape_norm)
+    z = torch.randn((L, T, Hv, D), generator=gen, device=device).to(torch.bfloat16)
+    weight = torch.ones(D, dtype=torch.bfloat16, device=device)
+    normed = torch.empty_like(z)
+    cur = torch.cuda.current_stream
+
+    def one_layer_then_norm(i):
+        one_layer(i)
+        y, l = sets[(i // L) % 4][7], i % L
+        rc = lib.dflash_gdn_gated_norm(y[l].data_ptr(), z[l].data_ptr(), weight.data_ptr(), normed[l].data_ptr(),
+                                       T * Hv, D, _DTYPE_CODE[y.dtype], _DTYPE_CODE[weight.dtype], 1e-6,
+                                       cur(device).cuda_stream)
+        _native.check(rc, "dflash_gdn_gated_norm")
+
+    def one_layer_with_norm(i):
+        q, k, v, g, beta, state, state_out, y, tape = sets[(i // L) % 4]
+        l = i % L
+        rc = lib.dflash_gdn_forward_tape_norm(
+            q[l].data_ptr(), k[l].data_ptr(), v[l].data_ptr(), g[l].data_ptr(), beta[l].data_ptr(),
+            state[l].data_ptr(), state_out[l].data_ptr(), z[l].data_ptr(), weight.data_ptr(), normed[l].data_ptr(),
+            tape[l].data_ptr(), None, 1, T, Hk, Hv, D, D, _DTYPE_CODE[q.dtype], _DTYPE_CODE[g.dtype],
+            _DTYPE_CODE[beta.dtype], _DTYPE_CODE[state.dtype], _DTYPE_CODE[weight.dtype], 0, 1e-6,
+            cur(device).cuda_stream)
+        _native.check(rc, "dflash_gdn_forward_tape_norm")
+
+    timings = {}
+    for name, fn in (("then_norm", one_layer_then_norm), ("with_norm", one_layer_with_norm)):
+        graph, _ = capture(lambda: [fn(i) for i in range(4 * L)])
+        graph.replay()
+        _, ev_ms = time_region(graph.replay, 3)
+        timings[name] = ev_ms / 3 / (4 * L) * 1e3
+        del graph
+    del sets
     torch.cuda.empty_cache()
     return dict(us_per_forward=us, us_per_layer=us / L, gbps=total / us / 1e3,
                 frac_hbm=total / (us * 1e-6) / HBM_PEAK, bytes=total, layers=L, heads=Hv, steps=T,
-                us_per_single_layer_launch=us_single)
+                us_per_single_layer_launch=us_single,
+                us_per_single_layer_forward_then_norm=timings["then_norm"],
+                us_per_single_layer_forward_with_norm=timings["with_norm"])
 
 
 def bench_gdn_glue(device: str, steps: int, warmup: int):

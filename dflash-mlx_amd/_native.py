@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
@@ -28,6 +28,7 @@ EXPORTED_SYMBOLS = (
     "dflash_qmm_m16_gather",
     "dflash_tape_replay",
     "dflash_gdn_forward_tape",
+    "dflash_gdn_forward_tape_norm",
     "dflash_gdn_prepare",
     "dflash_gdn_gated_norm",
     "dflash_sdpa_q16_workspace_bytes",
@@ -63,6 +64,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     )
     lib.dflash_gdn_forward_tape.restype = c.c_int
     lib.dflash_gdn_forward_tape.argtypes = [c.c_void_p] * 10 + [c.c_int] * 11 + [c.c_void_p]
+    lib.dflash_gdn_forward_tape_norm.restype = c.c_int
+    lib.dflash_gdn_forward_tape_norm.argtypes = [c.c_void_p] * 12 + [c.c_int] * 12 + [c.c_float, c.c_void_p]
     lib.dflash_gdn_prepare.restype = c.c_int
     lib.dflash_gdn_prepare.argtypes = [c.c_void_p] * 14 + [c.c_int] * 9 + [c.c_float, c.c_void_p]
     lib.dflash_gdn_gated_norm.restype = c.c_int

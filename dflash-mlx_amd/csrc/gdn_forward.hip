@@ -50,6 +50,12 @@ struct GdnArgs {
   const uint8_t* mask;
   int T, Hk, Hv, Dk, Dv;
   int in_dtype, g_dtype, beta_dtype, state_dtype, g_per_dk;
+  // gated output norm fused behind the recurrence (block kernel only): y is then
+  // silu(z) * rms_norm(recurrence output, norm_weight), z laid out like y
+  const void* z;
+  const void* norm_weight;  // [Dv]
+  int weight_dtype;
+  float eps;
 };
 
 // v + (v of the lane the DPP control names): butterfly steps inside a row of 16 lanes -
@@ -294,7 +300,8 @@ constexpr int kOffC = kOffM + 256;
 constexpr int kOffBeta = kOffC + 16;   // 0 for masked and missing steps
 constexpr int kOffGate = kOffBeta + 16;  // 1 for masked and missing steps
 constexpr int kOffOn = kOffGate + 16;    // 1 for steps that count, 0 for masked and missing ones
-constexpr int kChunkLdsFloats = kOffOn + 16;
+constexpr int kOffSS = kOffOn + 16;      // [wave][step]: a wave's share of a step's sum of squares
+constexpr int kChunkLdsFloats = kOffSS + 64;
 
 // Four consecutive elements at element i (a multiple of 4) of a 16-byte aligned array.
 __device__ __forceinline__ void store4_from_f32(void* p, size_t i, f32x4_t v, int dt) {
@@ -308,14 +315,27 @@ __device__ __forceinline__ void store4_from_f32(void* p, size_t i, f32x4_t v, in
                                                         f32_to_f16_bits(v.z) | (f32_to_f16_bits(v.w) << 16)};
   }
 }
+// The same for values that already are representable in dt (the bits are taken, not rounded).
+__device__ __forceinline__ void store4_rounded(void* p, size_t i, f32x4_t v, int dt) {
+  if (dt == DFLASH_BF16) {
+    *reinterpret_cast<uint2*>((uint16_t*)p + i) =
+        uint2{(__float_as_uint(v.x) >> 16) | (__float_as_uint(v.y) & 0xffff0000u),
+              (__float_as_uint(v.z) >> 16) | (__float_as_uint(v.w) & 0xffff0000u)};
+  } else {
+    store4_from_f32(p, i, v, dt);
+  }
+}
 // What one (slot, head) item brings in from memory, as it sits in registers while in flight.
 template <bool WIDE>
 struct Incoming {
   Raw8<WIDE> k, q, v;
   uint32_t gate_bits, beta_bits, mask_byte;  // of step tid (threads below 16), as loaded
+  // fused output norm: this lane's four columns of z (step li) and of the norm weight per row tile
+  uint2 z2[2], w2[2];    // 16-bit elements
+  f32x4_t z4[2], w4[2];  // fp32 elements
   f32x4_t st[2][8];
 };
-template <bool WIDE>
+template <bool WIDE, bool NORM>
 __device__ __forceinline__ void issue_item_loads(const GdnArgs& a, int item, int tid, Incoming<WIDE>& in) {
   const int T = a.T;
   const int slot = item / a.Hv, hv = item % a.Hv, hk = hv / (a.Hv / a.Hk);
@@ -350,6 +370,27 @@ __device__ __forceinline__ void issue_item_loads(const GdnArgs& a, int item, int
     }
     if (a.mask != nullptr) in.mask_byte = a.mask[slotT + tid];
   }
+  if (NORM) {
+    // ahead of the state, like every load whose width depends on a dtype: behind it, the branch
+    // around such a load would leave the number of loads in flight unknown at the first wait
+    const int tz = li < T ? li : T - 1;
+    const size_t zb = ((slotT + tz) * a.Hv + hv) * 128;
+    const bool wwide = a.weight_dtype == DFLASH_FP32;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      const int col = 32 * wave + 16 * t2 + 4 * kq;
+      if (WIDE) {
+        in.z4[t2] = *reinterpret_cast<const f32x4_t*>((const float*)a.z + zb + col);
+      } else {
+        in.z2[t2] = *reinterpret_cast<const uint2*>((const uint16_t*)a.z + zb + col);
+      }
+      if (wwide) {
+        in.w4[t2] = *reinterpret_cast<const f32x4_t*>((const float*)a.norm_weight + col);
+      } else {
+        in.w2[t2] = *reinterpret_cast<const uint2*>((const uint16_t*)a.norm_weight + col);
+      }
+    }
+  }
   const f32x4_t* src = reinterpret_cast<const f32x4_t*>((const float*)a.state_in + (size_t)item * 128 * 128);
 #pragma unroll
   for (int t2 = 0; t2 < 2; ++t2)
@@ -364,7 +405,7 @@ __device__ __forceinline__ float bits_as_f32(uint32_t bits, int dt) {
 }
 
 // One workgroup per (slot, head); the register cap keeps at least three on a compute unit.
-template <bool WIDE>
+template <bool WIDE, bool NORM>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void gdn_forward_chunk_128(GdnArgs a) {
   extern __shared__ __align__(16) float smem[];
   float* sK = smem + kOffK;
@@ -379,6 +420,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
   float* sBeta = smem + kOffBeta;
   float* sGate = smem + kOffGate;
   float* sOn = smem + kOffOn;
+  float* sSS = smem + kOffSS;
 
   const int T = a.T;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -387,11 +429,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
 
   Incoming<WIDE> cur;
   const int item = blockIdx.x;
-  issue_item_loads(a, item, tid, cur);
+  issue_item_loads<WIDE, NORM>(a, item, tid, cur);
   const int slot = item / a.Hv, hv = item % a.Hv;
   const size_t slotT = (size_t)slot * T;
   const size_t sbase = (size_t)item * 128 * 128;
   f32x4_t (&st)[2][8] = cur.st;
+  uint2 (&z2)[2] = cur.z2, (&w2)[2] = cur.w2;
+  f32x4_t (&z4)[2] = cur.z4, (&w4)[2] = cur.w4;
   {
     const int t = tid >> 4, seg = tid & 15;
     raw8_to_lds(cur.k, a.in_dtype, sK + t * kKPad + 8 * seg);
@@ -513,6 +557,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
   __syncthreads();
 
   // ---- Y = c W + Delta Lq^T -----------------------------------------------------------------------
+  float Yn[2][4];  // fused norm: Y rounded to the array dtype, kept until every wave's sum of squares is in
   float dA[2][4];  // Delta[row 16 t2 + li][s = 4j + kq]
 #pragma unroll
   for (int t2 = 0; t2 < 2; ++t2)
@@ -527,7 +572,23 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
 #pragma unroll
       for (int j = 0; j < 4; ++j) Y = mfma4(dA[t2][j], sLq[li * 16 + 4 * j + kq], Y);
       if (!on) Y = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      if (li < T) store4_from_f32(a.y, obase + 32 * wave + 16 * t2 + 4 * kq, Y, a.in_dtype);
+      if (!NORM) {
+        if (li < T) store4_from_f32(a.y, obase + 32 * wave + 16 * t2 + 4 * kq, Y, a.in_dtype);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Yn[t2][r] = round_through(Y[r], a.in_dtype);  // the recurrence's output, as an array
+      }
+    }
+    if (NORM) {
+      // this wave's 32 columns of step li: 8 per lane, the four lanes (li, kq) of a step added up
+      float ss = 0.f;
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) ss += Yn[t2][r] * Yn[t2][r];
+      ss += __shfl_xor(ss, 16, 64);
+      ss += __shfl_xor(ss, 32, 64);
+      if (kq == 0) sSS[16 * wave + li] = ss;  // read after the state update, behind its barrier
     }
   }
 
@@ -552,6 +613,61 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
         for (int j = 0; j < 4; ++j) acc = mfma4(kA[j], dA[t2][j], acc);
         st[t2][c] = acc;
       }
+    }
+  }
+  if (NORM) {
+    // silu(z) * rms_norm(y, weight) with the rounding points of the separate operators: y, the
+    // normalised and weighted y, sigmoid(z), z * sigmoid(z) and the product are arrays of the
+    // input dtype; sums and the reciprocal root are fp32.
+    // a bare barrier: __syncthreads() would also wait until every store issued so far has been
+    // acknowledged, and the stores of the state are about to follow
+    asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier" ::: "memory");
+    const float total = sSS[li] + sSS[16 + li] + sSS[32 + li] + sSS[48 + li];
+    float zf[2][4], wf[2][4];
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      if (WIDE) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) zf[t2][r] = z4[t2][r];
+      } else {
+        const uint32_t h[4] = {z2[t2].x & 0xFFFFu, z2[t2].x >> 16, z2[t2].y & 0xFFFFu, z2[t2].y >> 16};
+#pragma unroll
+        for (int r = 0; r < 4; ++r) zf[t2][r] = bits_as_f32(h[r], a.in_dtype);
+      }
+      if (a.weight_dtype == DFLASH_FP32) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) wf[t2][r] = w4[t2][r];
+      } else {
+        const uint32_t h[4] = {w2[t2].x & 0xFFFFu, w2[t2].x >> 16, w2[t2].y & 0xFFFFu, w2[t2].y >> 16};
+#pragma unroll
+        for (int r = 0; r < 4; ++r) wf[t2][r] = bits_as_f32(h[r], a.weight_dtype);
+      }
+    }
+    // A head's launch occupies one compute unit in eight, so whatever this tail costs per lane is
+    // added to the layer's latency in full: the 16-bit dtypes take the hardware's exp2,
+    // reciprocal and reciprocal root (each within an ulp of fp32, far below half an ulp of a
+    // 16-bit array) and a rounding written out for the dtype; fp32 arrays keep the library forms.
+    auto finish = [&](auto rnd, auto sigmoid, float inv_rms) __attribute__((always_inline)) {
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2) {
+        f32x4_t o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float normed = rnd(Yn[t2][r] * inv_rms * wf[t2][r]);
+          o[r] = rnd(rnd(zf[t2][r] * rnd(sigmoid(zf[t2][r]))) * normed);
+        }
+        if (li < T) store4_rounded(a.y, obase + 32 * wave + 16 * t2 + 4 * kq, o, a.in_dtype);
+      }
+    };
+    auto fast_sigmoid = [](float x) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * x)); };
+    if (a.in_dtype == DFLASH_BF16) {
+      finish([](float v) { uint32_t u = __float_as_uint(v); u += 0x7fffu + ((u >> 16) & 1u); return __uint_as_float(u & 0xffff0000u); },
+             fast_sigmoid, __builtin_amdgcn_rsqf(total * (1.0f / 128.0f) + a.eps));
+    } else if (a.in_dtype == DFLASH_FP16) {
+      finish([](float v) { return (float)(_Float16)v; }, fast_sigmoid, __builtin_amdgcn_rsqf(total * (1.0f / 128.0f) + a.eps));
+    } else {
+      finish([](float v) { return v; }, [](float x) { return 1.0f / (1.0f + expf(-x)); },
+             1.0f / sqrtf(total / 128.0f + a.eps));
     }
   }
   {
@@ -611,25 +727,26 @@ __global__ __launch_bounds__(kThreads) void gdn_forward_generic(GdnArgs a) {
 }  // namespace
 }  // namespace dflash
 
-extern "C" int dflash_gdn_forward_tape(const void* q, const void* k, const void* v, const void* g,
-                                       const void* beta, const void* state_in, void* state_out,
-                                       void* y, float* tape, const uint8_t* mask, int slots, int T,
-                                       int Hk, int Hv, int Dk, int Dv, int in_dtype, int g_dtype,
-                                       int beta_dtype, int state_dtype, int g_per_dk, void* stream) {
-  using namespace dflash;
-  DFLASH_REQUIRE(q && k && v && g && beta && state_in && state_out && y && tape, DFLASH_ERR_ARG,
-                 "dflash_gdn_forward_tape: null operand");
-  DFLASH_REQUIRE(state_in != state_out, DFLASH_ERR_ARG,
-                 "dflash_gdn_forward_tape: state_out must not alias state_in");
+namespace dflash {
+namespace {
+
+// Shared body of the two entry points; z == nullptr: no output norm.
+int gdn_forward_launch(const char* who, const void* q, const void* k, const void* v, const void* g, const void* beta,
+                       const void* state_in, void* state_out, void* y, float* tape, const uint8_t* mask,
+                       const void* z, const void* norm_weight, int weight_dtype, float eps, int slots, int T, int Hk,
+                       int Hv, int Dk, int Dv, int in_dtype, int g_dtype, int beta_dtype, int state_dtype,
+                       int g_per_dk, void* stream) {
+  DFLASH_REQUIRE(q && k && v && g && beta && state_in && state_out && y && tape, DFLASH_ERR_ARG, "%s: null operand", who);
+  DFLASH_REQUIRE(state_in != state_out, DFLASH_ERR_ARG, "%s: state_out must not alias state_in", who);
   auto ok = [](int dt) { return dt == DFLASH_BF16 || dt == DFLASH_FP16 || dt == DFLASH_FP32; };
-  DFLASH_REQUIRE(ok(in_dtype) && ok(g_dtype) && ok(beta_dtype) && ok(state_dtype), DFLASH_ERR_ARG,
-                 "dflash_gdn_forward_tape: unknown dtype code");
+  DFLASH_REQUIRE(ok(in_dtype) && ok(g_dtype) && ok(beta_dtype) && ok(state_dtype) && (!z || ok(weight_dtype)),
+                 DFLASH_ERR_ARG, "%s: unknown dtype code", who);
   DFLASH_REQUIRE(slots >= 0 && T >= 0 && Hk > 0 && Hv > 0 && Dk > 0 && Dv > 0, DFLASH_ERR_SHAPE,
-                 "dflash_gdn_forward_tape: non-positive dimension");
-  DFLASH_REQUIRE(Hv % Hk == 0, DFLASH_ERR_SHAPE,
-                 "dflash_gdn_forward_tape: cannot align K heads %d to V heads %d", Hk, Hv);
-  DFLASH_REQUIRE((long long)slots * Hv < (1ll << 31), DFLASH_ERR_SHAPE,
-                 "dflash_gdn_forward_tape: too many (slot, head) pairs");
+                 "%s: non-positive dimension", who);
+  DFLASH_REQUIRE(Hv % Hk == 0, DFLASH_ERR_SHAPE, "%s: cannot align K heads %d to V heads %d", who, Hk, Hv);
+  DFLASH_REQUIRE((long long)slots * Hv < (1ll << 31), DFLASH_ERR_SHAPE, "%s: too many (slot, head) pairs", who);
+  DFLASH_REQUIRE(!z || (norm_weight && Dv % 64 == 0 && Dv <= 256), DFLASH_ERR_SHAPE,
+                 "%s: the output norm needs a weight and a row length that is a multiple of 64 up to 256, got %d", who, Dv);
   if (slots == 0) return DFLASH_OK;
 
   GdnArgs a;
@@ -638,6 +755,7 @@ extern "C" int dflash_gdn_forward_tape(const void* q, const void* k, const void*
   a.T = T; a.Hk = Hk; a.Hv = Hv; a.Dk = Dk; a.Dv = Dv;
   a.in_dtype = in_dtype; a.g_dtype = g_dtype; a.beta_dtype = beta_dtype; a.state_dtype = state_dtype;
   a.g_per_dk = g_per_dk ? 1 : 0;
+  a.z = z; a.norm_weight = norm_weight; a.weight_dtype = weight_dtype; a.eps = eps;
 
   const dim3 grid((unsigned)(slots * Hv)), block(kThreads);
   hipStream_t s = (hipStream_t)stream;
@@ -648,14 +766,20 @@ extern "C" int dflash_gdn_forward_tape(const void* q, const void* k, const void*
   // DFLASH_GDN_SEQUENTIAL=1 keeps the step-by-step kernel for every shape (read per call: A/B runs)
   const char* sequential_env = getenv("DFLASH_GDN_SEQUENTIAL");
   const bool no_chunk = sequential_env && sequential_env[0] == '1';
-  const bool aligned16 = (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)y | (uintptr_t)tape) % 16) == 0;
+  const bool aligned16 = (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)y | (uintptr_t)tape |
+                           (uintptr_t)z | (uintptr_t)norm_weight) % 16) == 0;
   const bool chunk = fast && !g_per_dk && state_dtype == DFLASH_FP32 && T <= 16 && aligned16 && !no_chunk;
+  bool norm_done = false;
   if (chunk) {
     const size_t lds = kChunkLdsFloats * sizeof(float);
-    if (in_dtype == DFLASH_FP32) {
-      hipLaunchKernelGGL(gdn_forward_chunk_128<true>, grid, block, lds, s, a);
+    const bool wide = in_dtype == DFLASH_FP32;
+    if (z) {
+      if (wide) hipLaunchKernelGGL((gdn_forward_chunk_128<true, true>), grid, block, lds, s, a);
+      else hipLaunchKernelGGL((gdn_forward_chunk_128<false, true>), grid, block, lds, s, a);
+      norm_done = true;
     } else {
-      hipLaunchKernelGGL(gdn_forward_chunk_128<false>, grid, block, lds, s, a);
+      if (wide) hipLaunchKernelGGL((gdn_forward_chunk_128<true, false>), grid, block, lds, s, a);
+      else hipLaunchKernelGGL((gdn_forward_chunk_128<false, false>), grid, block, lds, s, a);
     }
   } else if (fast) {
     if (g_per_dk) {
@@ -669,5 +793,33 @@ extern "C" int dflash_gdn_forward_tape(const void* q, const void* k, const void*
     hipLaunchKernelGGL(gdn_forward_generic, grid, block, 0, s, a);
   }
   DFLASH_HIP_OK(hipGetLastError());
+  if (z && !norm_done)  // the other kernels leave the recurrence's output in y: normalise it in place
+    return dflash_gdn_gated_norm(y, z, norm_weight, y, (long long)slots * T * Hv, Dv, in_dtype, weight_dtype, eps,
+                                 stream);
   return DFLASH_OK;
+}
+
+}  // namespace
+}  // namespace dflash
+
+extern "C" int dflash_gdn_forward_tape(const void* q, const void* k, const void* v, const void* g,
+                                       const void* beta, const void* state_in, void* state_out,
+                                       void* y, float* tape, const uint8_t* mask, int slots, int T,
+                                       int Hk, int Hv, int Dk, int Dv, int in_dtype, int g_dtype,
+                                       int beta_dtype, int state_dtype, int g_per_dk, void* stream) {
+  return dflash::gdn_forward_launch("dflash_gdn_forward_tape", q, k, v, g, beta, state_in, state_out, y, tape, mask,
+                                    nullptr, nullptr, DFLASH_FP32, 0.f, slots, T, Hk, Hv, Dk, Dv, in_dtype, g_dtype,
+                                    beta_dtype, state_dtype, g_per_dk, stream);
+}
+
+extern "C" int dflash_gdn_forward_tape_norm(const void* q, const void* k, const void* v, const void* g,
+                                            const void* beta, const void* state_in, void* state_out,
+                                            const void* z, const void* norm_weight, void* out, float* tape,
+                                            const uint8_t* mask, int slots, int T, int Hk, int Hv, int Dk, int Dv,
+                                            int in_dtype, int g_dtype, int beta_dtype, int state_dtype,
+                                            int weight_dtype, int g_per_dk, float eps, void* stream) {
+  DFLASH_REQUIRE(z && norm_weight, DFLASH_ERR_ARG, "dflash_gdn_forward_tape_norm: null z or norm weight");
+  return dflash::gdn_forward_launch("dflash_gdn_forward_tape_norm", q, k, v, g, beta, state_in, state_out, out, tape,
+                                    mask, z, norm_weight, weight_dtype, eps, slots, T, Hk, Hv, Dk, Dv, in_dtype,
+                                    g_dtype, beta_dtype, state_dtype, g_per_dk, stream);
 }

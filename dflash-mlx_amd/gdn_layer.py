@@ -21,13 +21,14 @@ out_proj); its own ``forward`` is the plain, non-speculative call.
 """
 from __future__ import annotations
 
+import os
 from typing import Any, Optional, Tuple
 
 import torch
 import torch.nn as nn
 
 from . import _native
-from .kernels import _DTYPE_CODE, gated_delta_kernel_with_tape
+from .kernels import _DTYPE_CODE, fused_output_norm_applies, gated_delta_kernel_with_tape
 from .recurrent_rollback_cache import RecurrentRollbackCache
 
 _EXACT_SMALL_PROJ_PAD_M = 16
@@ -235,14 +236,20 @@ def _gdn_call(self, inputs: torch.Tensor, mask: Optional[torch.Tensor], cache: O
     state = cache[1] if cache is not None else None
     if state is None:
         state = torch.zeros((B, self.num_v_heads, self.head_v_dim, self.head_k_dim), dtype=q.dtype, device=q.device)
-    out, state, innovation_tape = gated_delta_kernel_with_tape(q, k, v, g, beta, state, mask)
+    # the layer's output norm rides on the recurrence's launch where the kernel takes it
+    norm = self.norm
+    fused = (isinstance(norm, RMSNormGated) and os.environ.get("DFLASH_GDN_FUSED_NORM", "1") != "0" and
+             fused_output_norm_applies(q, v, state, z, norm.weight))
+    out, state, innovation_tape = gated_delta_kernel_with_tape(
+        q, k, v, g, beta, state, mask, output_norm=(z, norm.weight, norm.eps) if fused else None)
     if record:
         if mask is not None:
             qkv = torch.where(mask.to(torch.bool)[..., None], qkv, torch.zeros_like(qkv))
         cache.record_tape(tape=innovation_tape, k=k, g=g, qkv=qkv)
     if cache is not None:
         cache[1] = state
-    out = self.norm(out, z)
+    if not fused:
+        out = self.norm(out, z)
     return self.out_proj(out.reshape(B, S, -1))
 
 

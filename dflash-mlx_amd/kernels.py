@@ -77,14 +77,30 @@ def _gated_delta_ops_with_tape(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor
     return torch.stack(ys, dim=1), state, torch.stack(tape, dim=1)
 
 
+def fused_output_norm_applies(q: torch.Tensor, v: torch.Tensor, state: torch.Tensor, z: torch.Tensor,
+                              weight: torch.Tensor) -> bool:
+    """Whether ``gated_delta_kernel_with_tape(..., output_norm=...)`` can be asked for: device
+    tensors of the kernels' dtypes, z shaped like v, rows of a multiple of 64 up to 256."""
+    dv = int(v.shape[-1])
+    return (state.is_cuda and z.shape == v.shape and z.dtype == q.dtype == v.dtype and weight.dtype in _DTYPE_CODE and
+            q.dtype in _DTYPE_CODE and int(weight.numel()) == dv and dv % 64 == 0 and dv <= 256 and
+            int(q.shape[-1]) >= 32 and int(q.shape[-1]) % 32 == 0 and int(q.shape[1]) > 0)
+
+
 def gated_delta_kernel_with_tape(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor,
                                  beta: torch.Tensor, state: torch.Tensor,
-                                 mask: Optional[torch.Tensor] = None):
+                                 mask: Optional[torch.Tensor] = None, *,
+                                 output_norm: Optional[tuple] = None):
     """GatedDeltaNet forward over a block that records the innovation tape (mirror of
     dflash_mlx/kernels.py:176-224): ``(y, state_out, tape)`` with y in q's dtype, the state in
     its own dtype and an fp32 tape.  Device tensors with Dk a multiple of 32 go to the gfx950
     kernel behind ``dflash_gdn_forward_tape``; host tensors and other shapes take the array
-    ops, as the reference does without its kernel."""
+    ops, as the reference does without its kernel.
+
+    ``output_norm=(z, weight, eps)`` (no counterpart in the reference, which calls the layer's
+    norm right after): the first result is then ``silu(z) * rms_norm(y, weight, eps)``, computed
+    by the same launch (``dflash_gdn_forward_tape_norm``); only for inputs the kernel takes -
+    callers check ``fused_output_norm_applies`` first."""
     B, T, hk, dk = (int(d) for d in k.shape)
     hv, dv = int(v.shape[2]), int(v.shape[3])
     if g.ndim not in (3, 4):
@@ -105,6 +121,19 @@ def gated_delta_kernel_with_tape(q: torch.Tensor, k: torch.Tensor, v: torch.Tens
     if mask is not None:
         mask = mask.to(torch.uint8).contiguous()
         mask_ptr = mask.data_ptr()
+    if output_norm is not None:
+        z, weight, eps = output_norm
+        if not fused_output_norm_applies(q, v, state, z, weight):
+            raise ValueError("output_norm: shapes or dtypes the fused kernel does not take")
+        z_c, w_c = z.contiguous(), weight.contiguous()
+        rc = lib.dflash_gdn_forward_tape_norm(
+            q_c.data_ptr(), k_c.data_ptr(), v_c.data_ptr(), g_c.data_ptr(), beta_c.data_ptr(),
+            state_c.data_ptr(), state_out.data_ptr(), z_c.data_ptr(), w_c.data_ptr(), y.data_ptr(), tape.data_ptr(),
+            mask_ptr, B, T, hk, hv, dk, dv, _DTYPE_CODE[q.dtype], _DTYPE_CODE[g.dtype], _DTYPE_CODE[beta.dtype],
+            _DTYPE_CODE[state.dtype], _DTYPE_CODE[weight.dtype], 1 if g.ndim == 4 else 0, float(eps),
+            torch.cuda.current_stream(q.device).cuda_stream)
+        _native.check(rc, "dflash_gdn_forward_tape_norm")
+        return y, state_out, tape
     rc = lib.dflash_gdn_forward_tape(
         q_c.data_ptr(), k_c.data_ptr(), v_c.data_ptr(), g_c.data_ptr(), beta_c.data_ptr(),
         state_c.data_ptr(), state_out.data_ptr(), y.data_ptr(), tape.data_ptr(), mask_ptr,

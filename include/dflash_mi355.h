@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 6
+#define DFLASH_ABI_VERSION 7
 
 enum {
   DFLASH_OK = 0,
@@ -168,6 +168,22 @@ int dflash_gdn_forward_tape(const void* q, const void* k, const void* v, const v
                             float* tape, const uint8_t* mask, int slots, int T, int Hk, int Hv,
                             int Dk, int Dv, int in_dtype, int g_dtype, int beta_dtype,
                             int state_dtype, int g_per_dk, void* stream);
+
+/*
+ * The same forward with the layer's gated output norm applied to its result: what
+ * dflash_mlx/runtime.py:441-448 computes with two calls (`gated_delta_kernel_with_tape`, then
+ * `self.norm(out, z)`), in one launch where the block kernel applies (else the forward into
+ * `out` followed by dflash_gdn_gated_norm in place).
+ *     out = silu(z) * rms_norm(y, norm_weight, eps),  y the recurrence's output rounded to in_dtype
+ *   z, out       [slots, T, Hv, Dv] in_dtype;  norm_weight [Dv] weight_dtype
+ * Dv a multiple of 64 up to 256.  Everything else as for dflash_gdn_forward_tape.
+ */
+int dflash_gdn_forward_tape_norm(const void* q, const void* k, const void* v, const void* g,
+                                 const void* beta, const void* state_in, void* state_out,
+                                 const void* z, const void* norm_weight, void* out, float* tape,
+                                 const uint8_t* mask, int slots, int T, int Hk, int Hv, int Dk, int Dv,
+                                 int in_dtype, int g_dtype, int beta_dtype, int state_dtype,
+                                 int weight_dtype, int g_per_dk, float eps, void* stream);
 
 /*
  * GatedDeltaNet layer, everything between the input projections and the recurrence, in one

@@ -9,8 +9,9 @@ import numpy as np
 import pytest
 import torch
 
-from dflash_mlx_amd.kernels import (_gated_delta_ops_with_tape, gated_delta_kernel_with_tape,
-                                    tape_replay_kernel)
+from dflash_mlx_amd.gdn_layer import gated_norm
+from dflash_mlx_amd.kernels import (_gated_delta_ops_with_tape, fused_output_norm_applies,
+                                    gated_delta_kernel_with_tape, tape_replay_kernel)
 from oracle import dflash_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -210,3 +211,41 @@ def test_speculative_cycle_through_the_rollback_cache(native_lib, accepted):
     want_conv = torch.cat([conv0, qkv], dim=1)[:, n:n + 3]
     assert torch.equal(cache[0], want_conv)
     assert not cache._armed and cache._tape is None
+
+
+@pytest.mark.parametrize("dtype,wdtype,state_dtype,T", [(torch.bfloat16, torch.bfloat16, torch.float32, 16),
+                                                        (torch.float16, torch.float32, torch.float32, 16),
+                                                        (torch.float32, torch.float32, torch.float32, 16),
+                                                        (torch.bfloat16, torch.bfloat16, torch.float32, 5),
+                                                        (torch.bfloat16, torch.bfloat16, torch.bfloat16, 16)])
+def test_output_norm_in_the_same_launch(native_lib, dtype, wdtype, state_dtype, T):
+    """silu(z) * rms_norm(y, weight) computed by the recurrence's launch: state and tape are those
+    of the plain call bit for bit, and the output is the norm operator applied to the plain
+    call's y - up to one rounding of the array dtype where the two add the squares in a different
+    order (block kernel), exactly where the entry point runs the two kernels itself (bf16 state)."""
+    args = [t.to(DEV) for t in _case(B=2, T=T, Hk=2, Hv=4, seed=40 + T, dtype=dtype, state_dtype=state_dtype)]
+    g = torch.Generator().manual_seed(7)
+    z = torch.randn((2, T, 4, 128), generator=g).to(dtype).to(DEV)
+    weight = (1 + 0.2 * torch.randn(128, generator=g)).to(wdtype).to(DEV)
+    mask = torch.ones((2, T), dtype=torch.bool)
+    mask[1, T // 2] = False
+    for m in (None, mask.to(DEV)):
+        assert fused_output_norm_applies(args[0], args[2], args[5], z, weight)
+        y, s_plain, tape_plain = gated_delta_kernel_with_tape(*args, mask=m)
+        out, s_fused, tape_fused = gated_delta_kernel_with_tape(*args, mask=m, output_norm=(z, weight, 1e-6))
+        torch.cuda.synchronize()
+        assert torch.equal(s_plain, s_fused) and torch.equal(tape_plain, tape_fused)
+        want = gated_norm(y, z, weight, 1e-6)
+        if state_dtype != torch.float32:
+            assert torch.equal(out, want)
+        else:
+            ulp = {torch.bfloat16: 2 ** -7, torch.float16: 2 ** -10, torch.float32: 2 ** -22}[dtype]
+            w64, o64 = want.double(), out.double()
+            assert bool(((o64 - w64).abs() <= 2 * ulp * w64.abs() + 1e-6).all())
+            assert float((o64 - w64).norm() / w64.norm()) <= ulp / 4
+        if m is not None:
+            assert float(out[1, T // 2].abs().max()) == 0.0   # a masked step's output is zero, normed or not
+    # a z of another shape is not taken
+    assert not fused_output_norm_applies(args[0], args[2], args[5], z[..., :64], weight)
+    with pytest.raises(ValueError):
+        gated_delta_kernel_with_tape(*args, output_norm=(z[..., :64], weight, 1e-6))
