@@ -199,6 +199,38 @@ def test_linearity_full_size(verify_env, native_lib):
     assert resid <= 4 * 2 ** -8 * max(y1.abs().max().item(), y2.abs().max().item())
 
 
+def test_random_shapes_repeat_bit_for_bit_and_stay_close(verify_env, native_lib):
+    """Shapes drawn at random (every split of the rows and of K over the workgroups comes up):
+    each call gives the same bits when repeated at once and again later, after other shapes
+    have used the workspace, and stays within the bf16 bar of an fp32 product on the device."""
+    gen = torch.Generator(device=DEV).manual_seed(seed_for(0, 77))
+    draw = torch.Generator().manual_seed(seed_for(0, 78))
+    pick = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=draw))
+    shifts = torch.arange(8, device=DEV, dtype=torch.int32) * 4
+    earlier = []
+    for i in range(48):
+        K = 512 * pick(1, 34)
+        N = 16 * pick(1, 1200) if i % 3 else 64 * pick(1, 300)
+        dtype = torch.float16 if i % 4 == 0 else torch.bfloat16
+        x = torch.randn((16, K), generator=gen, device=DEV).to(dtype)
+        w = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 8), generator=gen, device=DEV).to(torch.int32)
+        s = (torch.randn((N, K // 64), generator=gen, device=DEV).abs() * 0.02 + 1e-4).to(dtype)
+        b = (-8 * s.float() + 0.01 * torch.randn((N, K // 64), generator=gen, device=DEV)).to(dtype)
+        first, second = (VQ.verify_matmul(x, w, s, b, group_size=64, bits=4).clone() for _ in range(2))
+        codes = ((w.unsqueeze(-1) >> shifts) & 15).reshape(N, K).float()
+        dense = codes * s.float().repeat_interleave(64, 1) + b.float().repeat_interleave(64, 1)
+        exact = x.float() @ dense.t()
+        assert torch.equal(first, second), f"K={K} N={N} {dtype}: two calls in a row differ"
+        rel = ((first.float() - exact).norm() / exact.norm()).item()
+        assert rel <= 5e-3, f"K={K} N={N} {dtype}: rel-L2 {rel:.3g}"
+        earlier.append((K, N, x, w, s, b, first))
+        if len(earlier) == 8:
+            again = [VQ.verify_matmul(e[2], e[3], e[4], e[5], group_size=64, bits=4).clone() for e in earlier]
+            for e, y in zip(earlier, again):
+                assert torch.equal(y, e[6]), f"K={e[0]} N={e[1]}: differs after other shapes ran"
+            earlier = []
+
+
 def test_leading_shapes_and_stock_fallbacks_on_device(verify_env, native_lib):
     case = make_qmm_case(512, 64, 41).to(DEV)
     y = VQ.verify_matmul(case.x, case.w, case.scales, case.biases)
