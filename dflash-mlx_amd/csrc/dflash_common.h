@@ -28,6 +28,15 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
     }                                                                                    \
   } while (0)
 
+// Index of the current device for per-device caches (function attributes, CU counts); devices
+// beyond the table share its last entry, which is then refreshed on every call.
+constexpr int kMaxDevices = 16;
+inline int current_device_slot() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) dev = 0;
+  return dev < kMaxDevices ? dev : kMaxDevices - 1;
+}
+
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;

@@ -923,15 +923,15 @@ arrive:
 namespace dflash {
 
 int qmm_stream_grid() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256;
-    cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-    if (cus > 1024) cus = 1024;
+  static int cus[kMaxDevices] = {};
+  const int slot = current_device_slot();
+  if (cus[slot] == 0 || slot == kMaxDevices - 1) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 256;
+    cus[slot] = n > 0 ? (n > 1024 ? 1024 : n) : 256;
   }
-  return cus;
+  return cus[slot];
 }
 
 bool qmm_stream_eligible(int K, int N, int group_size) {
@@ -979,11 +979,13 @@ int launch_stream(stream::Params& p, bool gather, int grid, int act_dtype, int s
   const bool chunk4 = p.K % (kUnitK * 4) == 0;
   const void* fn = gather ? stream_kernel_for<true>(a16, s16, chunk4) : stream_kernel_for<false>(a16, s16, chunk4);
   const int lds_bytes = gather ? kLdsBytesGather : kLdsBytes;
-  static bool attr_set[16] = {};
+  // the attribute belongs to the device's copy of the kernel: once per device and kernel
+  static bool attr_set[kMaxDevices][16] = {};
   const int idx = (gather ? 8 : 0) + (chunk4 ? 4 : 0) + (a16 ? 2 : 0) + (s16 ? 1 : 0);
-  if (!attr_set[idx]) {
+  const int slot = current_device_slot();
+  if (!attr_set[slot][idx] || slot == kMaxDevices - 1) {
     DFLASH_HIP_OK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
-    attr_set[idx] = true;
+    attr_set[slot][idx] = true;
   }
   void* args[] = {&p};
   DFLASH_HIP_OK(hipLaunchKernel(fn, dim3(grid), dim3(kThreads), args, lds_bytes, stream));

@@ -441,11 +441,13 @@ extern "C" int dflash_sdpa_q16(const void* q, const void* k, const void* v, cons
   const bool masked = mask != nullptr;
   const int ics = cs == 1 ? 0 : cs == 2 ? 1 : 2;
   const void* fn = table[D == 256][f16][masked][ics];
-  static bool attr_set[24] = {};
+  // the attribute belongs to the device's copy of the kernel: once per device and kernel
+  static bool attr_set[kMaxDevices][24] = {};
   const int idx = (((D == 256) * 2 + f16) * 2 + masked) * 3 + ics;
-  if (!attr_set[idx]) {
+  const int slot = current_device_slot();
+  if (!attr_set[slot][idx] || slot == kMaxDevices - 1) {
     DFLASH_HIP_OK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-    attr_set[idx] = true;
+    attr_set[slot][idx] = true;
   }
   void* args[] = {&a};
   DFLASH_HIP_OK(hipLaunchKernel(fn, dim3((unsigned)(B * Hk * a.splits)), dim3(kThreads), args, lds_bytes, s));
