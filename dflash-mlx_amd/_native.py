@@ -111,6 +111,18 @@ def is_built() -> bool:
     return os.path.exists(LIB_PATH)
 
 
+def raw_stream(device) -> int:
+    """Handle of the current stream of ``device`` (torch's Stream object costs microseconds per
+    call to build; the handle is all the C ABI takes)."""
+    import torch
+
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    try:
+        return torch._C._cuda_getCurrentRawStream(index)
+    except AttributeError:  # a torch without the raw accessor
+        return torch.cuda.current_stream(device).cuda_stream
+
+
 def check(rc: int, what: str) -> None:
     if rc != 0:
         msg = lib().dflash_last_error().decode("utf-8", "replace")

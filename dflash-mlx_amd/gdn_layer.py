@@ -129,7 +129,7 @@ def gdn_prepare(qkv: torch.Tensor, conv_state: Optional[torch.Tensor], conv_w: t
         A_log.contiguous().data_ptr(), dt_bias.contiguous().data_ptr(),
         None if mask_c is None else mask_c.data_ptr(), conv_next.data_ptr(), q.data_ptr(), k.data_ptr(),
         v.data_ptr(), g.data_ptr(), beta.data_ptr(), B, S, Hk, Hv, Dk, Dv, K, _DTYPE_CODE[dt],
-        _DTYPE_CODE[A_log.dtype], float(eps), torch.cuda.current_stream(dev).cuda_stream)
+        _DTYPE_CODE[A_log.dtype], float(eps), _native.raw_stream(dev))
     _native.check(rc, "dflash_gdn_prepare")
     return conv_next, q, k, v, g, beta
 
@@ -144,7 +144,7 @@ def gated_norm(x: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: floa
     y = torch.empty_like(x_c)
     rc = lib.dflash_gdn_gated_norm(x_c.data_ptr(), z_c.data_ptr(), w_c.data_ptr(), y.data_ptr(),
                                    x_c.numel() // D, D, _DTYPE_CODE[x.dtype], _DTYPE_CODE[weight.dtype],
-                                   float(eps), torch.cuda.current_stream(x.device).cuda_stream)
+                                   float(eps), _native.raw_stream(x.device))
     _native.check(rc, "dflash_gdn_gated_norm")
     return y
 

@@ -131,7 +131,7 @@ def gated_delta_kernel_with_tape(q: torch.Tensor, k: torch.Tensor, v: torch.Tens
             state_c.data_ptr(), state_out.data_ptr(), z_c.data_ptr(), w_c.data_ptr(), y.data_ptr(), tape.data_ptr(),
             mask_ptr, B, T, hk, hv, dk, dv, _DTYPE_CODE[q.dtype], _DTYPE_CODE[g.dtype], _DTYPE_CODE[beta.dtype],
             _DTYPE_CODE[state.dtype], _DTYPE_CODE[weight.dtype], 1 if g.ndim == 4 else 0, float(eps),
-            torch.cuda.current_stream(q.device).cuda_stream)
+            _native.raw_stream(q.device))
         _native.check(rc, "dflash_gdn_forward_tape_norm")
         return y, state_out, tape
     rc = lib.dflash_gdn_forward_tape(
@@ -139,7 +139,7 @@ def gated_delta_kernel_with_tape(q: torch.Tensor, k: torch.Tensor, v: torch.Tens
         state_c.data_ptr(), state_out.data_ptr(), y.data_ptr(), tape.data_ptr(), mask_ptr,
         B, T, hk, hv, dk, dv, _DTYPE_CODE[q.dtype], _DTYPE_CODE[g.dtype], _DTYPE_CODE[beta.dtype],
         _DTYPE_CODE[state.dtype], 1 if g.ndim == 4 else 0,
-        torch.cuda.current_stream(q.device).cuda_stream)
+        _native.raw_stream(q.device))
     _native.check(rc, "dflash_gdn_forward_tape")
     return y, state_out, tape
 
@@ -196,7 +196,7 @@ def replay_launch(tape: torch.Tensor, k: torch.Tensor, g: torch.Tensor, state_in
     if mask is not None:
         mask = mask.to(torch.uint8).contiguous()
         mask_ptr = mask.data_ptr()
-    stream = torch.cuda.current_stream(state_in.device).cuda_stream
+    stream = _native.raw_stream(state_in.device)
     rc = lib.dflash_tape_replay(
         tape.data_ptr(), k.data_ptr(), g.data_ptr(), state_in.data_ptr(), state_out.data_ptr(),
         steps_dev, steps_host, mask_ptr, slots, T_alloc, Hk, Hv, Dk, Dv,
@@ -244,7 +244,7 @@ _SDPA_WORKSPACE: dict = {}
 
 def _sdpa_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     """Partial results of the key ranges, one buffer per device and stream, grown on demand."""
-    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    key = (device, _native.raw_stream(device))
     buf = _SDPA_WORKSPACE.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
@@ -298,6 +298,6 @@ def batched_sdpa_2pass_exact(queries: torch.Tensor, keys: torch.Tensor, values: 
         None if mask_tensor is None else mask_tensor.data_ptr(), out.data_ptr(),
         None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), bsz, hq, hk, n_kv, d,
         keys.stride(0), keys.stride(1), keys.stride(2), values.stride(0), values.stride(1), values.stride(2),
-        float(scale), _DTYPE_CODE[queries.dtype], torch.cuda.current_stream(queries.device).cuda_stream)
+        float(scale), _DTYPE_CODE[queries.dtype], _native.raw_stream(queries.device))
     _native.check(rc, "dflash_sdpa_q16")
     return out

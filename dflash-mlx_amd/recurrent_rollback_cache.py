@@ -51,7 +51,7 @@ def conv_state_rebuild(conv_prev: Optional[torch.Tensor], qkv: torch.Tensor,
         steps_dev = steps.data_ptr()
     else:
         steps_host = int(steps)
-    stream = torch.cuda.current_stream(qkv.device).cuda_stream
+    stream = _native.raw_stream(qkv.device)
     rc = _native.lib().dflash_conv_state_rebuild(prev_ptr, qkv.data_ptr(), out.data_ptr(), steps_dev,
                                                  steps_host, slots, T, keep, C, qkv.element_size(),
                                                  stream)

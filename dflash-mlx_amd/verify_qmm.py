@@ -74,6 +74,10 @@ def _should_use_verify(x: torch.Tensor, group_size: int, bits: int, transpose: b
 _WORKSPACES: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
+# what dflash_qmm_m16_workspace_bytes answered per (K, N, group size, variant, k_parts, kernel)
+_WORKSPACE_BYTES: Dict[Tuple[int, int, int, int, int, int], int] = {}
+
+
 def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
     ws = _WORKSPACES.get(key)
@@ -93,10 +97,13 @@ def _launch(x2: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: tor
     if scales.dtype not in _DTYPE_CODE or biases.dtype != scales.dtype:
         raise TypeError(f"scales/biases must both be bf16 or fp16, got {scales.dtype}/{biases.dtype}")
     y = torch.empty((16, N), dtype=x2.dtype, device=x2.device)
-    stream = torch.cuda.current_stream(x2.device).cuda_stream
+    stream = _native.raw_stream(x2.device)
     vcode = _VARIANT_CODE[variant]
     kernel = _kernel_select()
-    need = lib.dflash_qmm_m16_workspace_bytes(K, N, group_size, vcode, k_parts, kernel)
+    key = (K, N, group_size, vcode, k_parts, kernel)
+    need = _WORKSPACE_BYTES.get(key)
+    if need is None:
+        need = _WORKSPACE_BYTES[key] = int(lib.dflash_qmm_m16_workspace_bytes(*key))
     ws_ptr, ws_bytes = None, 0
     if need:
         ws = _workspace(x2.device, stream, need)
@@ -198,7 +205,7 @@ def gather_qmm(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: t
     if ids.numel() != P:
         raise ValueError("one expert id per row of x is required")
     y = torch.empty((P, N), dtype=x2.dtype, device=x2.device)
-    stream = torch.cuda.current_stream(x2.device).cuda_stream
+    stream = _native.raw_stream(x2.device)
     # DFLASH_QMM_KERNEL=tile keeps the streaming kernel out of the gathered form as well
     need = 0 if _kernel_select() == _native.QMM_KERNEL_TILE else \
         lib.dflash_qmm_m16_gather_workspace_bytes(P, K, N, E, group_size)
