@@ -231,6 +231,32 @@ def test_random_shapes_repeat_bit_for_bit_and_stay_close(verify_env, native_lib)
             earlier = []
 
 
+@pytest.mark.parametrize("K,N,rows", [(5120, 151936, 16), (2048, 262144, 5)])
+def test_vocabulary_sized_projection(verify_env, native_lib, kernel_mode, K, N, rows):
+    """An output head: more rows of W than any layer projection has (1187 and 2048 row blocks).
+    16 rows through verify_matmul, fewer through the stock operator's small-M route."""
+    if kernel_mode == "tile":
+        pytest.skip("one kernel is enough at this size")
+    gen = torch.Generator(device=DEV).manual_seed(seed_for(0, 91))
+    x = torch.randn((rows, K), generator=gen, device=DEV).to(torch.bfloat16)
+    w = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 8), generator=gen, device=DEV).to(torch.int32)
+    s = (torch.randn((N, K // 64), generator=gen, device=DEV).abs() * 0.02 + 1e-4).to(torch.bfloat16)
+    b = (-8 * s.float()).to(torch.bfloat16)
+    run = (lambda: VQ.verify_matmul(x, w, s, b, group_size=64, bits=4)) if rows == 16 else \
+        (lambda: stock_matmul(x, w, s, b, transpose=True, group_size=64, bits=4))
+    y = run()
+    assert y.shape == (rows, N) and torch.equal(y, run())
+    shifts = torch.arange(8, device=DEV, dtype=torch.int32) * 4
+    exact = torch.empty((rows, N), dtype=torch.float32, device=DEV)
+    for n0 in range(0, N, 16384):
+        rows_w = slice(n0, min(n0 + 16384, N))
+        codes = ((w[rows_w].unsqueeze(-1) >> shifts) & 15).reshape(-1, K).float()
+        dense = codes * s[rows_w].float().repeat_interleave(64, 1) + b[rows_w].float().repeat_interleave(64, 1)
+        exact[:, rows_w] = x.float() @ dense.t()
+    rel = ((y.float() - exact).norm() / exact.norm()).item()
+    assert rel <= 5e-3, rel
+
+
 def test_leading_shapes_and_stock_fallbacks_on_device(verify_env, native_lib):
     case = make_qmm_case(512, 64, 41).to(DEV)
     y = VQ.verify_matmul(case.x, case.w, case.scales, case.biases)
