@@ -34,7 +34,7 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 # HBM bytes per launch of the qmm kernel on each stack (mean over its launches), from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file scaled by the same counters'
 # reading for a 1 GiB copy (x2.000 / x1.000); None where not measured for the current kernel.
-MEASURED_TRAFFIC_BYTES = {"27b": 44.99e6, "9b": None}
+MEASURED_TRAFFIC_BYTES = {"27b": 44.32e6, "9b": None}
 
 
 def log(*a):
