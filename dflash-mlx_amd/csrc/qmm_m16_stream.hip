@@ -10,9 +10,11 @@
 //
 //  * The weight matrix is cut into units of 128 rows x 256 k (16 KiB of codes plus the
 //    8 KiB slice of x they multiply; scales/biases come per chunk of four units).  Units
-//    are numbered row-block-major and divided EVENLY among a persistent grid of one
-//    workgroup per CU: every CU streams the same number of bytes (+-1 unit) whatever N and
-//    K are, fills its load pipeline once, and there is no tail of half-empty rounds.
+//    are numbered row-block-major and divided EVENLY among a persistent grid of at most one
+//    workgroup per CU: every workgroup streams the same number of bytes (+-1 unit) whatever N
+//    and K are, fills its load pipeline once, and there is no tail of half-empty rounds.  The
+//    host prefers a grid that is a multiple of the number of row blocks when that costs at most
+//    two units of range length (qmm_stream_pick_grid): no range then crosses a row block.
 //  * A workgroup is 8 worker waves plus 4 loader waves.  Loaders do nothing but move units
 //    global -> LDS with 16-byte direct loads (no VGPR staging; each instruction moves
 //    128-byte row segments of 8 rows) into a ring of slots, a few units ahead of the
