@@ -89,19 +89,9 @@ def time_region(fn, steps: int):
 def capture(fn):
     """Run ``fn`` once on a side stream (so that every lazily created buffer exists), then
     record it into a HIP graph on that stream.  Returns (graph, outputs of the capture)."""
-    import torch
+    from dflash_mlx_amd.graph_replay import record
 
-    graph = torch.cuda.CUDAGraph()
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        fn()
-        side.synchronize()
-        with torch.cuda.graph(graph, stream=side):
-            out = fn()
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    return graph, out
+    return record(fn)
 
 
 def bench_qmm_stack(stack: str, steps: int, warmup: int, device: str, join_gate_up: bool = False):

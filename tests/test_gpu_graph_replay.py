@@ -11,6 +11,7 @@ import torch
 from dflash_mlx_amd import kernels as K
 from dflash_mlx_amd import verify_qmm as VQ
 from dflash_mlx_amd.gdn_layer import gated_norm, gdn_prepare
+from dflash_mlx_amd.graph_replay import record
 from dflash_mlx_amd.workloads import make_qmm_case, make_replay_case, seed_for
 
 pytestmark = pytest.mark.gpu
@@ -18,17 +19,7 @@ DEV = "cuda:0"
 
 
 def _capture(fn):
-    graph = torch.cuda.CUDAGraph()
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        fn()  # lazily created workspaces exist before the capture
-        side.synchronize()
-        with torch.cuda.graph(graph, stream=side):
-            out = fn()
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    return graph, out
+    return record(fn)
 
 
 def _replays_match(graph, captured, eager_fn, refill, rounds=3):
