@@ -166,16 +166,21 @@ def bench_single_call(device: str, launches: int = 200):
     return out
 
 
-def bench_moe(device: str, steps: int, warmup: int, layers: int = 40, join_gate_up: bool = False):
+def bench_moe(device: str, steps: int, warmup: int, layers: int = 40, join_gate_up: bool = False,
+              shared_as_expert: bool = False):
     """config[4]: MoE-shaped verify step at M=16 - 256 experts of intermediate 512 (gate/up
     2048->512, down 512->2048), top-8 routing, gathered per-expert qmm, plus a shared expert
     through verify_matmul; `layers` layers replayed from a HIP graph.  Algorithmic bytes
     count the weights of the experts the seeded routing actually touches.  ``join_gate_up``:
     gate and up, which read the same rows, laid end to end per expert (and for the shared
-    expert) and served by one launch each - four launches per layer instead of six."""
+    expert) and served by one launch each - four launches per layer instead of six.
+    ``shared_as_expert`` (with ``join_gate_up``): the shared expert, which has the shape of a
+    routed one, stored as expert 256 and its 16 rows appended to the 128 routed pairs - two
+    launches per layer, over the same weight bytes."""
     import torch
 
-    from dflash_mlx_amd.verify_qmm import gather_qmm, join_expert_projections, verify_matmul
+    from dflash_mlx_amd.verify_qmm import (append_shared_expert, gather_qmm, join_expert_projections,
+                                           shared_expert_rows, verify_matmul)
     from dflash_mlx_amd.workloads import MoeCase, QmmCase
     from dflash_mlx_amd.workloads import make_moe_case, make_qmm_case, qmm_algorithmic_bytes, seed_for
 
@@ -196,7 +201,17 @@ def bench_moe(device: str, steps: int, warmup: int, layers: int = 40, join_gate_
             sg, su, sd = shared
             shared_gu = QmmCase(sg.x, torch.cat([sg.w, su.w]), torch.cat([sg.scales, su.scales]),
                                 torch.cat([sg.biases, su.biases]), 64)
-            calls.append(((gate_up, down), (shared_gu, sd)))
+            if shared_as_expert:
+                both = []
+                for routed, sh in ((gate_up, shared_gu), (down, sd)):
+                    (w, sc, bi), sid = append_shared_expert((routed.w, routed.scales, routed.biases),
+                                                            (sh.w, sh.scales, sh.biases))
+                    x, ids = shared_expert_rows(routed.x, routed.expert_ids, sh.x, sid)
+                    both.append(MoeCase(x, ids, w, sc, bi, 64))
+                calls.append((tuple(both), ()))
+                del routed, sh, gate_up, shared_gu, sd
+            else:
+                calls.append(((gate_up, down), (shared_gu, sd)))
             del gate, up, sg, su
         else:
             calls.append(((gate, up, down), tuple(shared)))
@@ -596,6 +611,10 @@ def main() -> int:
         mj = bench_moe(device, args.steps, args.warmup, join_gate_up=True)
         extra["moe_35b_a3b_stack_gate_up_in_one_launch"] = {k: (round(v, 4) if isinstance(v, float) else v)
                                                             for k, v in mj.items()}
+        ms = bench_moe(device, args.steps, args.warmup, join_gate_up=True, shared_as_expert=True)
+        log(f"[bench] moe stack, shared expert stored as expert 256: {ms['ms_per_step']:.3f} ms/step")
+        extra["moe_35b_a3b_stack_shared_expert_in_the_gathered_launch"] = {
+            k: (round(v, 4) if isinstance(v, float) else v) for k, v in ms.items()}
         rp = bench_replay(device, args.steps, args.warmup)
         extra["gdn_tape_replay"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in rp.items()}
         fw = bench_gdn_forward(device, args.steps, args.warmup)

@@ -236,3 +236,35 @@ def join_expert_projections(*projections):
         bounds.append((row, row + int(p[0].shape[1])))
         row += int(p[0].shape[1])
     return (w, scales, biases), bounds
+
+
+def append_shared_expert(experts, shared):
+    """Stores an always-active shared expert behind the routed experts of the same shape: from
+    ``(w [E, N, K/8], scales, biases)`` and the shared expert's ``(w [N, K/8], scales, biases)`` to
+    one ``(w [E+1, N, K/8], scales, biases)`` and the shared expert's id ``E``.  With
+    ``shared_expert_rows`` one ``gather_qmm`` launch then serves the routed pairs and the shared
+    expert, instead of a gathered launch plus a ``verify_matmul`` launch per projection.  Done
+    once when the weights are loaded; no counterpart in the reference (its shared expert is a
+    plain linear next to mlx_lm's switch layers)."""
+    (w, scales, biases), (sw, ss, sb) = experts, shared
+    if tuple(sw.shape) != tuple(w.shape[1:]) or tuple(ss.shape) != tuple(scales.shape[1:]) \
+            or tuple(sb.shape) != tuple(biases.shape[1:]):
+        raise ValueError("the shared expert must have the shape of one routed expert")
+    if sw.dtype != w.dtype or ss.dtype != scales.dtype or sb.dtype != biases.dtype:
+        raise ValueError("the shared expert must have the dtypes of the routed experts")
+    joined = tuple(torch.cat([a, b.unsqueeze(0)], dim=0).contiguous()
+                   for a, b in ((w, sw), (scales, ss), (biases, sb)))
+    return joined, int(w.shape[0])
+
+
+def shared_expert_rows(x_pairs: torch.Tensor, expert_ids: torch.Tensor, x_tokens: torch.Tensor,
+                       shared_id: int):
+    """Rows and expert ids of a gathered launch that also runs the shared expert: the
+    ``[P, K]`` rows of the routed (token, expert) pairs followed by the ``[T, K]`` rows the
+    shared expert reads, all of the latter with id ``shared_id``.  Rows ``[:P]`` of the
+    launch's output belong to the routed pairs, rows ``[P:]`` to the shared expert."""
+    xt = x_tokens.reshape(-1, x_tokens.shape[-1])
+    x = torch.cat([x_pairs.reshape(-1, x_pairs.shape[-1]), xt], dim=0)
+    ids = torch.cat([expert_ids.reshape(-1).to(torch.int32),
+                     torch.full((xt.shape[0],), shared_id, dtype=torch.int32, device=expert_ids.device)])
+    return x, ids

@@ -5,8 +5,9 @@ import pytest
 import torch
 
 import dflash_mlx_amd._native as nat
-from dflash_mlx_amd.verify_qmm import gather_qmm, join_expert_projections
-from dflash_mlx_amd.workloads import make_moe_case, seed_for
+from dflash_mlx_amd.verify_qmm import (append_shared_expert, gather_qmm, join_expert_projections,
+                                       shared_expert_rows, verify_matmul)
+from dflash_mlx_amd.workloads import MoeCase, make_moe_case, make_qmm_case, seed_for
 from oracle import dflash_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -63,6 +64,32 @@ def test_gate_and_up_of_the_experts_in_one_launch(native_lib):
     assert bool(close.all())
     with pytest.raises(ValueError):
         join_expert_projections((g.w, g.scales, g.biases))
+
+
+@pytest.mark.parametrize("K,N", [(2048, 512), (512, 2048)])
+def test_shared_expert_in_the_gathered_launch(native_lib, K, N):
+    """config[4] with the shared expert stored as expert 256: one launch over 128 routed pairs and
+    16 shared rows gives both products, each to the bar of the closed form, and the shared rows
+    also agree with the dense call on the same weights."""
+    routed = make_moe_case(K, N, seed_for(4, K + 1), experts=256)
+    shared = make_qmm_case(K, N, seed_for(4, K + 2))
+    (w, sc, bi), sid = append_shared_expert((routed.w, routed.scales, routed.biases),
+                                            (shared.w, shared.scales, shared.biases))
+    assert sid == 256 and w.shape == (257, N, K // 8)
+    x, ids = shared_expert_rows(routed.x, routed.expert_ids, shared.x, sid)
+    assert x.shape == (144, K) and ids.dtype == torch.int32 and bool((ids[128:] == 256).all())
+    both = MoeCase(x, ids, w, sc, bi, 64)
+    d = both.to(DEV)
+    y = gather_qmm(d.x, d.w, d.scales, d.biases, d.expert_ids, group_size=64)
+    torch.cuda.synchronize()
+    assert y.shape == (144, N)
+    _check(both, y)
+    dense = verify_matmul(d.x[128:], d.w[256], d.scales[256], d.biases[256])
+    close = (y[128:].float() - dense.float()).abs() <= 2 ** -7 * dense.float().abs().amax(dim=-1, keepdim=True)
+    assert bool(close.all())
+    assert torch.equal(y, gather_qmm(d.x, d.w, d.scales, d.biases, d.expert_ids, group_size=64))
+    with pytest.raises(ValueError):
+        append_shared_expert((routed.w, routed.scales, routed.biases), (shared.w[:16], shared.scales, shared.biases))
 
 
 def test_more_than_sixteen_rows_per_expert_and_unused_experts(native_lib):
