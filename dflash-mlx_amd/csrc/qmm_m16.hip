@@ -184,14 +184,18 @@ __global__ __launch_bounds__(kThreads) void qmm_m16_kernel(
   }
 
   // Partial tiles travel as agent-scope relaxed atomics (written through to / read from
-  // the level all XCDs share); the barrier's vmcnt(0) retires the stores before the
-  // counter is bumped.  A release fence instead would write back the whole L2 per
-  // workgroup, which costs tens of microseconds.
+  // the level all XCDs share).  Every wave waits until its stores are acknowledged before
+  // it joins the barrier behind which the counter is bumped: the barrier alone does not -
+  // a workgroup-scope fence leaves global stores in flight on this target, and the arrival
+  // could overtake them, so that the last workgroup would add what an earlier call left in
+  // the slot.  A release fence instead would write back the whole L2 per workgroup, which
+  // costs tens of microseconds.
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     __hip_atomic_store(&partials[((size_t)part * 16 + m) * N + n0 + 16 * t + col], v[t],
                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (threadIdx.x == 0) {
     // wrapping increment: the k_parts-th arrival sees k_parts-1 and puts the counter
@@ -407,6 +411,13 @@ int qmm_stream_gather_launch(const void* x, const int32_t* expert_ids, const uin
                              const void* scales, const void* biases, void* y, void* workspace,
                              size_t workspace_bytes, int P, int K, int N, int E, int act_dtype,
                              int sb_dtype, hipStream_t stream);
+bool qmm_stream_packed_eligible(int K, int N, int group_size);
+void qmm_stream_packed_bytes(int K, int N, size_t* w_bytes, size_t* sb_bytes);
+int qmm_stream_pack(const uint32_t* w, const void* scales, const void* biases, void* w_out,
+                    void* s_out, void* b_out, int K, int N, hipStream_t stream);
+int qmm_stream_packed_launch(const void* x, const void* w_img, const void* s_img, const void* b_img,
+                             void* y, void* workspace, size_t workspace_bytes, int K, int N,
+                             int act_dtype, int sb_dtype, hipStream_t stream);
 }  // namespace dflash
 
 extern "C" size_t dflash_qmm_m16_workspace_bytes(int K, int N, int group_size, int variant,
@@ -478,6 +489,53 @@ extern "C" int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* sc
     default:
       return launch_gs<128>(act_dtype, sb_dtype, x, w_q, scales, biases, y, partials, counters, K, N, k_parts, s);
   }
+}
+
+extern "C" int dflash_qmm_m16_packed_bytes(int K, int N, int group_size, size_t* codes_bytes,
+                                           size_t* scales_bytes) {
+  using namespace dflash;
+  DFLASH_REQUIRE(codes_bytes && scales_bytes, DFLASH_ERR_ARG, "dflash_qmm_m16_packed_bytes: null result");
+  DFLASH_REQUIRE(qmm_stream_packed_eligible(K, N, group_size), DFLASH_ERR_SHAPE,
+                 "dflash_qmm_m16_packed_bytes: the packed form needs group_size 64, K %% 1024 == 0 and "
+                 "N %% 16 == 0 (K=%d N=%d gs=%d)", K, N, group_size);
+  qmm_stream_packed_bytes(K, N, codes_bytes, scales_bytes);
+  return DFLASH_OK;
+}
+
+extern "C" int dflash_qmm_m16_pack(const uint32_t* w_q, const void* scales, const void* biases,
+                                   void* codes_out, void* scales_out, void* biases_out, int K, int N,
+                                   int group_size, void* stream) {
+  using namespace dflash;
+  DFLASH_REQUIRE(w_q && scales && biases && codes_out && scales_out && biases_out, DFLASH_ERR_ARG,
+                 "dflash_qmm_m16_pack: null operand");
+  DFLASH_REQUIRE(qmm_stream_packed_eligible(K, N, group_size), DFLASH_ERR_SHAPE,
+                 "dflash_qmm_m16_pack: the packed form needs group_size 64, K %% 1024 == 0 and "
+                 "N %% 16 == 0 (K=%d N=%d gs=%d)", K, N, group_size);
+  DFLASH_REQUIRE(((uintptr_t)w_q % 16) == 0 && ((uintptr_t)scales % 16) == 0 && ((uintptr_t)biases % 16) == 0 &&
+                     ((uintptr_t)codes_out % 16) == 0 && ((uintptr_t)scales_out % 16) == 0 &&
+                     ((uintptr_t)biases_out % 16) == 0,
+                 DFLASH_ERR_ARG, "dflash_qmm_m16_pack: operands must be 16-byte aligned");
+  return qmm_stream_pack(w_q, scales, biases, codes_out, scales_out, biases_out, K, N, (hipStream_t)stream);
+}
+
+extern "C" int dflash_qmm_m16_packed(const void* x, const void* codes, const void* scales,
+                                     const void* biases, void* y, void* workspace,
+                                     size_t workspace_bytes, int K, int N, int group_size,
+                                     int act_dtype, int sb_dtype, void* stream) {
+  using namespace dflash;
+  DFLASH_REQUIRE(x && codes && scales && biases && y, DFLASH_ERR_ARG, "dflash_qmm_m16_packed: null operand");
+  DFLASH_REQUIRE(act_dtype == DFLASH_BF16 || act_dtype == DFLASH_FP16, DFLASH_ERR_ARG,
+                 "dflash_qmm_m16_packed: act_dtype %d is not bf16/fp16", act_dtype);
+  DFLASH_REQUIRE(sb_dtype == DFLASH_BF16 || sb_dtype == DFLASH_FP16, DFLASH_ERR_ARG,
+                 "dflash_qmm_m16_packed: sb_dtype %d is not bf16/fp16", sb_dtype);
+  DFLASH_REQUIRE(qmm_stream_packed_eligible(K, N, group_size), DFLASH_ERR_SHAPE,
+                 "dflash_qmm_m16_packed: the packed form needs group_size 64, K %% 1024 == 0 and "
+                 "N %% 16 == 0 (K=%d N=%d gs=%d)", K, N, group_size);
+  DFLASH_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)codes % 16) == 0 && ((uintptr_t)scales % 16) == 0 &&
+                     ((uintptr_t)biases % 16) == 0,
+                 DFLASH_ERR_ARG, "dflash_qmm_m16_packed: operands must be 16-byte aligned");
+  return qmm_stream_packed_launch(x, codes, scales, biases, y, workspace, workspace_bytes, K, N,
+                                  act_dtype, sb_dtype, (hipStream_t)stream);
 }
 
 extern "C" size_t dflash_qmm_m16_gather_workspace_bytes(int P, int K, int N, int E,

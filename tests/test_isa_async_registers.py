@@ -99,3 +99,35 @@ def test_no_instruction_touches_registers_of_reads_in_flight():
         assert reads >= 40, (name, reads)   # the operand reads are there at all
         assert not bad, (name, bad[:5])
         assert "scratch_" not in body, name  # nothing spilled
+
+
+def _compile_to_isa(src, out):
+    cmd = ["hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
+           "-Xclang", "-packed-fp32-ops", "-I", os.path.join(ROOT, "include"),
+           "-I", os.path.dirname(src), "--cuda-device-only", "-S", "-o", out, src]
+    subprocess.run(cmd, check=True, capture_output=True, timeout=600)
+    return open(out).read().split("\n")
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not available")
+@pytest.mark.parametrize("source,arrivals", [("qmm_m16.hip", 24), ("qmm_m16_stream.hip", 32)])
+def test_partial_tiles_are_acknowledged_before_the_arrival_counter(source, arrivals):
+    """Split K: a workgroup stores its partial tile and then bumps the row block's arrival
+    counter; the last to arrive adds the tiles.  Nothing but a wait for the stores'
+    acknowledgement keeps the counter from overtaking them (a workgroup barrier does not wait
+    for global stores on this target), so between the last store before an arrival and the
+    arrival itself the code must wait for all of the wave's memory operations."""
+    with tempfile.TemporaryDirectory() as tmp:
+        lines = _compile_to_isa(os.path.join(os.path.dirname(SRC), source), os.path.join(tmp, "k.s"))
+    found = 0
+    for i, line in enumerate(lines):
+        if "global_atomic_inc" not in line:
+            continue
+        found += 1
+        j, waited = i - 1, False
+        while j >= 0 and "global_store" not in lines[j] and ".Lfunc_begin" not in lines[j]:
+            waited = waited or bool(re.search(r"s_waitcnt\b.*vmcnt\(0\)", lines[j]))
+            j -= 1
+        assert j >= 0 and "global_store" in lines[j], (source, i)
+        assert waited, f"{source}: arrival at line {i + 1} follows the store at line {j + 1} without a wait"
+    assert found == arrivals, (source, found)
