@@ -70,6 +70,12 @@ def run_pass(calls):
     return [verify_matmul(c.x, c.w, c.scales, c.biases, group_size=c.group_size, bits=4) for c in calls]
 
 
+def run_pass_packed(calls, packed):
+    from dflash_mlx_amd.verify_qmm import verify_matmul_packed
+
+    return [verify_matmul_packed(c.x, p) for c, p in zip(calls, packed)]
+
+
 def time_region(fn, steps: int):
     """Wall time and HIP-event time (ms) of ``steps`` invocations of fn."""
     import torch
@@ -94,7 +100,11 @@ def capture(fn):
     return record(fn)
 
 
-def bench_qmm_stack(stack: str, steps: int, warmup: int, device: str, join_gate_up: bool = False):
+def bench_qmm_stack(stack: str, steps: int, warmup: int, device: str, join_gate_up: bool = False,
+                    packed: bool = False):
+    """``packed``: every linear's weights also stored in the streaming kernel's order
+    (``pack_weights``, done before the timed region as at model load) and the calls made through
+    ``verify_matmul_packed``; the results must equal those of the row-major calls bit for bit."""
     import torch
 
     from dflash_mlx_amd.workloads import qmm_algorithmic_bytes, stack_bytes
@@ -107,8 +117,14 @@ def bench_qmm_stack(stack: str, steps: int, warmup: int, device: str, join_gate_
 
     eager = run_pass(calls)  # also creates the split-K workspace outside of graph capture
     torch.cuda.synchronize()
+    one_pass = lambda: run_pass(calls)  # noqa: E731
+    if packed:
+        from dflash_mlx_amd.verify_qmm import pack_weights
 
-    graph, captured = capture(lambda: run_pass(calls))
+        images = [pack_weights(c.w, c.scales, c.biases) for c in calls]
+        one_pass = lambda: run_pass_packed(calls, images)  # noqa: E731
+
+    graph, captured = capture(one_pass)
 
     # every replay must reproduce the eager result bit for bit
     for r in range(2):
@@ -124,8 +140,8 @@ def bench_qmm_stack(stack: str, steps: int, warmup: int, device: str, join_gate_
     ms_per_step = wall_ms / steps
     # eager launches through the Python surface, for the record (one pass first: the outputs of
     # a pass are new tensors, and the allocator's pool has to have grown to hold them)
-    run_pass(calls)
-    e_wall, _ = time_region(lambda: run_pass(calls), max(1, min(steps, 3)))
+    one_pass()
+    e_wall, _ = time_region(one_pass, max(1, min(steps, 3)))
     res = dict(
         calls_per_step=len(calls), weight_bytes=weight_bytes, total_bytes=total_bytes,
         ms_per_step=ms_per_step, event_ms_per_step=ev_ms / steps,
@@ -603,6 +619,14 @@ def main() -> int:
             calls_per_step=j["calls_per_step"], ms_per_step=round(j["ms_per_step"], 4),
             weight_gbps=round(j["weight_gbps"], 1), avg_launch_us=round(j["avg_launch_us"], 3),
             frac_hbm=round(j["total_bytes"] / (j["event_ms_per_step"] * 1e-3) / HBM_PEAK, 4))
+        for label, kw in (("packed_weights", dict(packed=True)),
+                          ("gate_up_in_one_launch_packed_weights", dict(packed=True, join_gate_up=True))):
+            q = bench_qmm_stack(args.workload, args.steps, args.warmup, device, **kw)
+            log(f"[bench] {args.workload} stack, {label}: {q['ms_per_step']:.3f} ms/step")
+            extra[f"stack_{args.workload}_{label}"] = dict(
+                calls_per_step=q["calls_per_step"], ms_per_step=round(q["ms_per_step"], 4),
+                weight_gbps=round(q["weight_gbps"], 1), avg_launch_us=round(q["avg_launch_us"], 3),
+                frac_hbm=round(q["total_bytes"] / (q["event_ms_per_step"] * 1e-3) / HBM_PEAK, 4))
         extra["single_call_16x4096x4096"] = {k: {kk: round(vv, 4) for kk, vv in v.items()}
                                              for k, v in bench_single_call(device).items()}
         mo = bench_moe(device, args.steps, args.warmup)

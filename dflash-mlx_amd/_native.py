@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
@@ -24,6 +24,9 @@ EXPORTED_SYMBOLS = (
     "dflash_last_error",
     "dflash_qmm_m16_workspace_bytes",
     "dflash_qmm_m16",
+    "dflash_qmm_m16_packed_bytes",
+    "dflash_qmm_m16_pack",
+    "dflash_qmm_m16_packed",
     "dflash_qmm_m16_gather_workspace_bytes",
     "dflash_qmm_m16_gather",
     "dflash_tape_replay",
@@ -56,6 +59,12 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.dflash_qmm_m16.argtypes = (
         [c.c_void_p] * 6 + [c.c_size_t] + [c.c_int] * 8 + [c.c_void_p]
     )
+    lib.dflash_qmm_m16_packed_bytes.restype = c.c_int
+    lib.dflash_qmm_m16_packed_bytes.argtypes = [c.c_int] * 3 + [c.POINTER(c.c_size_t)] * 2
+    lib.dflash_qmm_m16_pack.restype = c.c_int
+    lib.dflash_qmm_m16_pack.argtypes = [c.c_void_p] * 6 + [c.c_int] * 3 + [c.c_void_p]
+    lib.dflash_qmm_m16_packed.restype = c.c_int
+    lib.dflash_qmm_m16_packed.argtypes = [c.c_void_p] * 6 + [c.c_size_t] + [c.c_int] * 5 + [c.c_void_p]
     lib.dflash_qmm_m16_gather_workspace_bytes.restype = c.c_size_t
     lib.dflash_qmm_m16_gather_workspace_bytes.argtypes = [c.c_int] * 5
     lib.dflash_qmm_m16_gather.restype = c.c_int

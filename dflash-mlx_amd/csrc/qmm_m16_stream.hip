@@ -58,6 +58,9 @@ constexpr int kRows = 128;   // rows per unit (16 per wave)
 constexpr int kUnitK = 256;  // k per unit (four groups of 64)
 constexpr int kGS = 64;
 constexpr int kGroups = kUnitK / kGS;
+// packed weight images: codes of one unit, scales (or biases) of one chunk of four units
+constexpr int kPackedUnitBytes = kRows * kUnitK / 2;      // 16 KiB
+constexpr int kPackedChunkBytes = kRows * 4 * kGroups * 2;  // 4 KiB
 constexpr int kDepth = 5;                      // ring slots of (codes + x)
 // Units a loader keeps issued beyond the one being consumed.  A CU holds about 64 KiB of
 // loads in flight (what HBM latency times its share of the bandwidth comes to); a loader
@@ -356,7 +359,51 @@ struct Params {
   // w, scales, biases hold E matrices of [N, .] back to back
   const int32_t* expert_ids;
   int P, E;
+  // dense form, K % 1024 == 0: w, scales, biases hold the images qmm_pack_kernel writes - per
+  // (row block, unit) the 16 KiB of codes in the order of the LDS slot, per (row block, chunk)
+  // 4 KiB of scales and of biases - so that every load instruction of a wave moves 1 KiB of
+  // consecutive memory
+  int packed;
 };
+
+// Writes the packed images of one [N, K] matrix (K % 1024 == 0): one thread per 16 bytes of
+// output.  Codes: granule (q, lane) of unit (rb, st) is granule (lane & 7) ^ sw(lane >> 3) of
+// row 128 rb + 8 q + (lane >> 3), bytes 128 st .. 128 st + 127 - the lane order of the loader
+// waves' instruction q.  Scales and biases: granule (part, lane) of chunk (rb, c) is granule
+// lane & 1 of row 128 rb + 32 part + (lane >> 1), groups 16 c .. 16 c + 15.  Rows past N repeat
+// row N - 1 (their products are never stored).
+__global__ __launch_bounds__(256) void qmm_pack_kernel(const uint32_t* __restrict__ w,
+                                                       const uint16_t* __restrict__ scales,
+                                                       const uint16_t* __restrict__ biases,
+                                                       uint4* __restrict__ w_out, uint4* __restrict__ s_out,
+                                                       uint4* __restrict__ b_out, int K, int N) {
+  const int stages = K / kUnitK, chunks = stages / 4;
+  const int RB = (N + kRows - 1) / kRows;
+  const size_t code_granules = (size_t)RB * stages * (kPackedUnitBytes / 16);
+  const size_t sb_granules = (size_t)RB * chunks * (kPackedChunkBytes / 16);
+  const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < code_granules) {
+    const int lane = (int)(t & 63), q = (int)((t >> 6) & 15);
+    const size_t unit = t >> 10;
+    const int st = (int)(unit % stages), rb = (int)(unit / stages);
+    const int r8 = lane >> 3;
+    int row = rb * kRows + 8 * q + r8;
+    row = row < N ? row : N - 1;
+    const int g = (lane & 7) ^ (((r8 >> 1) & 3) << 1);
+    w_out[t] = *reinterpret_cast<const uint4*>((const char*)w + (size_t)row * (K >> 1) + st * (kUnitK / 2) + g * 16);
+  } else if (t < code_granules + 2 * sb_granules) {
+    size_t u = t - code_granules;
+    const bool is_bias = u >= sb_granules;
+    if (is_bias) u -= sb_granules;
+    const int lane = (int)(u & 63), part = (int)((u >> 6) & 3);
+    const size_t chunk = u >> 8;
+    const int c = (int)(chunk % chunks), rb = (int)(chunk / chunks);
+    int row = rb * kRows + 32 * part + (lane >> 1);
+    row = row < N ? row : N - 1;
+    const char* src = (const char*)(is_bias ? biases : scales) + ((size_t)row * (K / kGS) + c * 16) * 2 + (lane & 1) * 16;
+    (is_bias ? b_out : s_out)[u] = *reinterpret_cast<const uint4*>(src);
+  }
+}
 
 // Unit range of workgroup i out of n: [units*i/n, units*(i+1)/n)  (units*n < 2^31).
 __device__ __forceinline__ int range_begin(int units, int i, int n) {
@@ -427,6 +474,10 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t lds0 = lds_address(lds);
   const int RB = (p.N + kRows - 1) / kRows;  // row blocks of one matrix
+  // bytes from one unit's codes to the next unit's of the same rows, and from chunk to chunk
+  const bool packed = !GATHER && CHUNK == 4 && p.packed;
+  const uint32_t w_unit_stride = packed ? kPackedUnitBytes : kUnitK / 2;
+  const uint32_t sb_chunk_stride = packed ? kPackedChunkBytes : CHUNK * kGroups * 2;
 
   int units = p.units;
   if (GATHER) {
@@ -561,7 +612,14 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
         row = row < p.N ? row : p.N - 1;
         wp[i] = (const char*)wmat + (size_t)row * row_bytes + w_c * 16;
       }
-      if (CHUNK == 4) {
+      if (!GATHER && CHUNK == 4 && p.packed) {
+        const char* img = (const char*)p.w + (size_t)wh.rb * p.stages * kPackedUnitBytes + lane * 16;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wp[i] = img + (ld + 4 * i) * 1024;
+        const size_t sb_img = (size_t)wh.rb * (p.stages / 4) * kPackedChunkBytes + ld * 1024 + lane * 16;
+        sbp[0] = (const char*)p.scales + sb_img;
+        sbp[1] = (const char*)p.biases + sb_img;
+      } else if (CHUNK == 4) {
         int row = row0 + 32 * ld + (lane >> 1);
         row = row < p.N ? row : p.N - 1;
         sbp[0] = (const char*)(smat + (size_t)row * G) + (lane & 1) * 16;
@@ -602,7 +660,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       char* slot = lds + slot_i * kSlotBytes;
       if ((st_i % CHUNK) == 0 || (!kFirst && issued == u0)) {
         char* sb = lds + kSbOffset + sb_slot_i * kSbSlotBytes;
-        const size_t off = (size_t)(st_i / CHUNK) * (CHUNK * kGroups * 2);
+        const size_t off = (size_t)(st_i / CHUNK) * sb_chunk_stride;
         if (CHUNK == 4) {
           load16_to_lds(sbp[0] + off, sb + ld * 1024);
           load16_to_lds(sbp[1] + off, sb + kSbArrayBytes + ld * 1024);
@@ -616,7 +674,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
         load16_to_lds(xp[i] + (size_t)st_i * (kUnitK * 2), slot + kXOffset + (ld + 4 * i) * 1024);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        load16_to_lds_stream(wp[i] + (size_t)st_i * (kUnitK / 2), slot + (ld + 4 * i) * 1024);
+        load16_to_lds_stream(wp[i] + (size_t)st_i * w_unit_stride, slot + (ld + 4 * i) * 1024);
       ++issued;
       if (++slot_i == kDepth) slot_i = 0;
       if (++st_i == p.stages) {
@@ -678,6 +736,9 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
     const uint16_t* mat = (wave < 4 ? p.scales : p.biases) + (size_t)wh.expert * p.N * G;
     const char* src = (const char*)(mat + (size_t)row * G) + (lane & 1) * 16 +
                       (size_t)(st0 / CHUNK) * (CHUNK * kGroups * 2);
+    if (packed)
+      src = (const char*)(wave < 4 ? p.scales : p.biases) +
+            ((size_t)wh.rb * (p.stages / 4) + st0 / CHUNK) * kPackedChunkBytes + part * 1024 + lane * 16;
     load16_to_lds(src, lds + kSbOffset + (wave < 4 ? 0 : kSbArrayBytes) + part * 1024);
     // x: instruction `wave` of the loaders' scheme; codes: instructions 2 wave and 2 wave + 1
     int xrow = lane & 15;
@@ -698,8 +759,10 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       const int q = 2 * wave + i;
       int wrow = wh.rb * kRows + 8 * q + w_r;
       wrow = wrow < p.N ? wrow : p.N - 1;
-      load16_to_lds_stream((const char*)wmat + (size_t)wrow * row_bytes + w_c * 16 + (size_t)st0 * (kUnitK / 2),
-                           lds + q * 1024);
+      const char* wsrc = (const char*)wmat + (size_t)wrow * row_bytes + w_c * 16 + (size_t)st0 * (kUnitK / 2);
+      if (packed)
+        wsrc = (const char*)p.w + ((size_t)wh.rb * p.stages + st0) * kPackedUnitBytes + q * 1024 + lane * 16;
+      load16_to_lds_stream(wsrc, lds + q * 1024);
     }
   }
   const int col = lane & 15;
@@ -1047,6 +1110,53 @@ int qmm_stream_launch(const void* x, const uint32_t* w, const void* scales, cons
   const size_t need = qmm_stream_workspace_bytes(N, grid);
   DFLASH_REQUIRE(workspace && workspace_bytes >= need, DFLASH_ERR_WORKSPACE,
                  "dflash_qmm_m16: workspace of %zu bytes needed, %zu given", need,
+                 workspace ? workspace_bytes : (size_t)0);
+  p.counters = (uint32_t*)workspace;
+  p.partials = (float*)((char*)workspace + 64 * 1024);
+  return launch_stream(p, false, grid, act_dtype, sb_dtype, stream);
+}
+
+bool qmm_stream_packed_eligible(int K, int N, int group_size) {
+  return qmm_stream_eligible(K, N, group_size) && K % (stream::kUnitK * 4) == 0;
+}
+
+void qmm_stream_packed_bytes(int K, int N, size_t* w_bytes, size_t* sb_bytes) {
+  const size_t RB = (size_t)(N + stream::kRows - 1) / stream::kRows, stages = (size_t)K / stream::kUnitK;
+  *w_bytes = RB * stages * stream::kPackedUnitBytes;
+  *sb_bytes = RB * (stages / 4) * stream::kPackedChunkBytes;
+}
+
+int qmm_stream_pack(const uint32_t* w, const void* scales, const void* biases, void* w_out,
+                    void* s_out, void* b_out, int K, int N, hipStream_t stream) {
+  size_t wb, sb;
+  qmm_stream_packed_bytes(K, N, &wb, &sb);
+  const size_t threads = (wb + 2 * sb) / 16;
+  hipLaunchKernelGGL(stream::qmm_pack_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
+                     w, (const uint16_t*)scales, (const uint16_t*)biases, (uint4*)w_out, (uint4*)s_out,
+                     (uint4*)b_out, K, N);
+  DFLASH_HIP_OK(hipGetLastError());
+  return DFLASH_OK;
+}
+
+int qmm_stream_packed_launch(const void* x, const void* w_img, const void* s_img, const void* b_img,
+                             void* y, void* workspace, size_t workspace_bytes, int K, int N,
+                             int act_dtype, int sb_dtype, hipStream_t stream) {
+  using namespace stream;
+  Params p{};
+  p.x = (const uint16_t*)x;
+  p.w = (const uint32_t*)w_img;
+  p.scales = (const uint16_t*)s_img;
+  p.biases = (const uint16_t*)b_img;
+  p.y = (uint16_t*)y;
+  p.K = K;
+  p.N = N;
+  p.stages = K / kUnitK;
+  p.units = ((N + kRows - 1) / kRows) * p.stages;
+  p.packed = 1;
+  const int grid = qmm_stream_pick_grid(p.units, p.units / p.stages, qmm_stream_grid());
+  const size_t need = qmm_stream_workspace_bytes(N, grid);
+  DFLASH_REQUIRE(workspace && workspace_bytes >= need, DFLASH_ERR_WORKSPACE,
+                 "dflash_qmm_m16_packed: workspace of %zu bytes needed, %zu given", need,
                  workspace ? workspace_bytes : (size_t)0);
   p.counters = (uint32_t*)workspace;
   p.partials = (float*)((char*)workspace + 64 * 1024);

@@ -19,6 +19,7 @@ and shape dispatch, with the device work done by the gfx950 kernel behind
 """
 from __future__ import annotations
 
+import ctypes
 import os
 from typing import Dict, Tuple
 
@@ -154,6 +155,81 @@ def verify_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases
 
 # the name the hot path is known by
 verify_qmm = verify_matmul
+
+
+class PackedWeights:
+    """One linear's codes, scales and biases in the order the streaming kernel consumes them
+    (``pack_weights``).  A second copy of the weights, made once when the model is loaded; the
+    row-major MLX triple it was made from is not referenced."""
+
+    __slots__ = ("codes", "scales", "biases", "K", "N", "group_size")
+
+    def __init__(self, codes, scales, biases, K, N, group_size):
+        self.codes, self.scales, self.biases = codes, scales, biases
+        self.K, self.N, self.group_size = K, N, group_size
+
+
+def packable(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, group_size: int = 64,
+             bits: int = 4) -> bool:
+    """Shapes the packed form covers: 4 bits, group 64, K a multiple of 1024, N of 32 (the
+    Python gate's rule for N), bf16/fp16 scales, device tensors."""
+    if bits != 4 or group_size != 64 or w.ndim != 2 or not w.is_cuda:
+        return False
+    K, N = int(w.shape[1]) * 8, int(w.shape[0])
+    return (K % 1024 == 0 and N % 32 == 0 and scales.dtype in _DTYPE_CODE and biases.dtype == scales.dtype
+            and tuple(scales.shape) == (N, K // 64) and tuple(biases.shape) == (N, K // 64))
+
+
+def pack_weights(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, *, group_size: int = 64,
+                 bits: int = 4) -> PackedWeights:
+    """Rewrites an MLX affine triple (``w [N, K/8]`` words, ``scales``/``biases [N, K/64]``) into the
+    packed images ``verify_matmul_packed`` reads: per 128 rows and 256 k the 16 KiB of codes in
+    the order of the kernel's LDS slot, per 128 rows and 1024 k the 4 KiB of scales and of
+    biases.  No counterpart in the reference, whose kernel gathers 4-byte words from the
+    row-major arrays (``verify_qmm.py:68-72``)."""
+    if not packable(w, scales, biases, group_size, bits):
+        raise ValueError("pack_weights: needs 4-bit codes, group 64, K % 1024 == 0, N % 32 == 0, "
+                         "bf16/fp16 scales and biases of shape [N, K/64], on the GPU")
+    lib = _native.lib()
+    K, N = int(w.shape[1]) * 8, int(w.shape[0])
+    cb, sb = ctypes.c_size_t(), ctypes.c_size_t()
+    _native.check(lib.dflash_qmm_m16_packed_bytes(K, N, group_size, ctypes.byref(cb), ctypes.byref(sb)),
+                  "dflash_qmm_m16_packed_bytes")
+    w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
+    codes = torch.empty(cb.value, dtype=torch.uint8, device=w.device)
+    s_img = torch.empty(sb.value // 2, dtype=scales.dtype, device=w.device)
+    b_img = torch.empty(sb.value // 2, dtype=scales.dtype, device=w.device)
+    rc = lib.dflash_qmm_m16_pack(w.data_ptr(), scales.data_ptr(), biases.data_ptr(), codes.data_ptr(),
+                                 s_img.data_ptr(), b_img.data_ptr(), K, N, group_size,
+                                 _native.raw_stream(w.device))
+    _native.check(rc, "dflash_qmm_m16_pack")
+    return PackedWeights(codes, s_img, b_img, K, N, group_size)
+
+
+def verify_matmul_packed(x: torch.Tensor, packed: PackedWeights) -> torch.Tensor:
+    """``verify_matmul`` on packed weights: 16 rows of bf16/fp16 device activations; the result is
+    bit for bit that of the streaming kernel on the triple the weights were packed from."""
+    K, N = packed.K, packed.N
+    m = 1
+    for d in x.shape[:-1]:
+        m *= int(d)
+    if m != 16 or int(x.shape[-1]) != K or x.dtype not in _DTYPE_CODE or not x.is_cuda:
+        raise ValueError("verify_matmul_packed: x must hold 16 rows of K bf16/fp16 values on the GPU")
+    lib = _native.lib()
+    x2 = x.reshape(16, K).contiguous()
+    y = torch.empty((16, N), dtype=x2.dtype, device=x2.device)
+    stream = _native.raw_stream(x2.device)
+    key = (K, N, packed.group_size, _VARIANT_CODE["mma2big"], 1, _native.QMM_KERNEL_STREAM)
+    need = _WORKSPACE_BYTES.get(key)
+    if need is None:
+        need = _WORKSPACE_BYTES[key] = int(lib.dflash_qmm_m16_workspace_bytes(*key))
+    ws = _workspace(x2.device, stream, need)
+    rc = lib.dflash_qmm_m16_packed(x2.data_ptr(), packed.codes.data_ptr(), packed.scales.data_ptr(),
+                                   packed.biases.data_ptr(), y.data_ptr(), ws.data_ptr(), ws.numel(),
+                                   K, N, packed.group_size, _DTYPE_CODE[x2.dtype],
+                                   _DTYPE_CODE[packed.scales.dtype], stream)
+    _native.check(rc, "dflash_qmm_m16_packed")
+    return y.reshape(*x.shape[:-1], N)
 
 
 def small_m_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 7
+#define DFLASH_ABI_VERSION 8
 
 enum {
   DFLASH_OK = 0,
@@ -81,6 +81,34 @@ size_t dflash_qmm_m16_workspace_bytes(int K, int N, int group_size, int variant,
 int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* scales, const void* biases,
                    void* y, void* workspace, size_t workspace_bytes, int K, int N, int group_size,
                    int act_dtype, int sb_dtype, int variant, int k_parts, int kernel, void* stream);
+
+/*
+ * The same product on weights stored in the order the streaming kernel consumes them.  No
+ * counterpart in the reference (MLX keeps the row-major triple of dflash_mlx/verify_qmm.py:70-72
+ * and its kernel gathers 4-byte words from it); a caller that may keep a second copy of a
+ * linear's weights packs them once when the model is loaded (the place where
+ * dflash_mlx/verify_linear.py:146-168 swaps the modules) and calls the packed form per step.
+ * In the row-major form a 128-row block contributes 128 pieces of 128 bytes of codes and 256
+ * pieces of 32 bytes of scales and biases per step along K, each piece a memory access of its
+ * own; packed, every load instruction of a wave reads 1 KiB of consecutive memory.
+ *
+ *   codes   [ceil(N/128), K/256, 16 KiB]   scales, biases [ceil(N/128), K/1024, 4 KiB]
+ *   (sizes from dflash_qmm_m16_packed_bytes; rows past N repeat row N-1)
+ * Requirements: group_size 64, K % 1024 == 0, N % 16 == 0; all pointers 16-byte aligned; the
+ * workspace of dflash_qmm_m16 (kernel = DFLASH_QMM_KERNEL_STREAM) with the same rules.
+ * dflash_qmm_m16_packed returns bit for bit what dflash_qmm_m16 returns through the streaming
+ * kernel for the unpacked operands.
+ */
+int dflash_qmm_m16_packed_bytes(int K, int N, int group_size, size_t* codes_bytes,
+                                size_t* scales_bytes /* = biases bytes */);
+
+int dflash_qmm_m16_pack(const uint32_t* w_q, const void* scales, const void* biases,
+                        void* codes_out, void* scales_out, void* biases_out, int K, int N,
+                        int group_size, void* stream);
+
+int dflash_qmm_m16_packed(const void* x, const void* codes, const void* scales, const void* biases,
+                          void* y, void* workspace, size_t workspace_bytes, int K, int N,
+                          int group_size, int act_dtype, int sb_dtype, void* stream);
 
 /*
  * Gathered per-expert M<=16-per-expert qmm for MoE layers: y[p,:] = x[p,:] . (s*q + b)^T of
