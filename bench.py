@@ -576,6 +576,9 @@ def main() -> int:
     ap.add_argument("--workload", default="27b", choices=["27b", "9b"])
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the cpu_baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the headline stack")
+    ap.add_argument("--packed-weights", action="store_true",
+                    help="headline stack through verify_matmul_packed (weights stored in the streaming "
+                         "kernel's order); off by default: the headline uses the reference's operands")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run three 1 GiB device-to-device copies (a kernel of known traffic, "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings) and exit")
@@ -604,7 +607,7 @@ def main() -> int:
     device = "cuda:0"
     torch.cuda.set_device(0)
 
-    main_res = bench_qmm_stack(args.workload, args.steps, args.warmup, device)
+    main_res = bench_qmm_stack(args.workload, args.steps, args.warmup, device, packed=args.packed_weights)
     log(f"[bench] {args.workload}: {main_res['ms_per_step']:.3f} ms/step, "
         f"{main_res['weight_gbps']:.0f} GB/s weights, {main_res['avg_launch_us']:.2f} us/launch")
     extra = {}
@@ -652,7 +655,8 @@ def main() -> int:
 
     achieved = main_res["bytes_per_launch"] / (main_res["avg_launch_us"] * 1e-6) / 1e9
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK / 1e9, unit="GB/s",
-                    frac=round(achieved * 1e9 / HBM_PEAK, 4), traffic=MEASURED_TRAFFIC_BYTES.get(args.workload),
+                    frac=round(achieved * 1e9 / HBM_PEAK, 4),
+                    traffic=None if args.packed_weights else MEASURED_TRAFFIC_BYTES.get(args.workload),
                     kernel="qmm_stream_kernel", bytes_per_launch=round(main_res["bytes_per_launch"]),
                     avg_launch_us=round(main_res["avg_launch_us"], 3))
     cpu = None if args.skip_cpu else bench_cpu_baseline(args.workload)
@@ -671,7 +675,8 @@ def main() -> int:
         "dtype": "bf16 x int4 (fp32 accumulate)",
         "data": "synthetic",
         "config": {"workload": f"{args.workload}-shaped dense int4 verify stack, M=16, group 64, "
-                               f"{main_res['calls_per_step']} verify_matmul calls per step (HIP graph replay)",
+                               f"{main_res['calls_per_step']} verify_matmul calls per step (HIP graph replay)"
+                               + (", packed weights" if args.packed_weights else ""),
                    "weight_bytes_per_step": main_res["weight_bytes"],
                    "eager_ms_per_step": round(main_res["eager_ms_per_step"], 3)},
         "pct_hbm_peak": round(100.0 * main_res["weight_gbps"] * 1e9 / HBM_PEAK, 2),
