@@ -121,6 +121,7 @@ class SharedInputGroup:
         self._input: Optional[torch.Tensor] = None
         self._product: Optional[torch.Tensor] = None
         self._pending = 0
+        self._packed = None  # the joint matrix in the streaming kernel's order (pack_verify_linears)
 
     @staticmethod
     def _key_of(x: torch.Tensor):
@@ -129,8 +130,11 @@ class SharedInputGroup:
     def member_output(self, index: int, x: torch.Tensor) -> torch.Tensor:
         bit = 1 << index
         if self._product is None or not (self._pending & bit) or self._key != self._key_of(x):
-            self._product = verify_matmul(x, self.weight, self.scales, self.biases, transpose=True,
-                                          group_size=self.group_size, bits=self.bits)
+            if self._packed is not None and x.is_cuda:
+                self._product = verify_matmul_packed(x, self._packed)
+            else:
+                self._product = verify_matmul(x, self.weight, self.scales, self.biases, transpose=True,
+                                              group_size=self.group_size, bits=self.bits)
             self._key, self._input = self._key_of(x), x
             self._pending = (1 << len(self.bounds)) - 1
         lo, hi = self.bounds[index]
@@ -225,8 +229,8 @@ def install_verify_linears(model: nn.Module, *,
 
 
 def pack_verify_linears(model: nn.Module) -> int:
-    """Gives every swapped linear that stands alone (not a member of a shared-input group) and
-    whose shape the packed form covers (group 64, K a multiple of 1024, on the GPU) a second copy
+    """Gives every swapped linear that stands alone, and every shared-input group (its joint
+    matrix, counted once), whose shape the packed form covers (group 64, K a multiple of 1024, on the GPU) a second copy
     of its weights in the order the streaming kernel reads them; its 16-row calls then go through
     ``verify_matmul_packed`` and return the same bits as before, 3-8 % sooner.  The row-major
     buffers stay for every other call shape.  Call it after ``install_verify_linears`` (and
@@ -235,6 +239,11 @@ def pack_verify_linears(model: nn.Module) -> int:
     the reference."""
     count = 0
     for m in model.modules():
+        shared = getattr(m, "_shared_input", None) if isinstance(m, VerifyQuantizedLinear) else None
+        if shared is not None and shared[0]._packed is None and shared[0].bits == 4 \
+                and packable(shared[0].weight, shared[0].scales, shared[0].biases, shared[0].group_size, 4):
+            shared[0]._packed = pack_weights(shared[0].weight, shared[0].scales, shared[0].biases)
+            count += 1
         if (isinstance(m, VerifyQuantizedLinear) and getattr(m, "_shared_input", None) is None
                 and getattr(m, "_packed", None) is None and m.biases is not None and m.mode == "affine"
                 and packable(m.weight, m.scales, m.biases, m.group_size, m.bits)):

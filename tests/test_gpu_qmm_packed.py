@@ -117,8 +117,9 @@ def test_packed_form_rejects_what_it_does_not_cover(native_lib):
 
 def test_modules_switch_to_their_packed_copy(verify_env, native_lib):
     """pack_verify_linears: stand-alone swapped linears of a covered shape get a packed copy and
-    return the same bits; members of a shared-input group and uncovered shapes are left alone;
-    other call shapes still use the row-major buffers; moving a module drops the copy."""
+    return the same bits; uncovered shapes are left alone;
+    a shared-input group gets one for its joint matrix; other call shapes still use the row-major
+    buffers; moving a module drops the copy."""
     verify_env.setenv("DFLASH_QMM_KERNEL", "auto")
     shapes = {"gate_proj": (1024, 512), "up_proj": (1024, 512), "down_proj": (2048, 1024), "odd": (1536, 256)}
     cases = {n: make_qmm_case(K, N, seed_for(0, 700 + i)) for i, (n, (K, N)) in enumerate(shapes.items())}
@@ -130,9 +131,13 @@ def test_modules_switch_to_their_packed_copy(verify_env, native_lib):
     assert install_verify_linears(model) == 4
     before = {n: getattr(model.mlp, n)(cases[n].x.to(DEV)) for n in cases}
     assert fuse_shared_input_linears(model) == 1
-    assert pack_verify_linears(model) == 1 and pack_verify_linears(model) == 0
+    group = model.mlp.gate_proj._shared_input[0]
+    xg = cases["gate_proj"].x.to(DEV)
+    joint = VQ.verify_matmul(xg, group.weight, group.scales, group.biases, group_size=64, bits=4)
+    assert pack_verify_linears(model) == 2 and pack_verify_linears(model) == 0  # down_proj and the gate/up group
     assert model.mlp.down_proj._packed is not None and model.mlp.odd._packed is None
-    assert model.mlp.gate_proj._packed is None
+    assert model.mlp.gate_proj._packed is None and group._packed is not None and group._packed.N == 1024
+    assert torch.equal(torch.cat([model.mlp.gate_proj(xg), model.mlp.up_proj(xg)], dim=-1), joint)
     called = []
     import dflash_mlx_amd.verify_linear as VL
     real = VL.verify_matmul_packed
@@ -143,7 +148,7 @@ def test_modules_switch_to_their_packed_copy(verify_env, native_lib):
     finally:
         VL.verify_matmul_packed = real
     torch.cuda.synchronize()
-    assert called == [1024]
+    assert called == [1024, 1024, 1024]  # the gate/up group for each of the two inputs, then down_proj
     for n in ("down_proj", "odd"):
         assert torch.equal(before[n], after[n])
     x3 = torch.randn(3, 2048, device=DEV).to(torch.bfloat16)
