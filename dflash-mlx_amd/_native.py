@@ -12,11 +12,12 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
 QMM_KERNEL_AUTO, QMM_KERNEL_TILE, QMM_KERNEL_STREAM = 0, 1, 2
+QMM_STATIC_SCRATCH_BYTES = 8 << 20  # DFLASH_QMM_STATIC_SCRATCH_BYTES
 
 # every symbol include/dflash_mi355.h declares
 EXPORTED_SYMBOLS = (
@@ -24,6 +25,7 @@ EXPORTED_SYMBOLS = (
     "dflash_last_error",
     "dflash_qmm_m16_workspace_bytes",
     "dflash_qmm_m16",
+    "dflash_qmm_m16_static",
     "dflash_qmm_m16_packed_bytes",
     "dflash_qmm_m16_pack",
     "dflash_qmm_m16_packed",
@@ -59,6 +61,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.dflash_qmm_m16.argtypes = (
         [c.c_void_p] * 6 + [c.c_size_t] + [c.c_int] * 8 + [c.c_void_p]
     )
+    lib.dflash_qmm_m16_static.restype = c.c_int
+    lib.dflash_qmm_m16_static.argtypes = [c.c_void_p] * 5 + [c.c_int] * 8 + [c.c_void_p]
     lib.dflash_qmm_m16_packed_bytes.restype = c.c_int
     lib.dflash_qmm_m16_packed_bytes.argtypes = [c.c_int] * 3 + [c.POINTER(c.c_size_t)] * 2
     lib.dflash_qmm_m16_pack.restype = c.c_int

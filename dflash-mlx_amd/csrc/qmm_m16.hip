@@ -29,6 +29,8 @@
 // tile; the last workgroup to arrive for a column block (agent-scope counter)
 // sums the partials in slice order and rounds once, so the result does not
 // depend on arrival order.
+#include <mutex>
+
 #include "dflash_common.h"
 
 namespace dflash {
@@ -489,6 +491,67 @@ extern "C" int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* sc
     default:
       return launch_gs<128>(act_dtype, sb_dtype, x, w_q, scales, biases, y, partials, counters, K, N, k_parts, s);
   }
+}
+
+// ---------------------------------------------------------------------------------
+// dflash_qmm_m16_static: the same product for callers that cannot allocate.
+// ---------------------------------------------------------------------------------
+// The workspace of dflash_qmm_m16 (arrival counters, then fp32 partial tiles) lives in a
+// device array that is part of the library's image: every GPU the library runs on holds
+// its own copy from the first use to the end of the process.
+constexpr size_t kStaticScratchBytes = DFLASH_QMM_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace dflash {
+namespace {
+// zero-fills the counter block (16 bytes per thread)
+__global__ __launch_bounds__(256) void scratch_clear_kernel(uint4* p, int n16) {
+  const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+  if (i < n16) p[i] = make_uint4(0u, 0u, 0u, 0u);
+}
+
+// Device address of `scratch` on the current device.  In host code the array's name is only
+// a handle for the runtime, never an address a kernel could use: the address is asked for
+// once per device (each device has its own copy at its own address) and kept.  The first
+// use on a device also puts the counter block to zero on `stream`, ahead of the caller's
+// kernel; from then on every call leaves the counters at zero.
+int static_scratch(void** out, hipStream_t stream) {
+  static std::mutex mu;
+  static void* ptrs[kMaxDevices] = {};
+  const int slot = current_device_slot();
+  std::lock_guard<std::mutex> lock(mu);
+  // devices beyond the table share its last entry: looked up (and cleared) on every call
+  if (ptrs[slot] == nullptr || slot == kMaxDevices - 1) {
+    void* ptr = nullptr;
+    DFLASH_HIP_OK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    DFLASH_REQUIRE(ptr != nullptr, DFLASH_ERR_HIP, "dflash_qmm_m16_static: no device address for the scratch array");
+    const int n16 = (int)(kCounterBytes / 16);
+    hipLaunchKernelGGL(scratch_clear_kernel, dim3((n16 + 255) / 256), dim3(256), 0, stream, (uint4*)ptr, n16);
+    DFLASH_HIP_OK(hipGetLastError());
+    ptrs[slot] = ptr;
+  }
+  *out = ptrs[slot];
+  return DFLASH_OK;
+}
+}  // namespace
+}  // namespace dflash
+
+extern "C" int dflash_qmm_m16_static(const void* x, const uint32_t* w_q, const void* scales,
+                                     const void* biases, void* y, int K, int N, int group_size,
+                                     int act_dtype, int sb_dtype, int variant, int k_parts,
+                                     int kernel, void* stream) {
+  using namespace dflash;
+  const size_t need = dflash_qmm_m16_workspace_bytes(K, N, group_size, variant,
+                                                     variant == DFLASH_QMM_MMA2BIG ? 1 : k_parts, kernel);
+  DFLASH_REQUIRE(need <= kStaticScratchBytes, DFLASH_ERR_WORKSPACE,
+                 "dflash_qmm_m16_static: this call needs %zu bytes of scratch memory, the built-in "
+                 "array holds %zu; use dflash_qmm_m16 with a workspace of the caller's",
+                 need, kStaticScratchBytes);
+  void* ptr = nullptr;
+  const int rc = static_scratch(&ptr, (hipStream_t)stream);
+  if (rc != DFLASH_OK) return rc;
+  return dflash_qmm_m16(x, w_q, scales, biases, y, ptr, kStaticScratchBytes, K, N, group_size,
+                        act_dtype, sb_dtype, variant, k_parts, kernel, stream);
 }
 
 extern "C" int dflash_qmm_m16_packed_bytes(int K, int N, int group_size, size_t* codes_bytes,

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 8
+#define DFLASH_ABI_VERSION 9
 
 enum {
   DFLASH_OK = 0,
@@ -81,6 +81,26 @@ size_t dflash_qmm_m16_workspace_bytes(int K, int N, int group_size, int variant,
 int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* scales, const void* biases,
                    void* y, void* workspace, size_t workspace_bytes, int K, int N, int group_size,
                    int act_dtype, int sb_dtype, int variant, int k_parts, int kernel, void* stream);
+
+/*
+ * dflash_qmm_m16 for callers that cannot allocate device memory: code under HIP graph
+ * capture, serving loops and harnesses that forbid hipMalloc.  No counterpart in the
+ * reference (MLX allocates behind every array).  The workspace is an array inside the
+ * library's own device image (DFLASH_QMM_STATIC_SCRATCH_BYTES, 8 MiB, held by
+ * every GPU the library is used on until the process ends); the call allocates and frees
+ * nothing.  Same operands, requirements, kernels and results (bit for bit) as dflash_qmm_m16.
+ * A call whose workspace would not fit the array returns DFLASH_ERR_WORKSPACE: the dense
+ * projections of the verify stacks need about 4 MiB; a pipe call served by the tile kernel
+ * needs 64 KiB + k_parts * 64 * N bytes.  All calls on one GPU share that GPU's array:
+ * calls that overlap in time on one GPU (two streams, two threads) race, as they would on a
+ * shared workspace.  The first call on a GPU also enqueues a small kernel on `stream` that
+ * zero-fills the array's counter block.
+ */
+#define DFLASH_QMM_STATIC_SCRATCH_BYTES ((size_t)8 << 20)
+
+int dflash_qmm_m16_static(const void* x, const uint32_t* w_q, const void* scales, const void* biases,
+                          void* y, int K, int N, int group_size, int act_dtype, int sb_dtype,
+                          int variant, int k_parts, int kernel, void* stream);
 
 /*
  * The same product on weights stored in the order the streaming kernel consumes them.  No
