@@ -222,17 +222,26 @@ def tape_replay_kernel(tape: torch.Tensor, k: torch.Tensor, g: torch.Tensor, sta
         raise ValueError(f"Cannot align K heads {hk} to tape heads {hv}")
     if any(t.dtype not in _DTYPE_CODE for t in (tape, k, g, state)):
         return _tape_replay_ops(tape, k, g, state, mask)
-    # LDS budget of the kernel: T*(Dv + 2*Dk + 1) floats
-    if steps * (dv + 2 * dk + 1) * 4 + dk * 4 > 64 * 1024:
+    def fits_lds(rows: int) -> bool:  # the kernel stages T_alloc*(Dv + 2*Dk + 1) floats
+        return rows * (dv + 2 * dk + 1) * 4 + dk * 4 <= 64 * 1024
+
+    if not fits_lds(steps):
         return _tape_replay_ops(tape, k, g, state, mask)
 
     state_c = state.contiguous()
     tape_c, T_tape = _slot_major(tape, hv * dv)
     k_c, T_k = _slot_major(k, hk * dk)
     g_c, T_g = _slot_major(g, hv * (dk if g.ndim == 4 else 1))
-    if not (T_tape == T_k == T_g):
+    # prefix slices are read in place only when all three share one row count that the kernel
+    # can stage; otherwise dense copies of the `steps` rows
+    if not (T_tape == T_k == T_g) or not fits_lds(T_tape):
         tape_c, k_c, g_c = tape.contiguous(), k.contiguous(), g.contiguous()
         T_tape = steps
+    if mask is not None:
+        # the kernel reads the mask with the tape's row count per slot
+        mask = mask.reshape(bsz, steps).to(torch.uint8)
+        if T_tape != steps:
+            mask = torch.nn.functional.pad(mask, (0, T_tape - steps))
     state_out = torch.empty_like(state_c)
     replay_launch(tape_c, k_c, g_c, state_c, state_out, steps=steps, T_alloc=T_tape, mask=mask,
                   slots=bsz)

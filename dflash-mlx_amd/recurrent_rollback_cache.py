@@ -63,8 +63,6 @@ class RecurrentRollbackCache:
     def __init__(self, size: int = 2, *, conv_kernel_size: int = 4):
         self.cache: List[Any] = [None] * size
         self.conv_kernel_size = int(conv_kernel_size)
-        self.left_padding = None
-        self.lengths = None
         self._armed = False
         self._tape = None
         self._tape_k = None
@@ -87,55 +85,6 @@ class RecurrentRollbackCache:
     @state.setter
     def state(self, value) -> None:
         self.cache = value
-
-    # -- batch-cache protocol of the generation loop (recurrent_rollback_cache.py:46-94)
-    def filter(self, batch_indices):
-        self.cache = [c[batch_indices] if c is not None else None for c in self.cache]
-        if self.lengths is not None:
-            self.lengths = self.lengths[batch_indices]
-
-    def extend(self, other):
-        def cat(lhs, rhs):
-            if lhs is None:
-                return rhs
-            if rhs is None:
-                return lhs
-            return torch.cat([lhs, rhs])
-
-        if len(self.cache) != len(other.cache):
-            raise ValueError("cache sizes differ")
-        self.cache = [cat(lhs, rhs) for lhs, rhs in zip(self.cache, other.cache)]
-
-    def extract(self, idx):
-        cache = RecurrentRollbackCache(len(self.cache), conv_kernel_size=self.conv_kernel_size)
-        cache.cache = [c[idx: idx + 1] if c is not None else None for c in self.cache]
-        return cache
-
-    def prepare(self, lengths=None, **kwargs):
-        self.lengths = None if lengths is None else torch.as_tensor(lengths)
-
-    def finalize(self):
-        self.lengths = None
-        self.left_padding = None
-        self.clear_transients()
-
-    def advance(self, n: int):
-        if self.lengths is not None:
-            self.lengths = self.lengths - n
-        if self.left_padding is not None:
-            self.left_padding = self.left_padding - n
-
-    def make_mask(self, n: int):
-        if self.left_padding is not None:
-            pos = torch.arange(n, device=self.left_padding.device)
-            return pos >= self.left_padding[:, None]
-        if self.lengths is not None:
-            pos = torch.arange(n, device=self.lengths.device)
-            return pos < self.lengths[:, None]
-        return None
-
-    def empty(self):
-        return self.cache[0] is None
 
     @property
     def nbytes(self):
@@ -236,7 +185,7 @@ class RollbackArena:
     def __init__(self, num_layers: int, *, batch: int = 1, max_steps: int = 16, Hk: int, Hv: int,
                  Dk: int, Dv: int, conv_dim: int, conv_kernel_size: int = 4,
                  device: Union[str, torch.device] = "cuda", state_dtype=torch.float32,
-                 tape_dtype=torch.bfloat16, k_dtype=torch.bfloat16, g_dtype=torch.float32,
+                 tape_dtype=torch.float32, k_dtype=torch.bfloat16, g_dtype=torch.float32,
                  qkv_dtype=torch.bfloat16, g_per_dk: bool = False):
         self.L, self.B, self.T = int(num_layers), int(batch), int(max_steps)
         self.Hk, self.Hv, self.Dk, self.Dv, self.C = Hk, Hv, Dk, Dv, int(conv_dim)
@@ -291,14 +240,12 @@ class RollbackArena:
         dst = self.tape_slots(layer)
         out = []
         for d, src, name in zip(dst, (tape, k, g, qkv), ("tape", "k", "g", "qkv")):
-            if src.dtype != d.dtype:
-                raise TypeError(f"arena holds {name} as {d.dtype}, got {src.dtype}")
             steps = int(src.shape[1])
             if steps > self.T:
                 raise ValueError(f"{name} has {steps} steps, arena holds {self.T}")
             view = d[:, :steps]
-            if src.data_ptr() != view.data_ptr():
-                view.copy_(src)
+            if src.data_ptr() != view.data_ptr() or src.dtype != d.dtype:
+                view.copy_(src)  # converts when the producer's dtype is not the arena's
             out.append(view)
         return tuple(out)
 
@@ -342,8 +289,8 @@ class RollbackArena:
     def rollback_all(self, n_accepted: Union[int, torch.Tensor], *, drafted_tokens: int = 0) -> None:
         """Roll every layer back to ``n_accepted`` accepted draft tokens.
 
-        ``n_accepted`` is a host int, or an int32 device tensor (scalar or one entry
-        per slot) when the acceptance length has not been read back; in that case
+        ``n_accepted`` is a host int, or an int32 device tensor (a scalar, one entry per
+        batch row, or one per layer and batch row) when the acceptance length has not been read back; in that case
         ``drafted_tokens`` cannot short-cut the fully-accepted case and the replay of
         all recorded steps reproduces the forward's state instead.
         """
@@ -364,8 +311,15 @@ class RollbackArena:
         if host:
             steps: Union[int, torch.Tensor] = int(n_accepted) + 1
         else:
-            acc = n_accepted.to(torch.int32).reshape(-1)
-            self.steps.copy_((acc + 1).expand(self.L * self.B) if acc.numel() == 1 else acc + 1)
+            acc = n_accepted.to(torch.int32).reshape(-1) + 1
+            if acc.numel() == 1:
+                acc = acc.expand(self.L * self.B)
+            elif acc.numel() == self.B:  # one per batch row: slot = layer * B + row
+                acc = acc.repeat(self.L)
+            elif acc.numel() != self.L * self.B:
+                raise ValueError(f"n_accepted has {acc.numel()} entries; expected 1, {self.B} (one per "
+                                 f"batch row) or {self.L * self.B} (one per layer and batch row)")
+            self.steps.copy_(acc)
             steps = self.steps
         replay_launch(self.tape, self.k, self.g, self.state[snap], self.state[nxt], steps=steps,
                       T_alloc=self.T, slots=self.L * self.B)

@@ -153,8 +153,11 @@ def verify_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases
     return y.reshape(*orig_shape[:-1], N)
 
 
-# the name the hot path is known by
-verify_qmm = verify_matmul
+def verify_qmm(x: torch.Tensor, w_packed: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
+               group_size: int = 64, bits: int = 4, *, transpose: bool = True) -> torch.Tensor:
+    """The name the hot path is known by: ``verify_matmul`` with ``group_size`` and ``bits``
+    accepted positionally as well."""
+    return verify_matmul(x, w_packed, scales, biases, transpose=transpose, group_size=group_size, bits=bits)
 
 
 class PackedWeights:

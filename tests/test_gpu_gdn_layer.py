@@ -153,3 +153,40 @@ def test_speculative_layer_call_on_the_device_matches_the_host(native_lib, monke
     assert rel(outs[1][1], outs[0][1]) < 2e-2
     assert rel(caches[1][1], caches[0][1]) < 2e-2
     assert rel(caches[1][0], caches[0][0]) < 1e-2
+
+
+def test_layer_hook_with_an_arena_cache_matches_the_per_layer_cache(native_lib, monkeypatch):
+    """The documented set-up - RollbackArena with its defaults, the layer's speculative hook
+    recording its fp32 tape into it, rollback_all - against a plain RecurrentRollbackCache."""
+    import copy
+
+    from dflash_mlx_amd.recurrent_rollback_cache import RollbackArena
+
+    monkeypatch.setenv("DFLASH_VERIFY_QMM", "1")
+    host = _layer(seed=18, hidden=512, Hk=2, Hv=4, D=128, dtype=torch.bfloat16, quantized=True)
+    G._install_exact_small_proj_hooks(host)
+    G._install_speculative_linear_cache_hook(host)
+    layer = copy.deepcopy(host).to(DEV)
+    gen = torch.Generator().manual_seed(19)
+    prompt = torch.randn((1, 7, 512), generator=gen).to(torch.bfloat16).to(DEV)
+    block = torch.randn((1, 16, 512), generator=gen).to(torch.bfloat16).to(DEV)
+    conv_dim = 2 * 2 * 128 + 4 * 128
+
+    plain = RecurrentRollbackCache()
+    layer(prompt, cache=plain)
+    plain[1] = plain[1].float()
+    conv0, state0 = plain[0].clone(), plain[1].clone()
+    plain.arm_rollback(prefix_len=7)
+    y_plain = layer(block, cache=plain)
+    plain.rollback(9)
+
+    arena = RollbackArena(1, Hk=2, Hv=4, Dk=128, Dv=128, conv_dim=conv_dim, device=DEV)
+    cache = arena.caches()[0]
+    cache[0].copy_(conv0); cache[1].copy_(state0)
+    arena.arm_all(prefix_len=7)
+    y_arena = layer(block, cache=cache)
+    assert cache._tape.dtype == torch.float32
+    arena.rollback_all(torch.tensor(9, dtype=torch.int32, device=DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(y_arena, y_plain)
+    assert torch.equal(cache[1], plain[1]) and torch.equal(cache[0], plain[0])

@@ -111,3 +111,45 @@ def test_long_prompt_takes_the_attention_kernel(native_lib, monkeypatch):
     torch.cuda.synchronize()
     assert len(seen) >= 2 and all(n >= 1116 for n in seen)
     _same_or_parting_at_a_near_tie(model, prompt, spec, greedy, True)
+
+
+def test_device_tokens_against_the_host_run_of_the_same_model(native_lib, monkeypatch):
+    """The same weights, prompt and drafts decoded on the host (array operators, stock matmul:
+    the path tests/test_generate_loop.py holds to exact greedy parity) and on the device (verify
+    kernels, fused glue, tape replay).  bf16 activations are rounded in different places, so the
+    two token sequences must be equal or part at a near-tie of the HOST model's two best logits."""
+    monkeypatch.setenv("DFLASH_VERIFY_QMM", "1")
+    host = ToyHybridLM(seed=11, hidden=512, Hk=2, Hv=4, D=128, dtype=torch.bfloat16).install_hooks()
+    dev = _model(11)
+    prompt = torch.randint(0, 384, (11,), generator=torch.Generator().manual_seed(5))
+    n_new = 48
+
+    def host_cache():
+        cache = make_target_cache(host.pattern)
+        for layer, c in zip(host.layers, cache):
+            if layer.is_linear:
+                la = layer.linear_attn
+                c[1] = torch.zeros((1, la.num_v_heads, la.head_v_dim, la.head_k_dim), dtype=torch.float32)
+        return cache
+
+    host_target = lambda ids, cache: host(ids, cache)
+    host_greedy = generate_greedy(host_target, host_cache(), prompt, n_new)
+    host_spec = generate_speculative(host_target, drafts(host_greedy, 384, seed=3)["partly"], host_cache(), prompt,
+                                     n_new, block_tokens=16)
+    assert torch.equal(host_spec, host_greedy)          # the host path's own guarantee
+    history = []
+    dev_spec = generate_speculative(lambda ids, cache: dev(ids, cache), drafts(host_greedy, 384, seed=3)["partly"],
+                                    _cache(dev, True), prompt.to(DEV), n_new, block_tokens=16,
+                                    acceptance_history=history)
+    torch.cuda.synchronize()
+    assert sum(history) > 0                               # drafts were accepted: rollbacks of every length ran
+    a, b = dev_spec.cpu(), host_spec
+    n = min(a.shape[0], b.shape[0])
+    diverged = (a[:n] != b[:n]).nonzero()
+    if diverged.numel():
+        at = int(diverged[0])
+        with torch.no_grad():
+            logits = host(torch.cat([prompt, b[:at]])[None], host_cache())[0, -1].float()
+        top = torch.topk(logits, 2)
+        assert float(top.values[0] - top.values[1]) < 0.05 * float(logits.std()), (at, top.values)
+        assert {int(a[at]), int(b[at])} == set(top.indices.tolist())

@@ -72,7 +72,8 @@ def test_config0_single_call(verify_env, native_lib, c_oracle):
     assert np.max(np.abs(y - O.round_bf16(exact.astype(np.float32)))) <= 2 ** -7 * np.max(np.abs(exact))
 
 
-@pytest.mark.parametrize("K,N", [(5120, 17408), (17408, 5120), (5120, 7168), (4096, 12288),
+@pytest.mark.parametrize("K,N", [(5120, 17408), (17408, 5120), (5120, 7168), (5120, 5120), (4096, 12288),
+                                 (4096, 6144), (12288, 4096),
                                  (512, 2048), (1536, 272)])  # the last two: K a multiple of 512 only
 def test_real_projection_shapes(verify_env, native_lib, c_oracle, K, N):
     """27B / 9B projection shapes at full size, both dispatch branches."""
@@ -101,6 +102,49 @@ def test_reference_tolerances_on_reference_style_data(verify_env, native_lib, dt
     max_rel = max_abs / (float(np.max(np.abs(ref))) + 1e-3)
     assert max_abs <= (8e-3 if dtype == torch.bfloat16 else 4e-3), max_abs
     assert max_rel <= 2e-2, max_rel
+
+
+def _reference_sweep_shapes(n=30, seed=0xDF1A):
+    """The shape sweep of the reference's parity test (tests/test_verify_qmm_parity.py:43-53):
+    the same generator, seed and order of draws, hence the same 30 (M, K, N)."""
+    rng = np.random.default_rng(seed)
+    levels = [1, 4, 8, 12, 15, 16]
+    shapes = []
+    for i in range(n):
+        K = int(rng.integers(2, 40)) * 64
+        N = int(rng.integers(1, 64)) * 8
+        shapes.append((i, levels[i % len(levels)], K, N))
+    return shapes
+
+
+def _kernel_sweep_shapes():
+    """The same draws with 16 rows and N rounded up to a multiple of 32: none of the sweep's own
+    five M = 16 shapes has N % 32 == 0, so on its own it never reaches the kernel."""
+    return [(100 + i, 16, K, (N + 31) // 32 * 32) for i, _, K, N in _reference_sweep_shapes()]
+
+
+@pytest.mark.parametrize("i,M,K,N", _reference_sweep_shapes() + _kernel_sweep_shapes())
+def test_reference_shape_sweep(verify_env, native_lib, i, M, K, N):
+    """Every shape of the reference's sweep through verify_matmul on the device - M = 16 with
+    N % 32 == 0 reaches the kernel, the rest the stock route, as verify_qmm.py:276-321 decides -
+    held to the reference's bars (8e-3 abs, 2e-2 rel, test_verify_qmm_parity.py:103-109) on its
+    data recipe (x, w ~ N(0,1)/sqrt(K), weights quantised from floats)."""
+    g = torch.Generator().manual_seed(0xDF1A + i)
+    scale = 1.0 / np.sqrt(K)
+    x = (torch.randn(M, K, generator=g) * scale).to(torch.bfloat16)
+    w_fp = (torch.randn(N, K, generator=g) * scale).to(torch.bfloat16)
+    wq, s, b = quantize(w_fp, 64, 4)
+    y = VQ.verify_matmul(x.to(DEV), wq.to(DEV), s.to(DEV), b.to(DEV), group_size=64, bits=4)
+    assert tuple(y.shape) == (M, N) and y.dtype == torch.bfloat16
+    kernel = VQ._should_use_verify(x, 64, 4, True) and N % 32 == 0
+    assert kernel == (M == 16 and N % 32 == 0)
+    ref = O.qmm_kernel_semantics(x.float().numpy(), wq.numpy().view(np.uint32), s.float().numpy(),
+                                 b.float().numpy(), 64, dtype="bf16")
+    max_abs = float(np.max(np.abs(_f32(y) - ref)))
+    assert max_abs <= 8e-3, (M, K, N, max_abs)
+    assert max_abs / (float(np.max(np.abs(ref))) + 1e-3) <= 2e-2
+    exact = O.qmm_exact(x.float().numpy(), wq.numpy().view(np.uint32), s.float().numpy(), b.float().numpy(), 64)
+    _check_north_star(_f32(y).astype(np.float64), exact)
 
 
 @pytest.mark.parametrize("gs", [32, 64, 128])

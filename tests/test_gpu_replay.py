@@ -302,3 +302,55 @@ def test_arena_batched_rollback_equals_per_layer(native_lib):
     # everything accepted: the forward's state is kept, transients dropped
     s_f, _, o_f = run(True, 15)
     assert o_f == [4096 + 16] * 2
+
+
+def test_mask_with_prefix_slices_of_a_longer_tape_and_several_batch_rows(native_lib):
+    """tape[:, :a] of a 16-step recording is read in place (row count 16 per slot); the mask
+    has `a` columns.  Every batch row must see its own mask row."""
+    case = make_replay_case(1, batch=3, T=16, Hk=2, Hv=4, steps=16, seed=171, tape_dtype=torch.float32)
+    d = case.to(DEV)
+    rng = np.random.default_rng(172)
+    for a in (1, 5, 11, 16):
+        mask = rng.random((3, a)) < 0.6
+        mask[1] = True
+        m = torch.from_numpy(mask).to(DEV)
+        tape, k, g = d.tape[0][:, :a], d.k[0][:, :a], d.g[0][:, :a]
+        assert a == 16 or not tape.is_contiguous()
+        got = tape_replay_kernel(tape, k, g, d.state[0], m)
+        want = _tape_replay_ops(tape, k, g, d.state[0], m)
+        torch.cuda.synchronize()
+        assert _rel_l2(_np(got), _np(want)) <= TOL, a
+        exact = O.tape_replay_ops(_np(case.tape[0])[:, :a], _np(case.k[0])[:, :a], _np(case.g[0])[:, :a],
+                                  _np(case.state[0]), mask)
+        assert _rel_l2(_np(got), exact) <= TOL, a
+
+
+def test_arena_takes_per_batch_row_acceptance_and_other_tape_dtypes(native_lib):
+    """One accepted count per batch row on the device is spread over the layers
+    (slot = layer * B + row); a bf16 tape handed to an fp32 arena is converted."""
+    L, B, T, Hk, Hv, Dk, Dv, C = 3, 2, 16, 2, 4, 128, 128, 64
+    case = make_replay_case(L, batch=B, T=T, Hk=Hk, Hv=Hv, steps=T, seed=173)      # bf16 tape
+    gen = torch.Generator().manual_seed(174)
+    qkv = torch.randn((L, B, T, C), generator=gen).to(torch.bfloat16)
+    arena = RollbackArena(L, batch=B, max_steps=T, Hk=Hk, Hv=Hv, Dk=Dk, Dv=Dv, conv_dim=C, device=DEV)
+    assert arena.tape.dtype == torch.float32
+    caches = arena.caches()
+    for l, c in enumerate(caches):
+        c[1].copy_(case.state[l].to(DEV))
+    arena.arm_all(prefix_len=5)
+    for l, c in enumerate(caches):
+        c[1], c[0] = arena.next_state(l).normal_(), arena.next_conv(l).zero_()
+        c.record_tape(tape=case.tape[l].to(DEV), k=case.k[l].to(DEV), g=case.g[l].to(DEV), qkv=qkv[l].to(DEV))
+    acc = torch.tensor([3, 12], dtype=torch.int32, device=DEV)
+    arena.rollback_all(acc)
+    torch.cuda.synchronize()
+    for l, c in enumerate(caches):
+        for b, a in enumerate((4, 13)):
+            want = O.tape_replay_ops(_np(case.tape[l])[b:b + 1, :a], _np(case.k[l])[b:b + 1, :a],
+                                     _np(case.g[l])[b:b + 1, :a], _np(case.state[l])[b:b + 1])
+            assert _rel_l2(_np(c[1][b:b + 1]), want) <= TOL, (l, b)
+    with pytest.raises(ValueError):
+        arena.arm_all()
+        for l, c in enumerate(caches):
+            c.record_tape(tape=case.tape[l].to(DEV), k=case.k[l].to(DEV), g=case.g[l].to(DEV), qkv=qkv[l].to(DEV))
+        arena.rollback_all(torch.zeros(5, dtype=torch.int32, device=DEV))

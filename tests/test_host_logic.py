@@ -90,6 +90,18 @@ def test_eligible_call_on_host_tensors_fails_loudly(verify_env):
         VQ.verify_matmul(c.x, c.w, c.scales, c.biases)
 
 
+def test_verify_qmm_takes_group_size_and_bits_positionally(verify_env):
+    """verify_qmm(x, w_packed, scales, biases, group_size, bits): the spelling of the hot path's
+    name; ineligible calls (4 rows here) go to the stock operator like verify_matmul's."""
+    c = make_qmm_case(256, 32, 6, M=4)
+    want = VQ.verify_matmul(c.x, c.w, c.scales, c.biases, group_size=64, bits=4)
+    assert torch.equal(VQ.verify_qmm(c.x, c.w, c.scales, c.biases, 64, 4), want)
+    assert torch.equal(VQ.verify_qmm(c.x, c.w, c.scales, c.biases, group_size=64, bits=4), want)
+    with pytest.raises(nat.NativeLibraryError):          # 16 rows: the kernel path, as for verify_matmul
+        c16 = make_qmm_case(256, 32, 6)
+        VQ.verify_qmm(c16.x, c16.w, c16.scales, c16.biases, 64, 4)
+
+
 def test_stock_dequant_matches_oracle():
     c = make_qmm_case(256, 32, 5)
     w_np = c.w.numpy().view(np.uint32)
