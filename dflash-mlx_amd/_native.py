@@ -12,12 +12,22 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
 QMM_KERNEL_AUTO, QMM_KERNEL_TILE, QMM_KERNEL_STREAM = 0, 1, 2
 QMM_STATIC_SCRATCH_BYTES = 8 << 20  # DFLASH_QMM_STATIC_SCRATCH_BYTES
+QMM_CHAIN_MAX = 16                       # DFLASH_QMM_CHAIN_MAX
+QMM_CHAIN_ERROR_OFFSET = (16384 - 64 + 1) * 4  # DFLASH_QMM_CHAIN_ERROR_OFFSET
+QMM_EPILOGUE_NONE, QMM_EPILOGUE_SILU_MUL = 0, 1
+
+
+class QmmProblem(ctypes.Structure):
+    """dflash_qmm_problem of include/dflash_mi355.h."""
+    _fields_ = [("x", ctypes.c_void_p), ("w_q", ctypes.c_void_p), ("scales", ctypes.c_void_p),
+                ("biases", ctypes.c_void_p), ("y", ctypes.c_void_p), ("K", ctypes.c_int), ("N", ctypes.c_int),
+                ("wait_for", ctypes.c_int), ("epilogue", ctypes.c_int)]
 
 # every symbol include/dflash_mi355.h declares
 EXPORTED_SYMBOLS = (
@@ -26,6 +36,8 @@ EXPORTED_SYMBOLS = (
     "dflash_qmm_m16_workspace_bytes",
     "dflash_qmm_m16",
     "dflash_qmm_m16_static",
+    "dflash_qmm_m16_chain_workspace_bytes",
+    "dflash_qmm_m16_chain",
     "dflash_qmm_m16_packed_bytes",
     "dflash_qmm_m16_pack",
     "dflash_qmm_m16_packed",
@@ -63,6 +75,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     )
     lib.dflash_qmm_m16_static.restype = c.c_int
     lib.dflash_qmm_m16_static.argtypes = [c.c_void_p] * 5 + [c.c_int] * 8 + [c.c_void_p]
+    lib.dflash_qmm_m16_chain_workspace_bytes.restype = c.c_size_t
+    lib.dflash_qmm_m16_chain_workspace_bytes.argtypes = [c.POINTER(QmmProblem), c.c_int, c.c_int]
+    lib.dflash_qmm_m16_chain.restype = c.c_int
+    lib.dflash_qmm_m16_chain.argtypes = [c.POINTER(QmmProblem), c.c_int, c.c_void_p, c.c_size_t] + [c.c_int] * 4 + [c.c_void_p]
     lib.dflash_qmm_m16_packed_bytes.restype = c.c_int
     lib.dflash_qmm_m16_packed_bytes.argtypes = [c.c_int] * 3 + [c.POINTER(c.c_size_t)] * 2
     lib.dflash_qmm_m16_pack.restype = c.c_int

@@ -14,7 +14,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libdflash_mi355.so")
 
-SOURCES = ["api.hip", "qmm_m16.hip", "qmm_m16_stream.hip", "tape_replay.hip", "gdn_forward.hip", "gdn_glue.hip", "sdpa_q16.hip",
+SOURCES = ["api.hip", "qmm_m16.hip", "qmm_m16_stream.hip", "qmm_m16_chain.hip", "tape_replay.hip", "gdn_forward.hip", "gdn_glue.hip", "sdpa_q16.hip",
            "conv_state.hip"]
 
 HIPCC_FLAGS = [

@@ -1,0 +1,763 @@
+// Chained M=16 int4 qmm for gfx950: several matrices in ONE launch.
+//
+// A verify step calls the quantized matmul once per projection (dflash_mlx/verify_linear.py:
+// 103-143, five times per layer), and a launch of the streaming kernel (qmm_m16_stream.hip)
+// spends more time around its weight stream than in it: the gap between two kernels of a
+// stream, the first memory round trips of cold workgroups, the split-K hand-over at the end.
+// This kernel runs a list of problems  y_p[16, N_p] = x_p[16, K_p] . (s*q + b)_p^T  back to back
+// inside one persistent grid.  Every problem is divided among the workgroups exactly as a
+// launch of its own would divide it (same grid rule, same unit ranges, same order of partial
+// sums: results are bit for bit those of separate launches), but the ring of LDS slots never
+// drains: while the workers of a workgroup finish problem p and hand over its partial tiles,
+// its loaders already stream the first units of problem p + 1.  Weights never depend on
+// activations; only x does:
+//
+//  * a problem whose x is the y of an earlier problem of the chain (wait_for) has its codes,
+//    scales and biases prefetched like any other, its x loads held back until the earlier
+//    problem's row blocks have all been stored (a counter per problem, bumped at agent scope
+//    after the stores are acknowledged; x is then read around the L2, which is per XCD).  The
+//    wait is bounded: after spin_limit polls a workgroup records an error word, goes on with
+//    whatever x holds, and the launch ends normally.
+//  * an epilogue turns a gate/up pair into the MLP's hidden activation inside the launch:
+//    the matrix holds gate rows then up rows, a row block takes 64 rows of each, and the
+//    workgroup that finishes it stores silu(gate) * up (each factor rounded to the activation
+//    type first, as separate operators would) - which the down projection then waits for.
+//
+// Everything else - units of 128 rows x 256 k, 8 worker + 4 loader waves, direct-to-LDS loads
+// into a ring, hand-written LDS reads, bare barriers - is the streaming kernel's, see there.
+#include <cstdlib>
+
+#include "dflash_common.h"
+#include "qmm_stream_device.h"
+
+namespace dflash {
+namespace stream {
+
+constexpr int kMaxChain = DFLASH_QMM_CHAIN_MAX;
+constexpr int kChainAhead = 3;  // units issued beyond the one being consumed
+// LDS behind the two rings: last-arriver flags, then the up half of an epilogue row block
+// (4 tiles of 1 KiB) for each of the two row blocks a workgroup can be last at.
+constexpr int kChainFlags = kLdsBytes;
+constexpr int kChainExchange = kChainFlags + 64;
+constexpr int kLdsBytesChain = kChainExchange + 2 * 4096;  // 152.1 KiB
+// The last words of the 64 KiB counter block: launch bookkeeping of chains.
+constexpr int kChainStatusWord = 16384 - 64;  // [0] exit counter, [1] error word
+constexpr int kChainDoneWord = kChainStatusWord + 8;  // [kMaxChain] row blocks stored, per problem
+constexpr int kChainCounterWords = kChainStatusWord;
+
+struct ChainProblem {
+  const uint16_t* x;
+  const uint32_t* w;
+  const uint16_t* scales;
+  const uint16_t* biases;
+  uint16_t* y;
+  int K, N;          // N counts the rows of w (gate and up rows for the epilogue)
+  int grid;          // workgroups that take part: what a launch of its own would use
+  int counter_base;  // first arrival counter of this problem
+  int partial_base;  // first partial tile of this problem (tiles of kPartialFloats floats)
+  int wait_for;      // earlier problem whose y is this x, or -1
+  int epilogue;      // DFLASH_QMM_EPILOGUE_*
+  int signal;        // a later problem waits for this one
+};
+struct ChainParams {
+  ChainProblem prob[kMaxChain];
+  int count;
+  float* partials;
+  uint32_t* counters;
+  int has_deps;
+  int spin_limit;
+};
+
+// The kernel reads its argument block in place, through the constant address space: a
+// reference to a by-value struct argument that is indexed at run time would make the compiler
+// copy the whole block into per-thread memory.
+typedef const __attribute__((address_space(4))) ChainProblem CProblem;
+typedef const __attribute__((address_space(4))) ChainParams CParams;
+
+// How one problem is divided: this workgroup's range of units, or wg < 0 if it has none.
+struct Range {
+  int stages, RB, units, grid, wg;
+  int u0, u1, rb0, st0;
+};
+__device__ __forceinline__ Range problem_range(CProblem& q, int block, int nblocks) {
+  Range r;
+  r.stages = q.K / kUnitK;
+  r.RB = (q.N + kRows - 1) / kRows;
+  r.units = r.RB * r.stages;
+  r.grid = q.grid;
+  // Workgroups are dealt to the eight XCDs in turn (block % 8); unit ranges follow the XCD-major
+  // order, so that the neighbours that share a row block sit behind one L2 (as a launch of its
+  // own with `grid` workgroups would place them).
+  if (r.grid % 8 == 0 && nblocks % 8 == 0) {
+    const int per = r.grid / 8, slot = block / 8;
+    r.wg = slot < per ? (block % 8) * per + slot : -1;
+  } else {
+    r.wg = block < r.grid ? block : -1;
+  }
+  r.u0 = r.u1 = r.rb0 = r.st0 = 0;
+  if (r.wg >= 0) {
+    r.u0 = range_begin(r.units, r.wg, r.grid);
+    r.u1 = range_begin(r.units, r.wg + 1, r.grid);
+    r.rb0 = r.u0 / r.stages;
+    r.st0 = r.u0 - r.rb0 * r.stages;
+  }
+  return r;
+}
+
+// Row of w behind row v (0..127) of row block rb.  Plain: 128 rb + v.  Epilogue: the first 64
+// rows are gate rows 64 rb .., the other 64 the up rows of the same output columns.
+__device__ __forceinline__ int weight_row(CProblem& q, int rb, int v) {
+  if (q.epilogue == DFLASH_QMM_EPILOGUE_SILU_MUL) {
+    const int half_rows = q.N >> 1;
+    int r = 64 * rb + (v & 63);
+    r = r < half_rows ? r : half_rows - 1;
+    return v < 64 ? r : half_rows + r;
+  }
+  const int r = kRows * rb + v;
+  return r < q.N ? r : q.N - 1;
+}
+
+__device__ __forceinline__ void load16_to_lds_coherent(const void* gptr, char* lds_base) {
+  __builtin_amdgcn_global_load_lds((global_cvoid_t*)gptr, (lds_void_t*)lds_base, 16, 0, 16);  // sc1
+}
+
+template <bool FP16>
+__device__ __forceinline__ float silu_mul(float g, float u) {
+  using A = Act<FP16>;
+  // each factor as the activation type would hold it between separate operators
+  g = A::to_f32(A::from_f32(g));
+  u = A::to_f32(A::from_f32(u));
+  const float s = A::to_f32(A::from_f32(g / (1.0f + __expf(-g))));
+  return s * u;
+}
+
+template <bool ACT_FP16, bool SB_FP16>
+__global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_value) {
+  using A = Act<ACT_FP16>;
+  (void)by_value;  // the first (and only) argument: offset 0 of the argument block
+  CParams& p = *(CParams*)__builtin_amdgcn_kernarg_segment_ptr();
+  constexpr int CHUNK = 4;
+  constexpr int SBROW = 8 * CHUNK;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t lds0 = lds_address(lds);
+  const int block = (int)blockIdx.x, nblocks = (int)gridDim.x;
+  uint32_t* const status = p.counters + kChainStatusWord;
+  uint32_t* const done = p.counters + kChainDoneWord;
+
+  // Both kinds of wave walk the same problems and units and pass the same barriers.  Per
+  // problem this workgroup takes part in:
+  //   one at its start (its first unit has landed),
+  //   one per unit u (the next unit of the problem has landed; every worker holds unit u in
+  //     registers, so the slot of unit u is free),
+  //   when a row block ends with unit u: one more (the slot of unit u carries the cross-wave
+  //     sum), and with an epilogue another one (the up half crosses to the gate half's waves),
+  //   after the last unit, if a row block was shared with other workgroups: two more (partial
+  //     tiles stored / arrival counters bumped), with an epilogue a third,
+  //   if a later problem waits for this one: one more (outputs stored).
+
+  if (wave >= kWaves) {
+    // ================================ loader waves ====================================
+    // See qmm_m16_stream.hip for which loader issues which 16-byte pieces of a unit.  The loop
+    // below is flat on purpose: one place that issues units, one that waits, one that opens a
+    // problem.  (A loader may not spill: spill traffic would count as loads of its own.)
+    const int ld = wave - kWaves;
+    const int w_r = lane >> 3;
+    const int w_c = (lane & 7) ^ (((w_r >> 1) & 3) << 1);
+
+    // ---- issue cursor: runs kChainAhead units ahead of the workers, across problems -----
+    enum { NEED_OPEN, OPEN, PARKED, EXHAUSTED };
+    int i_state = NEED_OPEN;
+    int ip = -1;  // problem being issued
+    Range ir{};
+    int iu = 0, irb = 0, ist = 0;   // next unit to issue: index, row block, stage
+    bool i_first = false;           // it is the first unit of this workgroup's range
+    bool i_coherent = false;        // x of problem ip is written by this launch
+    bool i_ready = true;            // ... and is known to be complete
+    // byte offsets of this lane's pieces from the problem's x, w and scales (= biases) arrays
+    uint32_t xo[2] = {0u, 0u}, wo[4] = {0u, 0u, 0u, 0u}, so = 0u;
+    int slot_i = 0, sb_slot_i = 0;
+    int n_issued = 0, n_cons = 0;   // units issued / units whose barrier has passed
+    int tot = 0;                    // loads this wave has issued
+    int mark0 = 0, mark1 = 0, mark2 = 0, mark3 = 0, fifo_n = 0;  // `tot` after each unit not yet waited for
+    int def_n = 0, def_slot = 0, def_st = 0;  // units of problem ip issued without their x
+
+    auto set_row_block = [&](int rb) __attribute__((always_inline)) {
+      CProblem& q = p.prob[ip];
+      const uint32_t row_bytes = (uint32_t)q.K >> 1;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        wo[i] = (uint32_t)weight_row(q, rb, 8 * (ld + 4 * i) + w_r) * row_bytes + w_c * 16;
+      so = (uint32_t)weight_row(q, rb, 32 * ld + (lane >> 1)) * (uint32_t)(q.K / kGS * 2) + (lane & 1) * 16;
+    };
+    auto issue_x = [&](int st, int slot) __attribute__((always_inline)) {
+      CProblem& q = p.prob[ip];
+      char* dst = lds + slot * kSlotBytes + kXOffset;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const char* src = (const char*)q.x + (xo[i] + (uint32_t)st * (kUnitK * 2));
+        if (i_coherent)
+          load16_to_lds_coherent(src, dst + (ld + 4 * i) * 1024);
+        else
+          load16_to_lds(src, dst + (ld + 4 * i) * 1024);
+      }
+      tot += 2;
+    };
+
+    // ---- consume cursor: mirrors the workers' barriers ---------------------------------
+    enum { START, UNIT, END, FINISHED };
+    int phase = FINISHED;
+    int cp = -1;
+    Range cr{};
+    int u = 0, rb_left = 0, in_rb = 0;
+    bool any_shared = false;
+    auto next_problem = [&]() __attribute__((always_inline)) {
+      phase = FINISHED;
+      while (++cp < p.count) {
+        cr = problem_range(p.prob[cp], block, nblocks);
+        if (cr.wg >= 0) {
+          phase = START;
+          break;
+        }
+      }
+    };
+    next_problem();
+
+#pragma unroll 1
+    while (phase != FINISHED) {
+      // ---- keep kChainAhead units issued beyond the one being consumed ------------------
+#pragma unroll 1
+      while (n_issued - n_cons < kChainAhead) {
+        if (i_state == NEED_OPEN) {
+          i_state = EXHAUSTED;
+          while (++ip < p.count) {
+            ir = problem_range(p.prob[ip], block, nblocks);
+            if (ir.wg >= 0) {
+              i_state = OPEN;
+              break;
+            }
+          }
+          if (i_state == OPEN) {
+            CProblem& q = p.prob[ip];
+            iu = ir.u0, irb = ir.rb0, ist = ir.st0;
+            i_first = true;
+            i_coherent = q.wait_for >= 0;
+            i_ready = !i_coherent;
+            const int xrow = lane & 15;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+              const int xi = ld + 4 * i;
+              xo[i] = (uint32_t)(xrow * q.K + (xi >> 1) * kGS + (2 * (xi & 1) + (lane >> 5)) * 16 +
+                                 ((lane >> 4) & 1) * 8) * 2u;
+            }
+            set_row_block(irb);
+          }
+        }
+        if (i_state != OPEN) break;
+        // ---- one unit: scales/biases with the first unit of a chunk or of the range, x unless
+        // it is still being computed, codes
+        CProblem& q = p.prob[ip];
+        char* slot = lds + slot_i * kSlotBytes;
+        if ((ist % CHUNK) == 0 || i_first) {
+          char* sb = lds + kSbOffset + sb_slot_i * kSbSlotBytes;
+          const uint32_t off = so + (uint32_t)(ist / CHUNK) * (CHUNK * kGroups * 2);
+          load16_to_lds((const char*)q.scales + off, sb + ld * 1024);
+          load16_to_lds((const char*)q.biases + off, sb + kSbArrayBytes + ld * 1024);
+          tot += 2;
+          if (++sb_slot_i == kSbDepth) sb_slot_i = 0;
+        }
+        i_first = false;
+        if (i_ready) {
+          issue_x(ist, slot_i);
+        } else {
+          if (def_n == 0) def_slot = slot_i, def_st = ist;
+          ++def_n;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          load16_to_lds_stream((const char*)q.w + (wo[i] + (uint32_t)ist * (kUnitK / 2)), slot + (ld + 4 * i) * 1024);
+        tot += 4;
+        // remember where this unit's loads end
+        if (fifo_n == 0) mark0 = tot;
+        else if (fifo_n == 1) mark1 = tot;
+        else if (fifo_n == 2) mark2 = tot;
+        else mark3 = tot;
+        ++fifo_n;
+        ++n_issued;
+        if (++slot_i == kDepth) slot_i = 0;
+        if (++iu == ir.u1) {
+          // A problem with held-back x loads keeps the cursor until they have been issued: the
+          // cursor never enters a second problem whose x is still being computed.
+          i_state = def_n == 0 ? NEED_OPEN : PARKED;
+        } else if (++ist == ir.stages) {
+          ist = 0;
+          ++irb;
+          set_row_block(irb);
+        }
+      }
+
+      if (phase == END) {
+        if (any_shared) {
+          asm volatile("s_barrier" ::: "memory");
+          asm volatile("s_barrier" ::: "memory");
+          if (p.prob[cp].epilogue == DFLASH_QMM_EPILOGUE_SILU_MUL) asm volatile("s_barrier" ::: "memory");
+        }
+        if (p.prob[cp].signal) asm volatile("s_barrier" ::: "memory");
+        next_problem();
+        continue;
+      }
+
+      if (phase == START && p.prob[cp].wait_for >= 0) {
+        // The x of problem cp is the y of an earlier problem: wait (bounded) until all its row
+        // blocks have been stored, then issue the x loads that were held back.  The issue
+        // cursor is on problem cp (inside it, or parked at its end).
+        CProblem& q = p.prob[cp];
+        const uint32_t want = (uint32_t)((p.prob[q.wait_for].N + kRows - 1) / kRows);  // its row blocks
+        int polls = 0;
+        while (__hip_atomic_load(&done[q.wait_for], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < want) {
+          if (++polls > p.spin_limit) {
+            if (lane == 0 && ld == 0)
+              __hip_atomic_store(&status[1], (uint32_t)(cp + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
+          __builtin_amdgcn_s_sleep(8);
+        }
+        if (ip == cp) {
+          int st = def_st, slot = def_slot;
+#pragma unroll 1
+          for (int j = 0; j < def_n; ++j) {
+            issue_x(st, slot);
+            // a held-back unit ends with its x loads (nothing else is waiting to be waited for:
+            // every unit of the problems before cp has been consumed)
+            if (j == 0) mark0 = tot;
+            else if (j == 1) mark1 = tot;
+            else if (j == 2) mark2 = tot;
+            else mark3 = tot;
+            if (++st == ir.stages) st = 0;
+            if (++slot == kDepth) slot = 0;
+          }
+          def_n = 0;
+          i_ready = true;
+          if (i_state == PARKED) i_state = NEED_OPEN;
+        }
+      }
+      // START: the first unit of problem cp has landed.  UNIT: unit u + 1 has landed, and every
+      // worker holds unit u in registers, so its slot is free.
+      if (phase == START || u + 1 < cr.u1) {
+        wait_loads(tot - mark0);
+        mark0 = mark1, mark1 = mark2, mark2 = mark3;
+        --fifo_n;
+      }
+      asm volatile("s_barrier" ::: "memory");
+      if (phase == START) {
+        u = cr.u0;
+        rb_left = cr.stages - cr.st0;
+        in_rb = 0;
+        any_shared = false;
+        phase = UNIT;
+        continue;
+      }
+      ++n_cons;
+      ++in_rb;
+      if (--rb_left == 0 || u + 1 == cr.u1) {
+        asm volatile("s_barrier" ::: "memory");
+        if (p.prob[cp].epilogue == DFLASH_QMM_EPILOGUE_SILU_MUL) asm volatile("s_barrier" ::: "memory");
+        if (in_rb != cr.stages) any_shared = true;
+        in_rb = 0;
+        rb_left = cr.stages;
+      }
+      if (++u == cr.u1) phase = END;
+    }
+    return;
+  }
+
+  // ================================== worker waves ====================================
+  const int col = lane & 15;
+  const int kblk = lane >> 4;
+  const uint4 ones = make_uint4(A::kOnes, A::kOnes, A::kOnes, A::kOnes);
+  uint32_t mask = 0x000F000Fu, magic = A::kMagic;
+  asm volatile("" : "+s"(mask), "+v"(magic));
+  const int grp = wave & 3;    // quantisation group of the unit this wave works on
+  const int half = wave >> 2;  // rows 64*half .. 64*half + 63: tiles j = 0..3
+  const uint32_t xoff =
+      lds0 + kXOffset + grp * 2048 + (kblk >> 1) * 1024 + (16 * (2 * (kblk & 1)) + col) * 16;
+  const uint32_t wrow = 64 * half + col;
+  const uint32_t woff =
+      lds0 + wrow * 128 + ((grp ^ ((wrow >> 1) & 3)) << 5) + (kblk >> 1) * 16 + (kblk & 1) * 8;
+  const uint32_t soff = lds0 + kSbOffset + wrow * SBROW + grp * 2;
+
+  int rd_slot = 0;            // byte offset of the ring slot of the unit whose operands are fetched next
+  int rd_sb = -kSbSlotBytes;  // byte offset of its scale/bias slot
+  int cur_slot = 0;           // byte offset of the current unit's ring slot
+  f32x4_t acc4[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc4[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  Operands op[2];
+
+#pragma unroll 1
+  for (int cp = 0; cp < p.count; ++cp) {
+    const Range cr = problem_range(p.prob[cp], block, nblocks);
+    if (cr.wg < 0) continue;
+    CProblem& q = p.prob[cp];
+    const bool epi = q.epilogue == DFLASH_QMM_EPILOGUE_SILU_MUL;
+    const int n_out = epi ? q.N >> 1 : q.N;  // columns of y
+    float* const partials = p.partials + (size_t)q.partial_base * kPartialFloats;
+    uint32_t* const counters = p.counters + q.counter_base;
+    int emitted = 0;  // row blocks of this problem whose output this workgroup has stored
+
+    int rd_q = cr.st0 % CHUNK;
+    bool rd_first = true;
+    uint32_t rd_x, rd_w, rd_s;
+    auto next_addresses = [&]() __attribute__((always_inline)) {
+      if (rd_q == 0 || rd_first) {
+        rd_sb += kSbSlotBytes;
+        if (rd_sb == kSbDepth * kSbSlotBytes) rd_sb = 0;
+        rd_first = false;
+      }
+      rd_x = xoff + rd_slot;
+      rd_w = woff + rd_slot;
+      rd_s = soff + rd_sb + rd_q * 8;
+      rd_slot += kSlotBytes;
+      if (rd_slot == kDepth * kSlotBytes) rd_slot = 0;
+      rd_q = (rd_q + 1) & (CHUNK - 1);
+    };
+
+    // Stores tile `wave` of row block rb.  Accumulator r of lane l is (m = 4*(l/16) + r,
+    // column 16*wave + l%16) of the row block.  With the epilogue, waves 0..3 hold the gate
+    // half and `other` the up half of the same 64 output columns; waves 4..7 store nothing.
+    auto store_out = [&](size_t index, float v) __attribute__((always_inline)) {
+      const uint16_t bits = (uint16_t)A::from_f32(v);
+      if (q.signal)
+        __hip_atomic_store(&q.y[index], bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else
+        q.y[index] = bits;
+    };
+    auto emit = [&](int rb, const f32x4_t& acc) __attribute__((always_inline)) {
+      const int n = rb * kRows + 16 * wave + col;
+      if (n >= n_out) return;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) store_out((size_t)(4 * kblk + r) * n_out + n, acc[r]);
+    };
+    auto emit_epilogue = [&](int rb, const f32x4_t& gate, const f32x4_t& up) __attribute__((always_inline)) {
+      const int n = rb * 64 + 16 * wave + col;
+      if (wave >= 4 || n >= n_out) return;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        store_out((size_t)(4 * kblk + r) * n_out + n, silu_mul<ACT_FP16>(gate[r], up[r]));
+    };
+    // The up half's waves (4..7) hand their tile to the gate half's (0..3) through LDS.
+    auto exchange_write = [&](int which, const f32x4_t& acc) __attribute__((always_inline)) {
+      if (wave >= 4) {
+        const uint32_t addr = lds0 + kChainExchange + which * 4096 + (wave - 4) * 1024 + lane * 16;
+        asm volatile("ds_write_b128 %0, %1\n s_waitcnt lgkmcnt(0)" : : "v"(addr), "v"(acc) : "memory");
+      }
+    };
+    auto exchange_read = [&](int which) __attribute__((always_inline)) -> f32x4_t {
+      f32x4_t v = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if (wave < 4) {
+        const uint32_t addr = lds0 + kChainExchange + which * 4096 + wave * 1024 + lane * 16;
+        asm volatile("ds_read_b128 %0, %1\n s_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
+      }
+      return v;
+    };
+
+    asm volatile("s_barrier" ::: "memory");  // the first unit of this problem has landed
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc4[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    next_addresses();
+    operands_issue_piece<0, SBROW>(rd_x, rd_w, rd_s, op[0], acc4[0]);
+    operands_issue_piece<1, SBROW>(rd_x, rd_w, rd_s, op[0], acc4[0]);
+    operands_issue_piece<2, SBROW>(rd_x, rd_w, rd_s, op[0], acc4[0]);
+    operands_issue_piece<3, SBROW>(rd_x, rd_w, rd_s, op[0], acc4[0]);
+    operands_wait(op[0], acc4[0], acc4[1], acc4[2], acc4[3]);
+    // The second operand set holds nothing yet (it is filled while the first unit is worked
+    // on): saying so keeps its registers free during the hand-over at the end of a problem.
+    asm volatile("" : "=v"(op[1].f0), "=v"(op[1].f1), "=v"(op[1].wq[0]), "=v"(op[1].wq[1]), "=v"(op[1].wq[2]),
+                 "=v"(op[1].wq[3]));
+    asm volatile("" : "=v"(op[1].sv[0]), "=v"(op[1].sv[1]), "=v"(op[1].sv[2]), "=v"(op[1].sv[3]),
+                 "=v"(op[1].bv[0]), "=v"(op[1].bv[1]), "=v"(op[1].bv[2]), "=v"(op[1].bv[3]));
+
+    int left = cr.u1 - cr.u0;         // units still to consume, the current one included
+    int rb_left = cr.stages - cr.st0;  // same, within the current row block
+    int in_rb = 0;                     // units of the current row block this workgroup has done
+    int rb = cr.rb0;
+    int shared_rb[2] = {-1, -1};       // row blocks whose partial tiles I have stored
+
+#pragma unroll 1
+    while (left > 0) {
+#pragma unroll
+      for (int par = 0; par < 2; ++par) {
+        if (left > 0) {
+          Operands& cur = op[par];
+          Operands& nxt = op[par ^ 1];
+          asm volatile("s_barrier" ::: "memory");
+          const bool fetch = left > 1;
+          if (fetch) next_addresses();
+          consume_unit<ACT_FP16, SB_FP16, SBROW>(cur, nxt, fetch, rd_x, rd_w, rd_s, acc4, ones, mask, magic);
+          if (fetch) operands_wait(nxt, acc4[0], acc4[1], acc4[2], acc4[3]);
+          --left;
+          ++in_rb;
+          if (--rb_left == 0 || left == 0) {
+            // ---- a row block ends inside my range -------------------------------------------
+            const uint32_t sbase = lds0 + cur_slot;
+            reduce_groups_write(sbase, acc4, wave, lane);
+            asm volatile("s_barrier" ::: "memory");
+            const f32x4_t acc = reduce_groups_read(sbase, acc4, wave, lane);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc4[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            const bool whole = in_rb == cr.stages;
+            if (epi) {
+              if (whole) exchange_write(0, acc);
+              asm volatile("s_barrier" ::: "memory");
+              if (whole) emit_epilogue(rb, acc, exchange_read(0));
+            } else if (whole) {
+              emit(rb, acc);
+            }
+            if (whole) {
+              ++emitted;
+            } else {
+              // Other workgroups hold the rest of this row block: partial slot 0 for the row
+              // block my range starts in, slot 1 for the one it ends in.
+              const int which = rb == cr.rb0 ? 0 : 1;
+              store_partial(partials + ((size_t)cr.wg * 2 + which) * kPartialFloats + tid * 4, acc);
+              shared_rb[which] = rb;
+            }
+            ++rb;
+            in_rb = 0;
+            rb_left = cr.stages;
+          }
+          cur_slot += kSlotBytes;
+          if (cur_slot == kDepth * kSlotBytes) cur_slot = 0;
+        }
+      }
+      // an odd number of units leaves the operands of the next problem's first unit to op[0]
+    }
+
+    if (shared_rb[0] >= 0 || shared_rb[1] >= 0) {
+      // ---- arrival at the shared row blocks (see qmm_m16_stream.hip) -----------------------
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      asm volatile("s_barrier" ::: "memory");
+      int wg_lo[2], wg_hi[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int lo = shared_rb[i] * cr.stages;
+        wg_lo[i] = (int)((((unsigned)lo + 1u) * (unsigned)cr.grid + cr.units - 1) / (unsigned)cr.units) - 1;
+        wg_hi[i] = (int)((((unsigned)(lo + cr.stages)) * (unsigned)cr.grid + cr.units - 1) / (unsigned)cr.units) - 1;
+      }
+      if (tid == 0) {
+        uint32_t prev[2] = {0u, 0u}, flag[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          if (shared_rb[i] >= 0) prev[i] = atomicInc(&counters[shared_rb[i]], (uint32_t)(wg_hi[i] - wg_lo[i]));
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          flag[i] = (shared_rb[i] >= 0 && prev[i] == (uint32_t)(wg_hi[i] - wg_lo[i])) ? 1u : 0u;
+        asm volatile("ds_write_b32 %0, %1\n ds_write_b32 %0, %2 offset:4\n s_waitcnt lgkmcnt(0)"
+                     :
+                     : "v"(lds0 + kChainFlags), "v"(flag[0]), "v"(flag[1])
+                     : "memory");
+      }
+      asm volatile("s_barrier" ::: "memory");
+      uint32_t last0, last1;
+      asm volatile("ds_read_b32 %0, %2\n ds_read_b32 %1, %2 offset:4\n s_waitcnt lgkmcnt(0)"
+                   : "=&v"(last0), "=&v"(last1)
+                   : "v"(lds0 + kChainFlags)
+                   : "memory");
+      const bool is_last[2] = {__builtin_amdgcn_readfirstlane(last0) != 0,
+                               __builtin_amdgcn_readfirstlane(last1) != 0};
+      auto sources = [&](int i, int wg0, const float* (&src)[8]) __attribute__((always_inline)) {
+        const int lo = shared_rb[i] * cr.stages;
+        const int which_first = range_begin(cr.units, wg_lo[i], cr.grid) < lo ? 1 : 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int w = wg0 + j <= wg_hi[i] ? wg0 + j : wg_hi[i];
+          src[j] = partials + ((size_t)w * 2 + (w == wg_lo[i] ? which_first : 0)) * kPartialFloats + tid * 4;
+        }
+      };
+      auto add_round = [&](int i, int wg0, const f32x4_t (&v)[8], f32x4_t& acc) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if (wg0 + j <= wg_hi[i]) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[r] += v[j][r];
+          }
+        }
+      };
+      f32x4_t sum[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        sum[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        if (!is_last[i]) continue;
+        for (int wg0 = wg_lo[i]; wg0 <= wg_hi[i]; wg0 += 8) {
+          const float* src[8];
+          sources(i, wg0, src);
+          f32x4_t v[8];
+          load_partials8(src, v);
+          add_round(i, wg0, v, sum[i]);
+        }
+        if (!epi) emit(shared_rb[i], sum[i]);
+        ++emitted;
+      }
+      if (epi) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          if (is_last[i]) exchange_write(i, sum[i]);
+        asm volatile("s_barrier" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          if (is_last[i]) emit_epilogue(shared_rb[i], sum[i], exchange_read(i));
+      }
+    }
+
+    if (q.signal) {
+      // every worker's output stores acknowledged, then one bump of the problem's counter
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      asm volatile("s_barrier" ::: "memory");
+      if (tid == 0 && emitted > 0)
+        __hip_atomic_fetch_add(&done[cp], (uint32_t)emitted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+
+  if (p.has_deps && tid == 0) {
+    // The last workgroup to leave puts the problems' counters back to zero for the next launch
+    // (every waiting workgroup has passed its waits by then).
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const uint32_t prev = atomicInc(&status[0], (uint32_t)(nblocks - 1));
+    if (prev == (uint32_t)(nblocks - 1)) {
+      for (int i = 0; i < p.count; ++i)
+        __hip_atomic_store(&done[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+}  // namespace stream
+
+// ---------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------
+int qmm_stream_grid();
+int qmm_stream_pick_grid(int units, int row_blocks, int cus);
+bool qmm_stream_eligible(int K, int N, int group_size);
+
+namespace {
+bool chain_problem_ok(const dflash_qmm_problem& q, int group_size) {
+  if (!qmm_stream_eligible(q.K, q.N, group_size) || q.K % (stream::kUnitK * 4) != 0) return false;
+  if ((long long)q.N * q.K / 2 >= (1ll << 32)) return false;  // 32-bit byte offsets inside a matrix
+  if (q.epilogue == DFLASH_QMM_EPILOGUE_SILU_MUL) return q.N % 128 == 0;  // 64 rows of each half per row block
+  return q.epilogue == DFLASH_QMM_EPILOGUE_NONE;
+}
+int chain_row_blocks(const dflash_qmm_problem& q) { return (q.N + stream::kRows - 1) / stream::kRows; }
+}  // namespace
+
+size_t qmm_chain_workspace_bytes(const dflash_qmm_problem* problems, int count, int group_size) {
+  if (!problems || count <= 0 || count > stream::kMaxChain) return 0;
+  const int cus = qmm_stream_grid();
+  size_t tiles = 0;
+  for (int i = 0; i < count; ++i) {
+    if (!chain_problem_ok(problems[i], group_size)) return 0;
+    const int rbs = chain_row_blocks(problems[i]);
+    tiles += 2 * (size_t)qmm_stream_pick_grid(rbs * (problems[i].K / stream::kUnitK), rbs, cus);
+  }
+  return (size_t)64 * 1024 + tiles * stream::kPartialFloats * sizeof(float);
+}
+
+int qmm_chain_launch(const dflash_qmm_problem* problems, int count, void* workspace,
+                     size_t workspace_bytes, int group_size, int act_dtype, int sb_dtype,
+                     int spin_limit, hipStream_t stream) {
+  using namespace stream;
+  DFLASH_REQUIRE(problems && count > 0, DFLASH_ERR_ARG, "dflash_qmm_m16_chain: no problems");
+  DFLASH_REQUIRE(count <= kMaxChain, DFLASH_ERR_SHAPE, "dflash_qmm_m16_chain: at most %d problems per launch, got %d",
+                 kMaxChain, count);
+  ChainParams p{};
+  const int cus = qmm_stream_grid();
+  int counters = 0, tiles = 0;
+  for (int i = 0; i < count; ++i) {
+    const dflash_qmm_problem& q = problems[i];
+    DFLASH_REQUIRE(q.x && q.w_q && q.scales && q.biases && q.y, DFLASH_ERR_ARG,
+                   "dflash_qmm_m16_chain: null operand in problem %d", i);
+    DFLASH_REQUIRE(chain_problem_ok(q, group_size), DFLASH_ERR_SHAPE,
+                   "dflash_qmm_m16_chain: problem %d needs group_size 64, K %% 1024 == 0, N %% 16 == 0 "
+                   "(N %% 128 == 0 with an epilogue), less than 4 GiB of codes and a known epilogue "
+                   "(K=%d N=%d gs=%d epilogue=%d)",
+                   i, q.K, q.N, group_size, q.epilogue);
+    DFLASH_REQUIRE(((uintptr_t)q.x % 16) == 0 && ((uintptr_t)q.w_q % 16) == 0 && ((uintptr_t)q.scales % 16) == 0 &&
+                       ((uintptr_t)q.biases % 16) == 0,
+                   DFLASH_ERR_ARG, "dflash_qmm_m16_chain: operands of problem %d must be 16-byte aligned", i);
+    DFLASH_REQUIRE(q.wait_for >= -1 && q.wait_for < i, DFLASH_ERR_ARG,
+                   "dflash_qmm_m16_chain: problem %d can only wait for an earlier problem (wait_for=%d)", i,
+                   q.wait_for);
+    if (q.wait_for >= 0) {
+      const dflash_qmm_problem& src = problems[q.wait_for];
+      const int src_cols = src.epilogue == DFLASH_QMM_EPILOGUE_SILU_MUL ? src.N / 2 : src.N;
+      DFLASH_REQUIRE(q.x == src.y && q.K == src_cols, DFLASH_ERR_ARG,
+                     "dflash_qmm_m16_chain: problem %d waits for problem %d, so its x must be that problem's y "
+                     "[16, %d] (K=%d)", i, q.wait_for, src_cols, q.K);
+      p.prob[q.wait_for].signal = 1;
+      p.has_deps = 1;
+    }
+    ChainProblem& d = p.prob[i];
+    d.x = (const uint16_t*)q.x;
+    d.w = q.w_q;
+    d.scales = (const uint16_t*)q.scales;
+    d.biases = (const uint16_t*)q.biases;
+    d.y = (uint16_t*)q.y;
+    d.K = q.K;
+    d.N = q.N;
+    const int rbs = chain_row_blocks(q);
+    d.grid = qmm_stream_pick_grid(rbs * (q.K / kUnitK), rbs, cus);
+    d.counter_base = counters;
+    d.partial_base = tiles;
+    d.wait_for = q.wait_for;
+    d.epilogue = q.epilogue;
+    counters += rbs;
+    tiles += 2 * d.grid;
+  }
+  DFLASH_REQUIRE(counters <= kChainCounterWords, DFLASH_ERR_SHAPE,
+                 "dflash_qmm_m16_chain: %d row blocks in one chain, at most %d", counters, kChainCounterWords);
+  const size_t need = (size_t)64 * 1024 + (size_t)tiles * kPartialFloats * sizeof(float);
+  DFLASH_REQUIRE(workspace && workspace_bytes >= need, DFLASH_ERR_WORKSPACE,
+                 "dflash_qmm_m16_chain: workspace of %zu bytes needed, %zu given", need,
+                 workspace ? workspace_bytes : (size_t)0);
+  p.count = count;
+  p.counters = (uint32_t*)workspace;
+  p.partials = (float*)((char*)workspace + 64 * 1024);
+  p.spin_limit = spin_limit > 0 ? spin_limit : (1 << 22);
+
+  const bool a16 = act_dtype == DFLASH_FP16, s16 = sb_dtype == DFLASH_FP16;
+  const void* fn = a16 ? (s16 ? (const void*)qmm_chain_kernel<true, true> : (const void*)qmm_chain_kernel<true, false>)
+                       : (s16 ? (const void*)qmm_chain_kernel<false, true> : (const void*)qmm_chain_kernel<false, false>);
+  static bool attr_set[kMaxDevices][4] = {};
+  const int idx = (a16 ? 2 : 0) + (s16 ? 1 : 0);
+  const int slot = current_device_slot();
+  if (!attr_set[slot][idx] || slot == kMaxDevices - 1) {
+    DFLASH_HIP_OK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytesChain));
+    attr_set[slot][idx] = true;
+  }
+  void* args[] = {&p};
+  // every workgroup must be resident at once (waits between problems): one per CU at most
+  DFLASH_HIP_OK(hipLaunchKernel(fn, dim3(cus), dim3(kThreads), args, kLdsBytesChain, stream));
+  return DFLASH_OK;
+}
+
+}  // namespace dflash
+
+extern "C" size_t dflash_qmm_m16_chain_workspace_bytes(const dflash_qmm_problem* problems, int count,
+                                                       int group_size) {
+  return dflash::qmm_chain_workspace_bytes(problems, count, group_size);
+}
+
+extern "C" int dflash_qmm_m16_chain(const dflash_qmm_problem* problems, int count, void* workspace,
+                                    size_t workspace_bytes, int group_size, int act_dtype, int sb_dtype,
+                                    int spin_limit, void* stream) {
+  using namespace dflash;
+  DFLASH_REQUIRE(act_dtype == DFLASH_BF16 || act_dtype == DFLASH_FP16, DFLASH_ERR_ARG,
+                 "dflash_qmm_m16_chain: act_dtype %d is not bf16/fp16", act_dtype);
+  DFLASH_REQUIRE(sb_dtype == DFLASH_BF16 || sb_dtype == DFLASH_FP16, DFLASH_ERR_ARG,
+                 "dflash_qmm_m16_chain: sb_dtype %d is not bf16/fp16", sb_dtype);
+  return qmm_chain_launch(problems, count, workspace, workspace_bytes, group_size, act_dtype, sb_dtype,
+                          spin_limit, (hipStream_t)stream);
+}

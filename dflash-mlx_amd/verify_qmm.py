@@ -21,7 +21,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from typing import Dict, Tuple
+from typing import Dict, Optional, Tuple
 
 import torch
 
@@ -158,6 +158,109 @@ def verify_qmm(x: torch.Tensor, w_packed: torch.Tensor, scales: torch.Tensor, bi
     """The name the hot path is known by: ``verify_matmul`` with ``group_size`` and ``bits``
     accepted positionally as well."""
     return verify_matmul(x, w_packed, scales, biases, transpose=transpose, group_size=group_size, bits=bits)
+
+
+class ChainProblem:
+    """One projection of a ``QmmChain``: ``y = x @ dequant(w, scales, biases).T`` for 16 rows.
+
+    ``x`` is a device tensor of 16 rows of K values, or the ``ChainProblem`` whose output this
+    projection reads (its weights then stream while that output is still being computed).
+    ``epilogue="silu_mul"``: ``w``/``scales``/``biases`` hold the gate rows followed by the up rows
+    of an MLP and the output is ``silu(gate) * up`` of ``[16, N/2]``."""
+
+    def __init__(self, x, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, *,
+                 epilogue: Optional[str] = None, out: Optional[torch.Tensor] = None):
+        if epilogue not in (None, "silu_mul"):
+            raise ValueError(f"unknown epilogue {epilogue!r}")
+        self.x, self.w, self.scales, self.biases = x, w, scales, biases
+        self.epilogue, self.out = epilogue, out
+
+
+class QmmChain:
+    """Several 16-row quantized matmuls in ONE launch (``dflash_qmm_m16_chain``): the projections
+    of a layer handed over as a list and run back to back by one persistent grid.  No counterpart
+    in the reference, which launches its kernel once per projection
+    (``dflash_mlx/verify_linear.py:103-143``); every output is bit for bit what ``verify_matmul``
+    gives for the same operands through the streaming kernel.
+
+    The chain is planned once (argument block, outputs, workspace) and can be launched any number
+    of times: ``chain()`` enqueues the launch on the current stream and returns the outputs, which
+    are the same tensors every time.  Inputs are read from where they were when the chain was
+    built (``x`` tensors are not copied).  Needs 4-bit codes, group 64, K a multiple of 1024,
+    N of 32, bf16/fp16 activations on the GPU; at most 16 projections."""
+
+    def __init__(self, problems, *, group_size: int = 64, bits: int = 4, spin_limit: int = 0):
+        problems = list(problems)
+        if bits != 4 or group_size != 64:
+            raise ValueError("QmmChain: 4-bit codes in groups of 64 only")
+        if not 1 <= len(problems) <= _native.QMM_CHAIN_MAX:
+            raise ValueError(f"QmmChain: 1 to {_native.QMM_CHAIN_MAX} projections, got {len(problems)}")
+        lib = _native.lib()
+        self._keep, self.outputs = [], []
+        self._table = (_native.QmmProblem * len(problems))()
+        index = {}
+        act = sb = device = None
+        for i, pr in enumerate(problems):
+            wait_for = -1
+            if isinstance(pr.x, ChainProblem):
+                if id(pr.x) not in index:
+                    raise ValueError(f"QmmChain: projection {i} reads a projection that does not come before it")
+                wait_for = index[id(pr.x)]
+                x2 = self.outputs[wait_for]
+            else:
+                m = 1
+                for d in pr.x.shape[:-1]:
+                    m *= int(d)
+                if m != 16 or not pr.x.is_cuda or pr.x.dtype not in _DTYPE_CODE:
+                    raise ValueError(f"QmmChain: x of projection {i} must hold 16 rows of bf16/fp16 values on the GPU")
+                x2 = pr.x.reshape(16, pr.x.shape[-1])
+                if not x2.is_contiguous():
+                    raise ValueError(f"QmmChain: x of projection {i} must be contiguous (it is read in place)")
+            w, s, b = pr.w.contiguous(), pr.scales.contiguous(), pr.biases.contiguous()
+            K, N = int(w.shape[1]) * 8, int(w.shape[0])
+            if int(x2.shape[1]) != K or s.dtype not in _DTYPE_CODE or b.dtype != s.dtype or N % 32 != 0:
+                raise ValueError(f"QmmChain: operands of projection {i} do not fit together (K={K}, N={N})")
+            act = x2.dtype if act is None else act
+            sb = s.dtype if sb is None else sb
+            device = x2.device if device is None else device
+            if x2.dtype != act or s.dtype != sb or x2.device != device or w.device != device:
+                raise ValueError("QmmChain: all projections share one activation dtype, one scale dtype and one device")
+            cols = N // 2 if pr.epilogue == "silu_mul" else N
+            y = pr.out if pr.out is not None else torch.empty((16, cols), dtype=act, device=device)
+            if tuple(y.shape) != (16, cols) or y.dtype != act or not y.is_contiguous() or y.device != device:
+                raise ValueError(f"QmmChain: out of projection {i} must be a contiguous [16, {cols}] tensor of {act}")
+            t = self._table[i]
+            t.x, t.w_q, t.scales, t.biases, t.y = x2.data_ptr(), w.data_ptr(), s.data_ptr(), b.data_ptr(), y.data_ptr()
+            t.K, t.N, t.wait_for = K, N, wait_for
+            t.epilogue = _native.QMM_EPILOGUE_SILU_MUL if pr.epilogue == "silu_mul" else _native.QMM_EPILOGUE_NONE
+            self._keep.append((x2, w, s, b))
+            self.outputs.append(y)
+            index[id(pr)] = i
+        self._count, self._group = len(problems), group_size
+        self._act, self._sb, self._device = _DTYPE_CODE[act], _DTYPE_CODE[sb], device
+        self._spin = int(spin_limit)
+        self._need = int(lib.dflash_qmm_m16_chain_workspace_bytes(self._table, self._count, group_size))
+        if self._need == 0:
+            raise ValueError("QmmChain: a projection has a shape the chained kernel does not cover "
+                             "(group 64, K % 1024 == 0, N % 32 == 0; N % 128 == 0 with an epilogue)")
+
+    def __call__(self):
+        stream = _native.raw_stream(self._device)
+        ws = _workspace(self._device, stream, self._need)
+        self._ws = ws
+        rc = _native.lib().dflash_qmm_m16_chain(self._table, self._count, ws.data_ptr(), ws.numel(), self._group,
+                                                self._act, self._sb, self._spin, stream)
+        _native.check(rc, "dflash_qmm_m16_chain")
+        return self.outputs
+
+    def error_word(self) -> int:
+        """0, or 1 + the index of a projection whose wait for its input was given up (read back
+        from the workspace of the last launch; synchronises with the device)."""
+        word = self._ws[_native.QMM_CHAIN_ERROR_OFFSET:_native.QMM_CHAIN_ERROR_OFFSET + 4]
+        return int(word.view(torch.int32).item())
+
+    def clear_error(self) -> None:
+        self._ws[_native.QMM_CHAIN_ERROR_OFFSET:_native.QMM_CHAIN_ERROR_OFFSET + 4].zero_()
 
 
 class PackedWeights:

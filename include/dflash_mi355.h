@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 9
+#define DFLASH_ABI_VERSION 10
 
 enum {
   DFLASH_OK = 0,
@@ -101,6 +101,55 @@ int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* scales, const
 int dflash_qmm_m16_static(const void* x, const uint32_t* w_q, const void* scales, const void* biases,
                           void* y, int K, int N, int group_size, int act_dtype, int sb_dtype,
                           int variant, int k_parts, int kernel, void* stream);
+
+/*
+ * Several qmm problems in one launch.  No counterpart in the reference, whose verify step
+ * calls the kernel once per projection (dflash_mlx/verify_linear.py:103-143): a launch costs
+ * more around its weight stream than inside it, so the projections of a layer are handed over
+ * as one list and run back to back by one persistent grid - each divided among the workgroups
+ * exactly as a dflash_qmm_m16 call of its own would be (streaming kernel), with results bit
+ * for bit the same, the weights of the next problem already streaming while the current one
+ * ends.
+ *
+ *   problems[i]: x [16, K], w_q [N, K/8], scales/biases [N, K/64], y [16, N] as for dflash_qmm_m16.
+ *   wait_for    -1, or the index j < i of the problem whose y is this problem's x (x == problems[j].y,
+ *               K == its number of output columns): the x loads of problem i are held back until
+ *               problem j's output has been stored; its weights stream regardless.
+ *   epilogue    DFLASH_QMM_EPILOGUE_NONE, or DFLASH_QMM_EPILOGUE_SILU_MUL: w_q, scales, biases hold
+ *               N/2 gate rows followed by N/2 up rows and y is [16, N/2],
+ *                   y = round(round(silu(round(gate))) * round(up))     (round: to act_dtype),
+ *               what `silu(gate_proj(x)) * up_proj(x)` of an MLP gives operator by operator.
+ * Requirements: 1 <= count <= DFLASH_QMM_CHAIN_MAX; group_size 64; K % 1024 == 0; N % 16 == 0
+ * (N % 128 == 0 with an epilogue); pointers 16-byte aligned; workspace of
+ * dflash_qmm_m16_chain_workspace_bytes(...) bytes under the rules of dflash_qmm_m16 (zero-filled
+ * once, reusable, shareable with the other qmm entry points on the same stream).
+ * spin_limit bounds the wait for an earlier problem (polls of its counter; <= 0: a default of
+ * several seconds).  A workgroup that gives up writes i + 1 into the 32-bit word at byte offset
+ * DFLASH_QMM_CHAIN_ERROR_OFFSET of the workspace (it stays there until the caller clears it),
+ * goes on with whatever x holds, and the launch ends normally: the outputs of problem i and of
+ * what depends on it are then undefined.  The grid is one workgroup per compute unit, all of
+ * which must be resident at once: the device must not be shared with other long-running kernels.
+ */
+#define DFLASH_QMM_CHAIN_MAX 16
+#define DFLASH_QMM_CHAIN_ERROR_OFFSET ((16384 - 64 + 1) * 4)
+enum { DFLASH_QMM_EPILOGUE_NONE = 0, DFLASH_QMM_EPILOGUE_SILU_MUL = 1 };
+
+typedef struct dflash_qmm_problem {
+  const void* x;
+  const uint32_t* w_q;
+  const void* scales;
+  const void* biases;
+  void* y;
+  int K, N;
+  int wait_for;
+  int epilogue;
+} dflash_qmm_problem;
+
+size_t dflash_qmm_m16_chain_workspace_bytes(const dflash_qmm_problem* problems, int count, int group_size);
+
+int dflash_qmm_m16_chain(const dflash_qmm_problem* problems, int count, void* workspace,
+                         size_t workspace_bytes, int group_size, int act_dtype, int sb_dtype,
+                         int spin_limit, void* stream);
 
 /*
  * The same product on weights stored in the order the streaming kernel consumes them.  No

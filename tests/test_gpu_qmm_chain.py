@@ -1,0 +1,209 @@
+"""dflash_qmm_m16_chain: several 16-row quantized matmuls in one launch.
+
+Bars: every projection's output equals, bit for bit, what a launch of its own gives for the same
+operands (streaming kernel: same unit ranges, same order of partial sums) - hence the oracle
+parity of tests/test_gpu_qmm.py carries over, and is checked directly on one chain as well.  The
+silu-mul epilogue equals silu(gate) * up computed operator by operator on separate launches'
+outputs on at least 99.8 % of the elements (a launch of its own splits K elsewhere, which can
+move the last bit of a factor), and meets the qmm bar (max-abs <= 2e-2 * row-inf, rel-L2 <= 5e-3)
+against silu(g) * u of the exact fp64 products.  A projection that reads another's output gives what a separate launch gives on
+that output, bit for bit.  The bounded wait is made to give up from the host: the launch still
+ends and says which projection gave up."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import dflash_mlx_amd._native as nat
+from dflash_mlx_amd import verify_qmm as VQ
+from dflash_mlx_amd.workloads import make_qmm_case
+from oracle import dflash_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(autouse=True)
+def _env(verify_env):
+    verify_env.setenv("DFLASH_QMM_KERNEL", "stream")
+
+
+def _separate(x, c):
+    return VQ.verify_matmul(x, c.w, c.scales, c.biases, group_size=64, bits=4)
+
+
+def _bits(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _exact(c_oracle, c, x=None):
+    y32, _ = c_oracle.qmm_m16(_bits(c.x if x is None else x), c.w.cpu().numpy().view(np.uint32), _bits(c.scales), _bits(c.biases),
+                              c.group_size, flavour=0)
+    return y32
+
+
+def _cases(shapes, seed, dtype=torch.bfloat16):
+    return [make_qmm_case(K, N, seed + i, dtype=dtype).to(DEV) for i, (K, N) in enumerate(shapes)]
+
+
+LAYER_27B = [(5120, 7168), (5120, 5120), (5120, 17408), (5120, 17408), (17408, 5120)]
+LAYER_9B = [(4096, 6144), (4096, 4096), (4096, 12288), (4096, 12288), (12288, 4096)]
+
+
+@pytest.mark.parametrize("shapes", [LAYER_27B, LAYER_9B, [(1024, 64), (2048, 32), (1024, 4096), (3072, 96)],
+                                    [(5120, 5120)], [(1024, 32)] * 16],
+                         ids=["27b-layer", "9b-layer", "small-and-ragged", "single", "sixteen-tiny"])
+def test_independent_projections_equal_separate_launches(native_lib, shapes):
+    cases = _cases(shapes, 700)
+    print(f"chain of {len(shapes)}: {shapes[:5]}", flush=True)
+    chain = VQ.QmmChain([VQ.ChainProblem(c.x, c.w, c.scales, c.biases) for c in cases])
+    for rep in range(3):                      # the workspace is left ready for the next launch
+        for y in chain.outputs:
+            y.fill_(float("nan"))
+        ys = chain()
+        torch.cuda.synchronize()
+        for i, (c, y) in enumerate(zip(cases, ys)):
+            want = _separate(c.x, c)
+            assert torch.equal(y.view(torch.int16), want.view(torch.int16)), (rep, i, shapes[i])
+    assert chain.error_word() == 0
+
+
+def test_chain_against_the_oracle(native_lib, c_oracle):
+    cases = _cases([(1024, 512), (2048, 256), (1024, 1024)], 720)
+    ys = VQ.QmmChain([VQ.ChainProblem(c.x, c.w, c.scales, c.biases) for c in cases])()
+    torch.cuda.synchronize()
+    for c, y in zip(cases, ys):
+        exact = O.qmm_exact(c.x.float().cpu().numpy(), c.w.cpu().numpy().view(np.uint32),
+                            c.scales.float().cpu().numpy(), c.biases.float().cpu().numpy(), 64)
+        got = y.float().cpu().numpy()
+        assert np.all(np.abs(got - exact) <= 2e-2 * np.abs(exact).max(axis=1, keepdims=True))
+        assert np.linalg.norm(got - exact) / np.linalg.norm(exact) <= 5e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fp16_and_bf16_activations(native_lib, dtype):
+    cases = _cases([(1024, 256), (2048, 2048)], 730, dtype)
+    ys = VQ.QmmChain([VQ.ChainProblem(c.x, c.w, c.scales, c.biases) for c in cases])()
+    torch.cuda.synchronize()
+    for c, y in zip(cases, ys):
+        assert torch.equal(y.view(torch.int16), _separate(c.x, c).view(torch.int16))
+
+
+@pytest.mark.parametrize("shapes", [[(1024, 1024), (1024, 2048), (2048, 1024)],
+                                    [(5120, 5120), (5120, 17408), (17408, 5120)],
+                                    [(1024, 1024)] * 6],
+                         ids=["small", "27b-sized", "six-in-a-row"])
+def test_projection_reading_an_earlier_output(native_lib, shapes):
+    """y0 = A x, y1 = B y0, y2 = C y1: every link waits for the one before it."""
+    cases = _cases(shapes, 740)
+    print(f"dependent chain {shapes}", flush=True)
+    # keep the activations in range: outputs of one matmul feed the next
+    for c in cases:
+        c.scales.mul_(0.05); c.biases.mul_(0.05)
+    problems, prev = [], cases[0].x
+    for c in cases:
+        pr = VQ.ChainProblem(prev, c.w, c.scales, c.biases)
+        problems.append(pr)
+        prev = pr
+    chain = VQ.QmmChain(problems)
+    for rep in range(3):
+        for y in chain.outputs:
+            y.fill_(float("nan"))
+        ys = chain()
+        torch.cuda.synchronize()
+        assert chain.error_word() == 0
+        x = cases[0].x
+        for i, (c, y) in enumerate(zip(cases, ys)):
+            want = _separate(x, c)
+            assert torch.isfinite(want.float()).all()
+            assert torch.equal(y.view(torch.int16), want.view(torch.int16)), (rep, i)
+            x = y
+
+
+@pytest.mark.parametrize("K,I", [(1024, 1024), (5120, 17408), (2048, 3072)])
+def test_mlp_in_one_launch(native_lib, c_oracle, K, I):
+    """gate/up with the silu-mul epilogue, then the down projection waiting for it."""
+    gate, up = make_qmm_case(K, I, 750).to(DEV), make_qmm_case(K, I, 751).to(DEV)
+    down = make_qmm_case(I, K, 752).to(DEV)
+    for c in (gate, up, down):
+        c.scales.mul_(0.1); c.biases.mul_(0.1)
+    joint = [torch.cat([a, b], dim=0).contiguous() for a, b in
+             ((gate.w, up.w), (gate.scales, up.scales), (gate.biases, up.biases))]
+    x = gate.x
+    print(f"mlp chain K={K} I={I}", flush=True)
+    p0 = VQ.ChainProblem(x, *joint, epilogue="silu_mul")
+    p1 = VQ.ChainProblem(p0, down.w, down.scales, down.biases)
+    chain = VQ.QmmChain([p0, p1])
+    for rep in range(2):
+        for y in chain.outputs:
+            y.fill_(float("nan"))
+        h, y = chain()
+        torch.cuda.synchronize()
+        assert chain.error_word() == 0
+        # operator by operator on separate launches: a launch of its own splits K elsewhere than
+        # the gate/up pair does, so g and u may differ in their last bit where sums cancel - equal
+        # on nearly all elements, and everywhere within the bar on the exact product below
+        g, u = _separate(x, gate), _separate(x, up)
+        want_h = torch.nn.functional.silu(g) * u
+        assert float((h != want_h).float().mean()) <= 2e-3
+        ge, ue = (_exact(c_oracle, c, x).astype(np.float64) for c in (gate, up))
+        exact = ge / (1.0 + np.exp(-ge)) * ue
+        got = h.float().cpu().numpy().astype(np.float64)
+        assert np.all(np.abs(got - exact) <= 2e-2 * np.abs(exact).max(axis=1, keepdims=True))
+        assert np.linalg.norm(got - exact) / np.linalg.norm(exact) <= 5e-3
+        # the down projection read exactly the h the launch stored
+        want_y = _separate(h, down)
+        assert torch.equal(y.view(torch.int16), want_y.view(torch.int16))
+
+
+def test_bounded_wait_gives_up_and_the_launch_still_ends(native_lib):
+    """spin_limit = 1: a projection that waits polls twice at most.  Whether its input was ready
+    by then is a matter of timing; either way every workgroup leaves, the launch ends, the error
+    word names the projection when a wait was given up, and the next launch (default limit) is
+    right again."""
+    cases = _cases([(5120, 17408), (17408, 5120)], 760)
+    for c in cases:
+        c.scales.mul_(0.05); c.biases.mul_(0.05)
+    p0 = VQ.ChainProblem(cases[0].x, cases[0].w, cases[0].scales, cases[0].biases)
+    p1 = VQ.ChainProblem(p0, cases[1].w, cases[1].scales, cases[1].biases)
+    hasty = VQ.QmmChain([p0, p1], spin_limit=1)
+    hasty()
+    torch.cuda.synchronize()                       # returns: nothing hangs
+    word = hasty.error_word()
+    assert word in (0, 2)
+    y0 = _separate(cases[0].x, cases[0])
+    assert torch.equal(hasty.outputs[0].view(torch.int16), y0.view(torch.int16))   # nothing waits for x0
+    hasty.clear_error()
+    patient = VQ.QmmChain([p0, p1])
+    ys = patient()
+    torch.cuda.synchronize()
+    assert patient.error_word() == 0
+    assert torch.equal(ys[1].view(torch.int16), _separate(ys[0], cases[1]).view(torch.int16))
+
+
+def test_argument_errors(native_lib):
+    L = native_lib
+    tab = (nat.QmmProblem * 2)()
+    one = 256
+    for t in tab:
+        t.x = t.w_q = t.scales = t.biases = t.y = one
+        t.K, t.N, t.wait_for, t.epilogue = 1024, 64, -1, 0
+    ws = ctypes.c_void_p(one)
+    assert L.dflash_qmm_m16_chain(tab, 0, ws, 1 << 30, 64, 0, 0, 0, None) == -1
+    assert L.dflash_qmm_m16_chain(tab, 17, ws, 1 << 30, 64, 0, 0, 0, None) == -2
+    tab[1].K = 512
+    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, None) == -2      # K % 1024
+    tab[1].K = 1024
+    tab[1].wait_for = 1
+    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, None) == -1      # waits for itself
+    tab[1].wait_for = 0
+    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, None) == -1      # x is not problem 0's y / K != N0
+    assert b"waits for" in L.dflash_last_error()
+    tab[1].wait_for = -1
+    tab[0].epilogue = 1
+    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, None) == -2      # N % 128 with an epilogue
+    tab[0].epilogue = 0
+    assert L.dflash_qmm_m16_chain(tab, 2, None, 0, 64, 0, 0, 0, None) == -3
+    assert L.dflash_qmm_m16_chain_workspace_bytes(tab, 2, 64) >= 64 * 1024 + 2 * 2 * 8192
+    assert L.dflash_qmm_m16_chain_workspace_bytes(tab, 2, 32) == 0
