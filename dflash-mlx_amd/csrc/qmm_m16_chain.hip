@@ -34,12 +34,16 @@ namespace dflash {
 namespace stream {
 
 constexpr int kMaxChain = DFLASH_QMM_CHAIN_MAX;
-constexpr int kChainAhead = 3;  // units issued beyond the one being consumed
-// LDS behind the two rings: last-arriver flags, then the up half of an epilogue row block
-// (4 tiles of 1 KiB) for each of the two row blocks a workgroup can be last at.
+#ifndef DFLASH_CHAIN_AHEAD
+#define DFLASH_CHAIN_AHEAD 3
+#endif
+constexpr int kChainAhead = DFLASH_CHAIN_AHEAD;  // units issued beyond the one being consumed
+// LDS behind the two rings: last-arriver flags, the up half of an epilogue row block (4 tiles of
+// 1 KiB) for each of the two row blocks a workgroup can be last at, the table of ranges.
 constexpr int kChainFlags = kLdsBytes;
 constexpr int kChainExchange = kChainFlags + 64;
-constexpr int kLdsBytesChain = kChainExchange + 2 * 4096;  // 152.1 KiB
+constexpr int kChainTable = kChainExchange + 2 * 4096;  // 32 bytes per problem: its Range
+constexpr int kLdsBytesChain = kChainTable + 32 * kMaxChain;  // 152.6 KiB
 // The last words of the 64 KiB counter block: launch bookkeeping of chains.
 constexpr int kChainStatusWord = 16384 - 64;  // [0] exit counter, [1] error word
 constexpr int kChainDoneWord = kChainStatusWord + 8;  // [kMaxChain] row blocks stored, per problem
@@ -104,6 +108,63 @@ __device__ __forceinline__ Range problem_range(CProblem& q, int block, int nbloc
   return r;
 }
 
+// The Range of problem i from the table in LDS (hand-written reads: see the file header of
+// qmm_m16_stream.hip).  All values are the same in every lane.
+__device__ __forceinline__ Range read_range(uint32_t lds0, int i) {
+  u32x4_t a, b;
+  const uint32_t addr = lds0 + kChainTable + i * 32;
+  asm volatile("ds_read_b128 %0, %2\n ds_read_b128 %1, %2 offset:16\n s_waitcnt lgkmcnt(0)"
+               : "=&v"(a), "=&v"(b)
+               : "v"(addr)
+               : "memory");
+  Range r;
+  r.wg = __builtin_amdgcn_readfirstlane((int)a.x);
+  r.u0 = __builtin_amdgcn_readfirstlane((int)a.y);
+  r.u1 = __builtin_amdgcn_readfirstlane((int)a.z);
+  r.rb0 = __builtin_amdgcn_readfirstlane((int)a.w);
+  r.st0 = __builtin_amdgcn_readfirstlane((int)b.x);
+  r.stages = __builtin_amdgcn_readfirstlane((int)b.y);
+  r.units = __builtin_amdgcn_readfirstlane((int)b.z);
+  r.grid = __builtin_amdgcn_readfirstlane((int)b.w);
+  r.RB = r.units / r.stages;
+  return r;
+}
+
+// wait_loads() rounded down to the thresholds that occur in steady state (one or two units
+// issued behind the one waited for, each 6 loads, 8 with its scales and biases): waiting for
+// fewer outstanding loads than allowed is always safe, and the full switch costs the wave tens
+// of instructions per unit.
+__device__ __forceinline__ void wait_loads_coarse(int n) {
+  if (n >= 12) {
+    if (n >= 20) __builtin_amdgcn_s_waitcnt(0x0F70 | (20 & 15) | ((20 >> 4) << 14));
+    else if (n >= 18) __builtin_amdgcn_s_waitcnt(0x0F70 | (18 & 15) | ((18 >> 4) << 14));
+    else if (n >= 14) __builtin_amdgcn_s_waitcnt(0x0F70 | 14);
+    else __builtin_amdgcn_s_waitcnt(0x0F70 | 12);
+  } else {
+    if (n >= 8) __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
+    else if (n >= 6) __builtin_amdgcn_s_waitcnt(0x0F70 | 6);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+  }
+}
+
+// The hand-over of a problem's shared row blocks needs three memory round trips.  Where nothing
+// waits for the result they are spread over the first units of the workgroup's next problem
+// instead of being sat out: not for a problem that another one waits for or that has an
+// epilogue (their outputs are needed at once / take one more barrier), and only if the next
+// problem this workgroup takes part in has its x at hand and at least kHandoverSumUnit + 1 units
+// here.  Loaders and workers decide alike: the rule fixes the barriers of the hand-over.
+constexpr int kHandoverArriveUnit = 1;  // unit of the next problem at whose barrier the arrival counters are bumped
+constexpr int kHandoverSumUnit = 3;     // ... and at whose barrier the last to arrive adds the partial tiles
+__device__ __forceinline__ bool handover_deferred(CParams& p, uint32_t lds0, int cp) {
+  if (p.prob[cp].signal || p.prob[cp].epilogue != DFLASH_QMM_EPILOGUE_NONE) return false;
+  for (int nx = cp + 1; nx < p.count; ++nx) {
+    const Range r = read_range(lds0, nx);
+    if (r.wg < 0) continue;
+    return p.prob[nx].wait_for < 0 && r.u1 - r.u0 > kHandoverSumUnit;
+  }
+  return false;
+}
+
 // Row of w behind row v (0..127) of row block rb.  Plain: 128 rb + v.  Epilogue: the first 64
 // rows are gate rows 64 rb .., the other 64 the up rows of the same output columns.
 __device__ __forceinline__ int weight_row(CProblem& q, int rb, int v) {
@@ -120,6 +181,20 @@ __device__ __forceinline__ int weight_row(CProblem& q, int rb, int v) {
 __device__ __forceinline__ void load16_to_lds_coherent(const void* gptr, char* lds_base) {
   __builtin_amdgcn_global_load_lds((global_cvoid_t*)gptr, (lds_void_t*)lds_base, 16, 0, 16);  // sc1
 }
+
+#ifdef DFLASH_CHAIN_STAMPS
+// Experiment builds only: per workgroup, wave 0 (a worker) and wave 8 (a loader) record the
+// constant-rate wall clock at every unit.  [block][role][slot]
+constexpr int kStampSlots = 512;
+__device__ unsigned long long g_stamps[64][13][kStampSlots];
+#define DFLASH_STAMP(role, idx)                                                          \
+  do {                                                                                   \
+    if (lane == 0 && (idx) < kStampSlots && blockIdx.x < 64)                             \
+      g_stamps[blockIdx.x][role][idx] = wall_clock64();                                  \
+  } while (0)
+#else
+#define DFLASH_STAMP(role, idx) do {} while (0)
+#endif
 
 template <bool FP16>
 __device__ __forceinline__ float silu_mul(float g, float u) {
@@ -148,6 +223,15 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
   uint32_t* const status = p.counters + kChainStatusWord;
   uint32_t* const done = p.counters + kChainDoneWord;
 
+  // How every problem is divided (this workgroup's range): computed once, lane i of wave 0 for
+  // problem i, and kept in LDS; the waves look a problem up when they reach it.
+  if (wave == 0 && lane < p.count) {
+    const Range r = problem_range(p.prob[lane], block, nblocks);
+    int* t = reinterpret_cast<int*>(lds + kChainTable + lane * 32);
+    t[0] = r.wg, t[1] = r.u0, t[2] = r.u1, t[3] = r.rb0, t[4] = r.st0, t[5] = r.stages, t[6] = r.units, t[7] = r.grid;
+  }
+  __syncthreads();
+
   // Both kinds of wave walk the same problems and units and pass the same barriers.  Per
   // problem this workgroup takes part in:
   //   one at its start (its first unit has landed),
@@ -161,9 +245,11 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
 
   if (wave >= kWaves) {
     // ================================ loader waves ====================================
-    // See qmm_m16_stream.hip for which loader issues which 16-byte pieces of a unit.  The loop
-    // below is flat on purpose: one place that issues units, one that waits, one that opens a
-    // problem.  (A loader may not spill: spill traffic would count as loads of its own.)
+    // See qmm_m16_stream.hip for which loader issues which 16-byte pieces of a unit.  The
+    // workers wait for this wave at every unit, so its path from one barrier to the next is
+    // kept short: 32-bit offsets from base pointers held in scalar registers, unit ranges read
+    // from the table in LDS, waits rounded to a few thresholds.  (A loader may not spill: spill
+    // traffic would count as loads of its own.)
     const int ld = wave - kWaves;
     const int w_r = lane >> 3;
     const int w_c = (lane & 7) ^ (((w_r >> 1) & 3) << 1);
@@ -172,100 +258,86 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
     enum { NEED_OPEN, OPEN, PARKED, EXHAUSTED };
     int i_state = NEED_OPEN;
     int ip = -1;  // problem being issued
-    Range ir{};
-    int iu = 0, irb = 0, ist = 0;   // next unit to issue: index, row block, stage
-    bool i_first = false;           // it is the first unit of this workgroup's range
-    bool i_coherent = false;        // x of problem ip is written by this launch
-    bool i_ready = true;            // ... and is known to be complete
+    int iu = 0, iu1 = 0, irb = 0, ist = 0, istages = 1;  // next unit to issue: index, end of range, row block, stage
+    bool i_first = false;     // it is the first unit of this workgroup's range
+    bool i_coherent = false;  // x of problem ip is written by this launch
+    bool i_ready = true;      // ... and is known to be complete
+    const char* bx = nullptr;  // arrays of problem ip
+    const char* bw = nullptr;
+    const char* bs = nullptr;
+    const char* bb = nullptr;
     // byte offsets of this lane's pieces from the problem's x, w and scales (= biases) arrays
-    uint32_t xo[2] = {0u, 0u}, wo[4] = {0u, 0u, 0u, 0u}, so = 0u;
+    // (named one by one: an array indexed inside these loops would be placed in memory)
+    uint32_t xo0 = 0u, xo1 = 0u, wo0 = 0u, wo1 = 0u, wo2 = 0u, wo3 = 0u, so = 0u;
     int slot_i = 0, sb_slot_i = 0;
-    int n_issued = 0, n_cons = 0;   // units issued / units whose barrier has passed
-    int tot = 0;                    // loads this wave has issued
-    int mark0 = 0, mark1 = 0, mark2 = 0, mark3 = 0, fifo_n = 0;  // `tot` after each unit not yet waited for
+    int n_issued = 0, n_cons = 0;  // units issued / units whose barrier has passed
+    int tot = 0;                   // loads this wave has issued
+    int mark0 = 0, mark1 = 0, mark2 = 0, mark3 = 0, fifo_n = 0;  // `tot` after each of the last units issued, newest first; how many are not yet waited for
     int def_n = 0, def_slot = 0, def_st = 0;  // units of problem ip issued without their x
 
     auto set_row_block = [&](int rb) __attribute__((always_inline)) {
       CProblem& q = p.prob[ip];
       const uint32_t row_bytes = (uint32_t)q.K >> 1;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        wo[i] = (uint32_t)weight_row(q, rb, 8 * (ld + 4 * i) + w_r) * row_bytes + w_c * 16;
+      wo0 = (uint32_t)weight_row(q, rb, 8 * (ld + 0) + w_r) * row_bytes + w_c * 16;
+      wo1 = (uint32_t)weight_row(q, rb, 8 * (ld + 4) + w_r) * row_bytes + w_c * 16;
+      wo2 = (uint32_t)weight_row(q, rb, 8 * (ld + 8) + w_r) * row_bytes + w_c * 16;
+      wo3 = (uint32_t)weight_row(q, rb, 8 * (ld + 12) + w_r) * row_bytes + w_c * 16;
       so = (uint32_t)weight_row(q, rb, 32 * ld + (lane >> 1)) * (uint32_t)(q.K / kGS * 2) + (lane & 1) * 16;
     };
     auto issue_x = [&](int st, int slot) __attribute__((always_inline)) {
-      CProblem& q = p.prob[ip];
-      char* dst = lds + slot * kSlotBytes + kXOffset;
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const char* src = (const char*)q.x + (xo[i] + (uint32_t)st * (kUnitK * 2));
-        if (i_coherent)
-          load16_to_lds_coherent(src, dst + (ld + 4 * i) * 1024);
-        else
-          load16_to_lds(src, dst + (ld + 4 * i) * 1024);
+#ifdef DFLASH_CHAIN_NOX  // (timing experiments: the stream without the x loads; results are wrong)
+      (void)st, (void)slot;
+      return;
+#endif
+      char* dst = lds + slot * kSlotBytes + kXOffset + ld * 1024;
+      const uint32_t step = (uint32_t)st * (kUnitK * 2);
+      if (i_coherent) {
+        load16_to_lds_coherent(bx + (xo0 + step), dst);
+        load16_to_lds_coherent(bx + (xo1 + step), dst + 4096);
+      } else {
+        load16_to_lds(bx + (xo0 + step), dst);
+        load16_to_lds(bx + (xo1 + step), dst + 4096);
       }
       tot += 2;
     };
-
-    // ---- consume cursor: mirrors the workers' barriers ---------------------------------
-    enum { START, UNIT, END, FINISHED };
-    int phase = FINISHED;
-    int cp = -1;
-    Range cr{};
-    int u = 0, rb_left = 0, in_rb = 0;
-    bool any_shared = false;
-    auto next_problem = [&]() __attribute__((always_inline)) {
-      phase = FINISHED;
-      while (++cp < p.count) {
-        cr = problem_range(p.prob[cp], block, nblocks);
-        if (cr.wg >= 0) {
-          phase = START;
-          break;
-        }
-      }
-    };
-    next_problem();
-
-#pragma unroll 1
-    while (phase != FINISHED) {
-      // ---- keep kChainAhead units issued beyond the one being consumed ------------------
+    // Keeps kChainAhead units issued beyond the one being consumed.
+    auto top_up = [&]() __attribute__((always_inline)) {
 #pragma unroll 1
       while (n_issued - n_cons < kChainAhead) {
         if (i_state == NEED_OPEN) {
           i_state = EXHAUSTED;
           while (++ip < p.count) {
-            ir = problem_range(p.prob[ip], block, nblocks);
-            if (ir.wg >= 0) {
+            const Range r = read_range(lds0, ip);
+            if (r.wg >= 0) {
+              iu = r.u0, iu1 = r.u1, irb = r.rb0, ist = r.st0, istages = r.stages;
               i_state = OPEN;
               break;
             }
           }
           if (i_state == OPEN) {
             CProblem& q = p.prob[ip];
-            iu = ir.u0, irb = ir.rb0, ist = ir.st0;
+            bx = (const char*)q.x, bw = (const char*)q.w, bs = (const char*)q.scales, bb = (const char*)q.biases;
             i_first = true;
             i_coherent = q.wait_for >= 0;
             i_ready = !i_coherent;
+            // x: instruction i of 8 moves group i >> 1, k-blocks 2 (i & 1) and 2 (i & 1) + 1; this
+            // loader issues i = ld and ld + 4
             const int xrow = lane & 15;
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-              const int xi = ld + 4 * i;
-              xo[i] = (uint32_t)(xrow * q.K + (xi >> 1) * kGS + (2 * (xi & 1) + (lane >> 5)) * 16 +
-                                 ((lane >> 4) & 1) * 8) * 2u;
-            }
+            const uint32_t xbase = (uint32_t)(xrow * q.K + (2 * (ld & 1) + (lane >> 5)) * 16 + ((lane >> 4) & 1) * 8);
+            xo0 = (xbase + (uint32_t)((ld >> 1) * kGS)) * 2u;
+            xo1 = (xbase + (uint32_t)(((ld + 4) >> 1) * kGS)) * 2u;
             set_row_block(irb);
           }
         }
         if (i_state != OPEN) break;
         // ---- one unit: scales/biases with the first unit of a chunk or of the range, x unless
         // it is still being computed, codes
-        CProblem& q = p.prob[ip];
         char* slot = lds + slot_i * kSlotBytes;
-        if ((ist % CHUNK) == 0 || i_first) {
+        if ((ist & (CHUNK - 1)) == 0 || i_first) {
           char* sb = lds + kSbOffset + sb_slot_i * kSbSlotBytes;
           const uint32_t off = so + (uint32_t)(ist / CHUNK) * (CHUNK * kGroups * 2);
-          load16_to_lds((const char*)q.scales + off, sb + ld * 1024);
-          load16_to_lds((const char*)q.biases + off, sb + kSbArrayBytes + ld * 1024);
+          load16_to_lds(bs + off, sb + ld * 1024);
+          load16_to_lds(bb + off, sb + kSbArrayBytes + ld * 1024);
           tot += 2;
           if (++sb_slot_i == kSbDepth) sb_slot_i = 0;
         }
@@ -276,41 +348,47 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
           if (def_n == 0) def_slot = slot_i, def_st = ist;
           ++def_n;
         }
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          load16_to_lds_stream((const char*)q.w + (wo[i] + (uint32_t)ist * (kUnitK / 2)), slot + (ld + 4 * i) * 1024);
+        {
+          const uint32_t step = (uint32_t)ist * (kUnitK / 2);
+          char* dst = slot + ld * 1024;
+          load16_to_lds_stream(bw + (wo0 + step), dst);
+          load16_to_lds_stream(bw + (wo1 + step), dst + 4096);
+          load16_to_lds_stream(bw + (wo2 + step), dst + 8192);
+          load16_to_lds_stream(bw + (wo3 + step), dst + 12288);
+        }
         tot += 4;
-        // remember where this unit's loads end
-        if (fifo_n == 0) mark0 = tot;
-        else if (fifo_n == 1) mark1 = tot;
-        else if (fifo_n == 2) mark2 = tot;
-        else mark3 = tot;
+        // remember where this unit's loads end: newest first
+        mark3 = mark2, mark2 = mark1, mark1 = mark0, mark0 = tot;
         ++fifo_n;
         ++n_issued;
         if (++slot_i == kDepth) slot_i = 0;
-        if (++iu == ir.u1) {
+        if (++iu == iu1) {
           // A problem with held-back x loads keeps the cursor until they have been issued: the
           // cursor never enters a second problem whose x is still being computed.
           i_state = def_n == 0 ? NEED_OPEN : PARKED;
-        } else if (++ist == ir.stages) {
+        } else if (++ist == istages) {
           ist = 0;
           ++irb;
           set_row_block(irb);
         }
       }
+    };
+    // Waits until this loader's part of the oldest unit not yet waited for has landed.
+    auto wait_oldest = [&]() __attribute__((always_inline)) {
+      const int oldest = fifo_n == 1 ? mark0 : fifo_n == 2 ? mark1 : fifo_n == 3 ? mark2 : mark3;
+      wait_loads_coarse(tot - oldest);
+      --fifo_n;
+    };
 
-      if (phase == END) {
-        if (any_shared) {
-          asm volatile("s_barrier" ::: "memory");
-          asm volatile("s_barrier" ::: "memory");
-          if (p.prob[cp].epilogue == DFLASH_QMM_EPILOGUE_SILU_MUL) asm volatile("s_barrier" ::: "memory");
-        }
-        if (p.prob[cp].signal) asm volatile("s_barrier" ::: "memory");
-        next_problem();
-        continue;
-      }
-
-      if (phase == START && p.prob[cp].wait_for >= 0) {
+#ifdef DFLASH_CHAIN_STAMPS
+    int st_idx = 0;
+#endif
+#pragma unroll 1
+    for (int cp = 0; cp < p.count; ++cp) {
+      const Range cr = read_range(lds0, cp);
+      if (cr.wg < 0) continue;
+      top_up();
+      if (p.prob[cp].wait_for >= 0) {
         // The x of problem cp is the y of an earlier problem: wait (bounded) until all its row
         // blocks have been stored, then issue the x loads that were held back.  The issue
         // cursor is on problem cp (inside it, or parked at its end).
@@ -330,49 +408,131 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
 #pragma unroll 1
           for (int j = 0; j < def_n; ++j) {
             issue_x(st, slot);
-            // a held-back unit ends with its x loads (nothing else is waiting to be waited for:
-            // every unit of the problems before cp has been consumed)
-            if (j == 0) mark0 = tot;
-            else if (j == 1) mark1 = tot;
-            else if (j == 2) mark2 = tot;
-            else mark3 = tot;
-            if (++st == ir.stages) st = 0;
+            if (++st == istages) st = 0;
             if (++slot == kDepth) slot = 0;
           }
+          // Nothing but held-back units is waiting to be waited for (every unit of the problems
+          // before cp has been consumed), and they end with the x loads just issued.
+          mark0 = mark1 = mark2 = mark3 = tot;
           def_n = 0;
           i_ready = true;
           if (i_state == PARKED) i_state = NEED_OPEN;
         }
       }
-      // START: the first unit of problem cp has landed.  UNIT: unit u + 1 has landed, and every
-      // worker holds unit u in registers, so its slot is free.
-      if (phase == START || u + 1 < cr.u1) {
-        wait_loads(tot - mark0);
-        mark0 = mark1, mark1 = mark2, mark2 = mark3;
-        --fifo_n;
-      }
-      asm volatile("s_barrier" ::: "memory");
-      if (phase == START) {
-        u = cr.u0;
-        rb_left = cr.stages - cr.st0;
-        in_rb = 0;
-        any_shared = false;
-        phase = UNIT;
-        continue;
-      }
-      ++n_cons;
-      ++in_rb;
-      if (--rb_left == 0 || u + 1 == cr.u1) {
+      wait_oldest();
+      asm volatile("s_barrier" ::: "memory");  // the first unit of problem cp has landed
+      const bool epi = p.prob[cp].epilogue == DFLASH_QMM_EPILOGUE_SILU_MUL;
+      int rb_left = cr.stages - cr.st0;
+      int in_rb = 0;
+      bool any_shared = false;
+#pragma unroll 1
+      for (int u = cr.u0; u < cr.u1; ++u) {
+        // ---- the common case in a loop of its own -------------------------------------------
+        // Units in the interior of a row block, for both cursors: per unit one wait, one
+        // barrier and the loads of one unit, nothing else.  The general code below does the
+        // same thing one unit at a time and handles everything that can happen at a boundary.
+        if (n_issued - n_cons == kChainAhead && i_state == OPEN && i_ready && fifo_n == 2) {
+          int n = rb_left - 1;
+          n = n < cr.u1 - 1 - u ? n : cr.u1 - 1 - u;
+          n = n < iu1 - iu - 1 ? n : iu1 - iu - 1;
+          n = n < istages - ist - 1 ? n : istages - ist - 1;
+          if (n > 0) {
+            bool newest_had_sb = mark0 - mark1 == 8;  // loads of the unit issued last: 6, or 8 with scales and biases
+            int sb_issued = 0;
+            uint32_t slot_off = (uint32_t)slot_i * kSlotBytes + ld * 1024;
+            uint32_t sb_off = kSbOffset + (uint32_t)sb_slot_i * kSbSlotBytes + ld * 1024;
+            uint32_t w_step = (uint32_t)ist * (kUnitK / 2), x_step = (uint32_t)ist * (kUnitK * 2);
+            int st = ist;
+#pragma unroll 1
+            for (int k = 0; k < n; ++k) {
+              // unit u + 1 has landed once at most the newest unit's loads are outstanding
+              if (newest_had_sb) __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
+              else __builtin_amdgcn_s_waitcnt(0x0F70 | 6);
+              asm volatile("s_barrier" ::: "memory");
+              newest_had_sb = (st & (CHUNK - 1)) == 0;
+              if (newest_had_sb) {
+                const uint32_t off = so + (uint32_t)(st / CHUNK) * (CHUNK * kGroups * 2);
+                load16_to_lds(bs + off, lds + sb_off);
+                load16_to_lds(bb + off, lds + sb_off + kSbArrayBytes);
+                ++sb_issued;
+                sb_off += kSbSlotBytes;
+                if (sb_off >= kSbOffset + kSbDepth * kSbSlotBytes) sb_off -= kSbDepth * kSbSlotBytes;
+              }
+              char* dst = lds + slot_off;
+              if (i_coherent) {
+                load16_to_lds_coherent(bx + (xo0 + x_step), dst + kXOffset);
+                load16_to_lds_coherent(bx + (xo1 + x_step), dst + kXOffset + 4096);
+              } else {
+                load16_to_lds(bx + (xo0 + x_step), dst + kXOffset);
+                load16_to_lds(bx + (xo1 + x_step), dst + kXOffset + 4096);
+              }
+              load16_to_lds_stream(bw + (wo0 + w_step), dst);
+              load16_to_lds_stream(bw + (wo1 + w_step), dst + 4096);
+              load16_to_lds_stream(bw + (wo2 + w_step), dst + 8192);
+              load16_to_lds_stream(bw + (wo3 + w_step), dst + 12288);
+              ++st;
+              w_step += kUnitK / 2;
+              x_step += kUnitK * 2;
+              slot_off += kSlotBytes;
+              if (slot_off >= kDepth * kSlotBytes) slot_off -= kDepth * kSlotBytes;
+            }
+            // the books, all at once
+            ist = st, iu += n;
+            slot_i = (slot_i + n) % kDepth;
+            sb_slot_i = (sb_slot_i + sb_issued) % kSbDepth;
+            tot += 6 * n + 2 * sb_issued;
+            mark0 = tot, mark1 = tot - (newest_had_sb ? 8 : 6);  // the two units not yet waited for
+            n_issued += n, n_cons += n;
+            u += n, rb_left -= n, in_rb += n;
+          }
+        }
+        // unit u + 1 has landed, and every worker holds unit u in registers: its slot is free
+#if defined(DFLASH_CHAIN_STAMPS) && DFLASH_CHAIN_STAMPS == 2
+        if (ld == 0) DFLASH_STAMP(8, st_idx);
+#endif
+        if (u + 1 < cr.u1) wait_oldest();
+#if defined(DFLASH_CHAIN_STAMPS) && DFLASH_CHAIN_STAMPS == 2
+        if (ld == 0) DFLASH_STAMP(9, st_idx);
+#elif defined(DFLASH_CHAIN_STAMPS)
+        DFLASH_STAMP(wave, st_idx); ++st_idx;
+#endif
         asm volatile("s_barrier" ::: "memory");
-        if (p.prob[cp].epilogue == DFLASH_QMM_EPILOGUE_SILU_MUL) asm volatile("s_barrier" ::: "memory");
-        if (in_rb != cr.stages) any_shared = true;
-        in_rb = 0;
-        rb_left = cr.stages;
+#if defined(DFLASH_CHAIN_STAMPS) && DFLASH_CHAIN_STAMPS == 2
+        if (ld == 0) DFLASH_STAMP(10, st_idx);
+#endif
+        ++n_cons;
+        top_up();
+#if defined(DFLASH_CHAIN_STAMPS) && DFLASH_CHAIN_STAMPS == 2
+        if (ld == 0) { DFLASH_STAMP(11, st_idx); ++st_idx; }
+#endif
+        ++in_rb;
+        if (--rb_left == 0 || u + 1 == cr.u1) {
+          asm volatile("s_barrier" ::: "memory");
+          if (epi) asm volatile("s_barrier" ::: "memory");
+#ifndef DFLASH_CHAIN_NOHANDOVER
+          if (in_rb != cr.stages) any_shared = true;
+#endif
+          in_rb = 0;
+          rb_left = cr.stages;
+        }
       }
-      if (++u == cr.u1) phase = END;
+      if (any_shared && !handover_deferred(p, lds0, cp)) {
+        asm volatile("s_barrier" ::: "memory");
+        asm volatile("s_barrier" ::: "memory");
+        if (epi) asm volatile("s_barrier" ::: "memory");
+      }
+      if (p.prob[cp].signal) asm volatile("s_barrier" ::: "memory");
     }
     return;
   }
+
+  // Contributors of row block rb of a problem divided as `rx`: the workgroups whose ranges
+  // intersect [lo, lo + stages); owner(v) = ceil((v+1)*grid/units) - 1 holds unit v.
+  auto contributors = [&](const Range& rx, int rb, int& lo_wg, int& hi_wg) __attribute__((always_inline)) {
+    const int lo = rb * rx.stages;
+    lo_wg = (int)((((unsigned)lo + 1u) * (unsigned)rx.grid + rx.units - 1) / (unsigned)rx.units) - 1;
+    hi_wg = (int)((((unsigned)(lo + rx.stages)) * (unsigned)rx.grid + rx.units - 1) / (unsigned)rx.units) - 1;
+  };
 
   // ================================== worker waves ====================================
   const int col = lane & 15;
@@ -396,16 +556,148 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
 #pragma unroll
   for (int j = 0; j < 4; ++j) acc4[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   Operands op[2];
+#ifdef DFLASH_CHAIN_STAMPS
+  int wst_idx = 0;
+#endif
+
+  // ---- output of whole row blocks; `cpx` names the problem they belong to -------------------
+  // Stores tile `wave` of row block rb.  Accumulator r of lane l is (m = 4*(l/16) + r,
+  // column 16*wave + l%16) of the row block.  With the epilogue, waves 0..3 hold the gate
+  // half and `up` the up half of the same 64 output columns; waves 4..7 store nothing.
+  auto store_out = [&](int cpx, size_t index, float v) __attribute__((always_inline)) {
+    CProblem& q = p.prob[cpx];
+    const uint16_t bits = (uint16_t)A::from_f32(v);
+    if (q.signal)
+      __hip_atomic_store(&q.y[index], bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+      q.y[index] = bits;
+  };
+  auto emit = [&](int cpx, int rb, const f32x4_t& acc) __attribute__((always_inline)) {
+    const int n_out = p.prob[cpx].N;
+    const int n = rb * kRows + 16 * wave + col;
+    if (n >= n_out) return;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) store_out(cpx, (size_t)(4 * kblk + r) * n_out + n, acc[r]);
+  };
+  auto emit_epilogue = [&](int cpx, int rb, const f32x4_t& gate, const f32x4_t& up) __attribute__((always_inline)) {
+    const int n_out = p.prob[cpx].N >> 1;
+    const int n = rb * 64 + 16 * wave + col;
+    if (wave >= 4 || n >= n_out) return;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      store_out(cpx, (size_t)(4 * kblk + r) * n_out + n, silu_mul<ACT_FP16>(gate[r], up[r]));
+  };
+  // The up half's waves (4..7) hand their tile to the gate half's (0..3) through LDS.
+  auto exchange_write = [&](int which, const f32x4_t& acc) __attribute__((always_inline)) {
+    if (wave >= 4) {
+      const uint32_t addr = lds0 + kChainExchange + which * 4096 + (wave - 4) * 1024 + lane * 16;
+      asm volatile("ds_write_b128 %0, %1\n s_waitcnt lgkmcnt(0)" : : "v"(addr), "v"(acc) : "memory");
+    }
+  };
+  auto exchange_read = [&](int which) __attribute__((always_inline)) -> f32x4_t {
+    f32x4_t v = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (wave < 4) {
+      const uint32_t addr = lds0 + kChainExchange + which * 4096 + wave * 1024 + lane * 16;
+      asm volatile("ds_read_b128 %0, %1\n s_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
+    }
+    return v;
+  };
+  // ---- hand-over of a problem's shared row blocks `srb` (at most two: the one this workgroup's
+  // range starts in and the one it ends in; see qmm_m16_stream.hip), in three steps:
+  //   1. once every worker's partial stores have been acknowledged, and after a barrier: thread 0
+  //      bumps the arrival counters (wrapping: the last arrival sees n-1 and leaves 0 behind);
+  //   2. thread 0 waits for the counters' answers and leaves "last to arrive" flags in LDS;
+  //   3. after a barrier: a workgroup that arrived last adds the partial tiles in contributor
+  //      order and stores the result.
+  // The steps run back to back at the end of the problem, or - where nothing waits for the
+  // result - at the second and the fourth unit of the next problem, whose barriers then stand
+  // between them and whose arithmetic hides the first two round trips.
+  auto handover_arrive = [&](int cpx, const Range& rx, const int (&srb)[2], uint32_t (&prev)[2]) __attribute__((always_inline)) {
+    if (tid == 0) {
+      uint32_t* const counters = p.counters + p.prob[cpx].counter_base;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        prev[i] = 0u;
+        if (srb[i] >= 0) {
+          int lo_wg, hi_wg;
+          contributors(rx, srb[i], lo_wg, hi_wg);
+          prev[i] = atomicInc(&counters[srb[i]], (uint32_t)(hi_wg - lo_wg));
+        }
+      }
+    }
+  };
+  auto handover_flags = [&](const Range& rx, const int (&srb)[2], uint32_t (&prev)[2]) __attribute__((always_inline)) {
+    if (tid == 0) {
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(prev[0]), "+v"(prev[1]) : : "memory");
+      uint32_t flag[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        int lo_wg = 0, hi_wg = 0;
+        if (srb[i] >= 0) contributors(rx, srb[i], lo_wg, hi_wg);
+        flag[i] = (srb[i] >= 0 && prev[i] == (uint32_t)(hi_wg - lo_wg)) ? 1u : 0u;
+      }
+      asm volatile("ds_write_b32 %0, %1\n ds_write_b32 %0, %2 offset:4\n s_waitcnt lgkmcnt(0)"
+                   :
+                   : "v"(lds0 + kChainFlags), "v"(flag[0]), "v"(flag[1])
+                   : "memory");
+    }
+  };
+  // Returns the number of row blocks summed; `sum` keeps the totals (for the epilogue's second half).
+  auto handover_reduce = [&](int cpx, const Range& rx, const int (&srb)[2], bool (&is_last)[2],
+                             f32x4_t (&sum)[2], bool store) __attribute__((always_inline)) -> int {
+    uint32_t last0, last1;
+    asm volatile("ds_read_b32 %0, %2\n ds_read_b32 %1, %2 offset:4\n s_waitcnt lgkmcnt(0)"
+                 : "=&v"(last0), "=&v"(last1)
+                 : "v"(lds0 + kChainFlags)
+                 : "memory");
+    is_last[0] = __builtin_amdgcn_readfirstlane(last0) != 0;
+    is_last[1] = __builtin_amdgcn_readfirstlane(last1) != 0;
+    const float* const tiles = p.partials + (size_t)p.prob[cpx].partial_base * kPartialFloats;
+    int summed = 0;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      sum[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if (!is_last[i]) continue;
+      int lo_wg, hi_wg;
+      contributors(rx, srb[i], lo_wg, hi_wg);
+      // Only the first contributor can have started before the row block (then the block is the
+      // one its range ends in, slot 1); every later one starts inside it (slot 0).
+      const int which_first = range_begin(rx.units, lo_wg, rx.grid) < srb[i] * rx.stages ? 1 : 0;
+      for (int wg0 = lo_wg; wg0 <= hi_wg; wg0 += 8) {
+        const float* src[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int w = wg0 + j <= hi_wg ? wg0 + j : hi_wg;  // surplus slots re-read the last tile
+          src[j] = tiles + ((size_t)w * 2 + (w == lo_wg ? which_first : 0)) * kPartialFloats + tid * 4;
+        }
+        f32x4_t v[8];
+        load_partials8(src, v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if (wg0 + j <= hi_wg) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sum[i][r] += v[j][r];
+          }
+        }
+      }
+      if (store) emit(cpx, srb[i], sum[i]);
+      ++summed;
+    }
+    return summed;
+  };
+
+  // a hand-over that is spread over the first units of the next problem
+  int ho_cp = -1;           // the problem it belongs to (-1: none)
+  int ho_rb[2] = {-1, -1};  // its shared row blocks
+  uint32_t ho_prev[2] = {0u, 0u};
 
 #pragma unroll 1
   for (int cp = 0; cp < p.count; ++cp) {
-    const Range cr = problem_range(p.prob[cp], block, nblocks);
+    const Range cr = read_range(lds0, cp);
     if (cr.wg < 0) continue;
     CProblem& q = p.prob[cp];
     const bool epi = q.epilogue == DFLASH_QMM_EPILOGUE_SILU_MUL;
-    const int n_out = epi ? q.N >> 1 : q.N;  // columns of y
     float* const partials = p.partials + (size_t)q.partial_base * kPartialFloats;
-    uint32_t* const counters = p.counters + q.counter_base;
     int emitted = 0;  // row blocks of this problem whose output this workgroup has stored
 
     int rd_q = cr.st0 % CHUNK;
@@ -425,46 +717,10 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
       rd_q = (rd_q + 1) & (CHUNK - 1);
     };
 
-    // Stores tile `wave` of row block rb.  Accumulator r of lane l is (m = 4*(l/16) + r,
-    // column 16*wave + l%16) of the row block.  With the epilogue, waves 0..3 hold the gate
-    // half and `other` the up half of the same 64 output columns; waves 4..7 store nothing.
-    auto store_out = [&](size_t index, float v) __attribute__((always_inline)) {
-      const uint16_t bits = (uint16_t)A::from_f32(v);
-      if (q.signal)
-        __hip_atomic_store(&q.y[index], bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      else
-        q.y[index] = bits;
-    };
-    auto emit = [&](int rb, const f32x4_t& acc) __attribute__((always_inline)) {
-      const int n = rb * kRows + 16 * wave + col;
-      if (n >= n_out) return;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) store_out((size_t)(4 * kblk + r) * n_out + n, acc[r]);
-    };
-    auto emit_epilogue = [&](int rb, const f32x4_t& gate, const f32x4_t& up) __attribute__((always_inline)) {
-      const int n = rb * 64 + 16 * wave + col;
-      if (wave >= 4 || n >= n_out) return;
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        store_out((size_t)(4 * kblk + r) * n_out + n, silu_mul<ACT_FP16>(gate[r], up[r]));
-    };
-    // The up half's waves (4..7) hand their tile to the gate half's (0..3) through LDS.
-    auto exchange_write = [&](int which, const f32x4_t& acc) __attribute__((always_inline)) {
-      if (wave >= 4) {
-        const uint32_t addr = lds0 + kChainExchange + which * 4096 + (wave - 4) * 1024 + lane * 16;
-        asm volatile("ds_write_b128 %0, %1\n s_waitcnt lgkmcnt(0)" : : "v"(addr), "v"(acc) : "memory");
-      }
-    };
-    auto exchange_read = [&](int which) __attribute__((always_inline)) -> f32x4_t {
-      f32x4_t v = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      if (wave < 4) {
-        const uint32_t addr = lds0 + kChainExchange + which * 4096 + wave * 1024 + lane * 16;
-        asm volatile("ds_read_b128 %0, %1\n s_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
-      }
-      return v;
-    };
-
     asm volatile("s_barrier" ::: "memory");  // the first unit of this problem has landed
+#ifdef DFLASH_CHAIN_STAMPS
+    if (wave == 0) DFLASH_STAMP(12, cp * 4 + 0);
+#endif
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc4[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     next_addresses();
@@ -474,7 +730,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
     operands_issue_piece<3, SBROW>(rd_x, rd_w, rd_s, op[0], acc4[0]);
     operands_wait(op[0], acc4[0], acc4[1], acc4[2], acc4[3]);
     // The second operand set holds nothing yet (it is filled while the first unit is worked
-    // on): saying so keeps its registers free during the hand-over at the end of a problem.
+    // on): saying so keeps its registers free across the problem boundary.
     asm volatile("" : "=v"(op[1].f0), "=v"(op[1].f1), "=v"(op[1].wq[0]), "=v"(op[1].wq[1]), "=v"(op[1].wq[2]),
                  "=v"(op[1].wq[3]));
     asm volatile("" : "=v"(op[1].sv[0]), "=v"(op[1].sv[1]), "=v"(op[1].sv[2]), "=v"(op[1].sv[3]),
@@ -485,6 +741,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
     int in_rb = 0;                     // units of the current row block this workgroup has done
     int rb = cr.rb0;
     int shared_rb[2] = {-1, -1};       // row blocks whose partial tiles I have stored
+    int unit_no = 0;                   // units of this problem consumed so far
 
 #pragma unroll 1
     while (left > 0) {
@@ -493,13 +750,36 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
         if (left > 0) {
           Operands& cur = op[par];
           Operands& nxt = op[par ^ 1];
+          // ---- the previous problem's hand-over, between this problem's barriers ---------
+          if (ho_cp >= 0) {
+            if (unit_no == kHandoverArriveUnit) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // partial stores acknowledged
+            if (unit_no == kHandoverSumUnit) handover_flags(read_range(lds0, ho_cp), ho_rb, ho_prev);
+          }
+#ifdef DFLASH_CHAIN_STAMPS
+          DFLASH_STAMP(wave, wst_idx);
+#endif
           asm volatile("s_barrier" ::: "memory");
+#ifdef DFLASH_CHAIN_STAMPS
+          ++wst_idx;
+#endif
+          if (ho_cp >= 0) {
+            if (unit_no == kHandoverArriveUnit) handover_arrive(ho_cp, read_range(lds0, ho_cp), ho_rb, ho_prev);
+            if (unit_no == kHandoverSumUnit) {
+              bool is_last[2];
+              f32x4_t sum[2];
+              handover_reduce(ho_cp, read_range(lds0, ho_cp), ho_rb, is_last, sum, true);
+              ho_cp = -1;
+            }
+          }
           const bool fetch = left > 1;
           if (fetch) next_addresses();
+#ifndef DFLASH_CHAIN_NOCOMPUTE  // (timing experiments: the stream without the arithmetic; results are wrong)
           consume_unit<ACT_FP16, SB_FP16, SBROW>(cur, nxt, fetch, rd_x, rd_w, rd_s, acc4, ones, mask, magic);
           if (fetch) operands_wait(nxt, acc4[0], acc4[1], acc4[2], acc4[3]);
+#endif
           --left;
           ++in_rb;
+          ++unit_no;
           if (--rb_left == 0 || left == 0) {
             // ---- a row block ends inside my range -------------------------------------------
             const uint32_t sbase = lds0 + cur_slot;
@@ -512,9 +792,9 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
             if (epi) {
               if (whole) exchange_write(0, acc);
               asm volatile("s_barrier" ::: "memory");
-              if (whole) emit_epilogue(rb, acc, exchange_read(0));
+              if (whole) emit_epilogue(cp, rb, acc, exchange_read(0));
             } else if (whole) {
-              emit(rb, acc);
+              emit(cp, rb, acc);
             }
             if (whole) {
               ++emitted;
@@ -522,8 +802,12 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
               // Other workgroups hold the rest of this row block: partial slot 0 for the row
               // block my range starts in, slot 1 for the one it ends in.
               const int which = rb == cr.rb0 ? 0 : 1;
+#ifndef DFLASH_CHAIN_NOHANDOVER  // (timing experiments: shared row blocks are dropped; results are wrong)
               store_partial(partials + ((size_t)cr.wg * 2 + which) * kPartialFloats + tid * 4, acc);
               shared_rb[which] = rb;
+#else
+              (void)which;
+#endif
             }
             ++rb;
             in_rb = 0;
@@ -536,83 +820,38 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
       // an odd number of units leaves the operands of the next problem's first unit to op[0]
     }
 
+#ifdef DFLASH_CHAIN_STAMPS
+    if (wave == 0) DFLASH_STAMP(12, cp * 4 + 1);
+#endif
     if (shared_rb[0] >= 0 || shared_rb[1] >= 0) {
-      // ---- arrival at the shared row blocks (see qmm_m16_stream.hip) -----------------------
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      asm volatile("s_barrier" ::: "memory");
-      int wg_lo[2], wg_hi[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int lo = shared_rb[i] * cr.stages;
-        wg_lo[i] = (int)((((unsigned)lo + 1u) * (unsigned)cr.grid + cr.units - 1) / (unsigned)cr.units) - 1;
-        wg_hi[i] = (int)((((unsigned)(lo + cr.stages)) * (unsigned)cr.grid + cr.units - 1) / (unsigned)cr.units) - 1;
-      }
-      if (tid == 0) {
-        uint32_t prev[2] = {0u, 0u}, flag[2];
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          if (shared_rb[i] >= 0) prev[i] = atomicInc(&counters[shared_rb[i]], (uint32_t)(wg_hi[i] - wg_lo[i]));
-        }
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-          flag[i] = (shared_rb[i] >= 0 && prev[i] == (uint32_t)(wg_hi[i] - wg_lo[i])) ? 1u : 0u;
-        asm volatile("ds_write_b32 %0, %1\n ds_write_b32 %0, %2 offset:4\n s_waitcnt lgkmcnt(0)"
-                     :
-                     : "v"(lds0 + kChainFlags), "v"(flag[0]), "v"(flag[1])
-                     : "memory");
-      }
-      asm volatile("s_barrier" ::: "memory");
-      uint32_t last0, last1;
-      asm volatile("ds_read_b32 %0, %2\n ds_read_b32 %1, %2 offset:4\n s_waitcnt lgkmcnt(0)"
-                   : "=&v"(last0), "=&v"(last1)
-                   : "v"(lds0 + kChainFlags)
-                   : "memory");
-      const bool is_last[2] = {__builtin_amdgcn_readfirstlane(last0) != 0,
-                               __builtin_amdgcn_readfirstlane(last1) != 0};
-      auto sources = [&](int i, int wg0, const float* (&src)[8]) __attribute__((always_inline)) {
-        const int lo = shared_rb[i] * cr.stages;
-        const int which_first = range_begin(cr.units, wg_lo[i], cr.grid) < lo ? 1 : 0;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int w = wg0 + j <= wg_hi[i] ? wg0 + j : wg_hi[i];
-          src[j] = partials + ((size_t)w * 2 + (w == wg_lo[i] ? which_first : 0)) * kPartialFloats + tid * 4;
-        }
-      };
-      auto add_round = [&](int i, int wg0, const f32x4_t (&v)[8], f32x4_t& acc) __attribute__((always_inline)) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          if (wg0 + j <= wg_hi[i]) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) acc[r] += v[j][r];
-          }
-        }
-      };
-      f32x4_t sum[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        sum[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-        if (!is_last[i]) continue;
-        for (int wg0 = wg_lo[i]; wg0 <= wg_hi[i]; wg0 += 8) {
-          const float* src[8];
-          sources(i, wg0, src);
-          f32x4_t v[8];
-          load_partials8(src, v);
-          add_round(i, wg0, v, sum[i]);
-        }
-        if (!epi) emit(shared_rb[i], sum[i]);
-        ++emitted;
-      }
-      if (epi) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-          if (is_last[i]) exchange_write(i, sum[i]);
+      if (handover_deferred(p, lds0, cp)) {
+        // the next problem's first units carry it
+        ho_cp = cp, ho_rb[0] = shared_rb[0], ho_rb[1] = shared_rb[1];
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         asm volatile("s_barrier" ::: "memory");
+        uint32_t prev[2];
+        handover_arrive(cp, cr, shared_rb, prev);
+        handover_flags(cr, shared_rb, prev);
+        asm volatile("s_barrier" ::: "memory");
+        bool is_last[2];
+        f32x4_t sum[2];
+        emitted += handover_reduce(cp, cr, shared_rb, is_last, sum, !epi);
+        if (epi) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-          if (is_last[i]) emit_epilogue(shared_rb[i], sum[i], exchange_read(i));
+          for (int i = 0; i < 2; ++i)
+            if (is_last[i]) exchange_write(i, sum[i]);
+          asm volatile("s_barrier" ::: "memory");
+#pragma unroll
+          for (int i = 0; i < 2; ++i)
+            if (is_last[i]) emit_epilogue(cp, shared_rb[i], sum[i], exchange_read(i));
+        }
       }
     }
 
+#ifdef DFLASH_CHAIN_STAMPS
+    if (wave == 0) DFLASH_STAMP(12, cp * 4 + 2);
+#endif
     if (q.signal) {
       // every worker's output stores acknowledged, then one bump of the problem's counter
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -621,7 +860,6 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
         __hip_atomic_fetch_add(&done[cp], (uint32_t)emitted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
-
   if (p.has_deps && tid == 0) {
     // The last workgroup to leave puts the problems' counters back to zero for the next launch
     // (every waiting workgroup has passed its waits by then).
@@ -744,6 +982,13 @@ int qmm_chain_launch(const dflash_qmm_problem* problems, int count, void* worksp
 }
 
 }  // namespace dflash
+
+#ifdef DFLASH_CHAIN_STAMPS
+extern "C" int dflash_debug_read_stamps(unsigned long long* out_host) {
+  return (int)hipMemcpyFromSymbol(out_host, HIP_SYMBOL(dflash::stream::g_stamps),
+                                  sizeof(unsigned long long) * 64 * 13 * dflash::stream::kStampSlots);
+}
+#endif
 
 extern "C" size_t dflash_qmm_m16_chain_workspace_bytes(const dflash_qmm_problem* problems, int count,
                                                        int group_size) {
