@@ -31,10 +31,13 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
-# HBM bytes per launch of the qmm kernel on each stack (mean over its launches), from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file scaled by the same counters'
-# reading for a 1 GiB copy (x2.000 / x1.000); None where not measured for the current kernel.
+# HBM bytes per launch of the qmm kernel on each stack (mean over its launches).  Not measured
+# by this file: counters need the profiler.  The figure is copied from the two rocprofv3 --pmc
+# runs (FETCH_SIZE, WRITE_SIZE) of this file summarised in TRAFFIC_SOURCE, scaled by the same
+# counters' reading for a 1 GiB copy (x2.000 / x1.000), and is reported under that label;
+# None where no such run exists for the current kernel.
 MEASURED_TRAFFIC_BYTES = {"27b": 44.32e6, "9b": None}
+TRAFFIC_SOURCE = "profiles/qmm_stream_kernel_27b_stack_pmc.txt"
 
 
 def log(*a):
@@ -155,6 +158,121 @@ def bench_qmm_stack(stack: str, steps: int, warmup: int, device: str, join_gate_
     return res
 
 
+def bench_qmm_chain_stack(stack: str, steps: int, warmup: int, device: str, layers_per_launch: int = 1):
+    """The same stack with the projections of ``layers_per_launch`` layers handed over as one list
+    per launch (``QmmChain``, dflash_qmm_m16_chain): one persistent grid runs them back to back,
+    each divided among the workgroups as a launch of its own would be.  Every projection has an
+    input of its own here, as in the headline (no dependencies between them), and the outputs
+    must equal those of the separate launches bit for bit."""
+    import torch
+
+    from dflash_mlx_amd._native import QMM_CHAIN_MAX
+    from dflash_mlx_amd.verify_qmm import ChainProblem, QmmChain
+    from dflash_mlx_amd.workloads import stack_bytes, stack_linears
+
+    calls = build_stack(stack, device)
+    per_layer = len(stack_linears(stack)[0])
+    per_chain = per_layer * layers_per_launch
+    assert per_chain <= QMM_CHAIN_MAX
+    _, total_bytes = stack_bytes(stack)
+    chains = [QmmChain([ChainProblem(c.x, c.w, c.scales, c.biases) for c in calls[i:i + per_chain]])
+              for i in range(0, len(calls), per_chain)]
+
+    def one_pass():
+        return [chain() for chain in chains]
+
+    separate = run_pass(calls[:per_chain])
+    got = one_pass()
+    torch.cuda.synchronize()
+    for a, b in zip(separate, got[0]):
+        if not torch.equal(a, b):
+            raise RuntimeError("a chained launch differs from the separate launches")
+    graph, _ = capture(one_pass)
+    for _ in range(warmup):
+        graph.replay()
+    wall_ms, ev_ms = time_region(graph.replay, steps)
+    res = dict(launches_per_step=len(chains), projections_per_launch=per_chain,
+               ms_per_step=wall_ms / steps, us_per_layer=ev_ms / steps / (len(calls) / per_layer) * 1e3,
+               avg_launch_us=ev_ms / steps / len(chains) * 1e3, bytes_per_launch=total_bytes / len(chains),
+               frac_hbm=total_bytes / (ev_ms / steps * 1e-3) / HBM_PEAK)
+    del graph, chains, calls, got, separate
+    torch.cuda.empty_cache()
+    return res
+
+
+def bench_mlp_chain(stack: str, steps: int, warmup: int, device: str):
+    """The MLP of every layer of the stack, three ways: (a) gate, up, silu * mul (array
+    operators), down as four separate steps; (b) gate and up in one launch, silu * mul, down;
+    (c) one launch per layer: gate/up with the silu * mul epilogue, and down, which waits
+    inside the launch for the hidden activation while its weights already stream."""
+    import torch
+
+    from dflash_mlx_amd.verify_qmm import ChainProblem, QmmChain, verify_matmul
+    from dflash_mlx_amd.workloads import make_qmm_case, qmm_algorithmic_bytes, seed_for, stack_linears
+
+    linears, layers, cfg = stack_linears(stack)
+    dims = {name: (K, N) for name, K, N in linears}
+    (H, I) = dims["gate_proj"]
+    mlps, nbytes = [], 0
+    for layer in range(layers):
+        g = make_qmm_case(H, I, seed_for(cfg, layer) * 8 + 2, device=device)
+        u = make_qmm_case(H, I, seed_for(cfg, layer) * 8 + 3, device=device)
+        d = make_qmm_case(I, H, seed_for(cfg, layer) * 8 + 4, device=device)
+        gu = tuple(torch.cat([a, b]) for a, b in ((g.w, u.w), (g.scales, u.scales), (g.biases, u.biases)))
+        mlps.append((g, u, d, gu))
+        nbytes += 2 * qmm_algorithmic_bytes(H, I)[1] + qmm_algorithmic_bytes(I, H)[1]
+    torch.cuda.synchronize()
+    silu = torch.nn.functional.silu
+
+    def separate():
+        out = []
+        for g, u, d, _ in mlps:
+            h = silu(verify_matmul(g.x, g.w, g.scales, g.biases)) * verify_matmul(g.x, u.w, u.scales, u.biases)
+            out.append(verify_matmul(h, d.w, d.scales, d.biases))
+        return out
+
+    def joined():
+        out = []
+        for g, u, d, gu in mlps:
+            both = verify_matmul(g.x, *gu)
+            h = silu(both[:, :I]) * both[:, I:]
+            out.append(verify_matmul(h, d.w, d.scales, d.biases))
+        return out
+
+    chains = []
+    for g, u, d, gu in mlps:
+        hidden = ChainProblem(g.x, *gu, epilogue="silu_mul")
+        chains.append(QmmChain([hidden, ChainProblem(hidden, d.w, d.scales, d.biases)]))
+
+    def chained():
+        return [chain()[1] for chain in chains]
+
+    res = {}
+    ref = joined()
+    got = chained()
+    torch.cuda.synchronize()
+    if any(c.error_word() for c in chains):
+        raise RuntimeError("a chained launch gave up waiting")
+    # the hidden activation of (c) is that of (b) rounded once less between gate/up and silu:
+    # the outputs agree to bf16 rounding of the hidden activation, not bit for bit
+    rel = max(float((a.float() - b.float()).norm() / b.float().norm()) for a, b in zip(got, ref))
+    if rel > 2e-2:
+        raise RuntimeError(f"chained MLP differs from the separate launches (relative {rel:.3g})")
+    res["rel_diff_chained_vs_joined"] = rel
+    for name, fn in (("separate_launches", separate), ("gate_up_in_one_launch", joined), ("one_launch_per_layer", chained)):
+        fn()
+        graph, _ = capture(fn)
+        for _ in range(warmup):
+            graph.replay()
+        _, ev_ms = time_region(graph.replay, steps)
+        res[name] = dict(us_per_layer=ev_ms / steps / layers * 1e3,
+                         frac_hbm=nbytes / (ev_ms / steps * 1e-3) / HBM_PEAK)
+        del graph
+    del chains, mlps, ref, got
+    torch.cuda.empty_cache()
+    return res
+
+
 def bench_single_call(device: str, launches: int = 200):
     """config[0]: one 16x4096x4096 call, cold (ring of distinct weight sets larger than
     the 256 MB Infinity Cache) and hot (same weights every launch)."""
@@ -256,10 +374,11 @@ def bench_moe(device: str, steps: int, warmup: int, layers: int = 40, join_gate_
                 frac_hbm=total / (ms * 1e-3) / HBM_PEAK)
 
 
-def bench_replay(device: str, steps: int, warmup: int):
+def bench_replay(device: str, steps: int, warmup: int, tape_dtype: str = "bfloat16"):
     """config[2]: 48 layers x 32 value heads, fp32 128x128 state, 16 recorded steps, all
     applied; one launch per rollback.  Four state sets (800 MB) are rotated so that the
-    Infinity Cache cannot hold the working set."""
+    Infinity Cache cannot hold the working set.  ``tape_dtype``: bfloat16 is what a bf16 model's
+    forward hands over, float32 what the arena keeps by default."""
     import torch
 
     from dflash_mlx_amd.cache import KVCache
@@ -267,7 +386,8 @@ def bench_replay(device: str, steps: int, warmup: int):
     from dflash_mlx_amd.workloads import make_replay_case, replay_algorithmic_bytes
 
     L, H, T = 48, 32, 16
-    sets = [make_replay_case(L, steps=T, seed=7000 + i, device=device) for i in range(4)]
+    dt = getattr(torch, tape_dtype)
+    sets = [make_replay_case(L, steps=T, seed=7000 + i, tape_dtype=dt, device=device) for i in range(4)]
     outs = [torch.empty_like(s.state) for s in sets]
     steps_dev = sets[0].steps
 
@@ -286,7 +406,7 @@ def bench_replay(device: str, steps: int, warmup: int):
     stop.record()
     torch.cuda.synchronize()
     us = start.elapsed_time(stop) / n * 1e3
-    total = replay_algorithmic_bytes(128, 128, T) * L * H
+    total = replay_algorithmic_bytes(128, 128, T, tape_bytes=dt.itemsize) * L * H
     # KV trim of the 16 full-attention layers: offset arithmetic, no device work
     kv = [KVCache() for _ in range(16)]
     for c in kv:
@@ -300,7 +420,55 @@ def bench_replay(device: str, steps: int, warmup: int):
     torch.cuda.empty_cache()
     return dict(us_per_rollback=us, us_per_layer=us / L, gbps=total / us / 1e3,
                 frac_hbm=total / (us * 1e-6) / HBM_PEAK, bytes=total, layers=L, heads=H,
-                steps=T, kv_trim_host_ns_16_layers=trim_ns)
+                steps=T, tape_dtype=tape_dtype, kv_trim_host_ns_16_layers=trim_ns)
+
+
+def bench_rollback_per_layer(device: str, steps: int, warmup: int, tape_dtype: str = "float32"):
+    """The same rollback as the engine makes it without an arena: 48 ``RecurrentRollbackCache``
+    objects, each armed, handed its tape and rolled back on its own (one replay launch and one
+    conv-state rebuild per layer; dflash_mlx/recurrent_rollback_cache.py:149-171).  Arming and
+    recording are reference bookkeeping (no device work) and are left out of the timed region."""
+    import torch
+
+    from dflash_mlx_amd.recurrent_rollback_cache import RecurrentRollbackCache
+    from dflash_mlx_amd.workloads import make_replay_case, replay_algorithmic_bytes
+
+    L, H, T, D, conv_dim = 48, 32, 16, 128, 3 * 32 * 128
+    dt = getattr(torch, tape_dtype)
+    case = make_replay_case(L, steps=T, seed=7100, tape_dtype=dt, device=device)
+    qkv = torch.randn((L, 1, T, conv_dim), device=device, dtype=torch.bfloat16)
+    conv0 = torch.randn((L, 1, 3, conv_dim), device=device, dtype=torch.bfloat16)
+    caches = [RecurrentRollbackCache() for _ in range(L)]
+
+    def arm():
+        for i, c in enumerate(caches):
+            c[0], c[1] = conv0[i], case.state[i]
+            c.arm_rollback(prefix_len=4096)
+            c.record_tape(tape=case.tape[i], k=case.k[i], g=case.g[i], qkv=qkv[i])
+
+    def rollback():
+        for c in caches:
+            c.rollback(T - 1)
+
+    for _ in range(max(warmup, 3)):
+        arm(); rollback()
+    n = max(steps * 3, 20)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev_us = wall_us = 0.0
+    for _ in range(n):
+        arm()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        start.record()
+        rollback()
+        stop.record()
+        torch.cuda.synchronize()
+        wall_us += (time.perf_counter() - t0) * 1e6
+        ev_us += start.elapsed_time(stop) * 1e3
+    total = replay_algorithmic_bytes(D, D, T, tape_bytes=dt.itemsize) * L * H
+    return dict(tape_dtype=tape_dtype, launches_per_rollback=2 * L, us_per_rollback=ev_us / n,
+                us_per_layer=ev_us / n / L, host_us_per_rollback=wall_us / n,
+                frac_hbm=total / (ev_us / n * 1e-6) / HBM_PEAK, bytes=total)
 
 
 def bench_gdn_forward(device: str, steps: int, warmup: int):
@@ -630,6 +798,16 @@ def main() -> int:
                 calls_per_step=q["calls_per_step"], ms_per_step=round(q["ms_per_step"], 4),
                 weight_gbps=round(q["weight_gbps"], 1), avg_launch_us=round(q["avg_launch_us"], 3),
                 frac_hbm=round(q["total_bytes"] / (q["event_ms_per_step"] * 1e-3) / HBM_PEAK, 4))
+        for n_layers in (1, 3):
+            ch = bench_qmm_chain_stack(args.workload, args.steps, args.warmup, device, layers_per_launch=n_layers)
+            log(f"[bench] {args.workload} stack, {n_layers} layer(s) per chained launch: {ch['ms_per_step']:.3f} ms/step, "
+                f"{ch['us_per_layer']:.2f} us/layer")
+            extra[f"stack_{args.workload}_chained_{n_layers}_layer_per_launch"] = {
+                k: (round(v, 4) if isinstance(v, float) else v) for k, v in ch.items()}
+        mlp = bench_mlp_chain(args.workload, args.steps, args.warmup, device)
+        extra[f"mlp_{args.workload}"] = {k: ({kk: round(vv, 4) for kk, vv in v.items()} if isinstance(v, dict)
+                                            else round(v, 6)) for k, v in mlp.items()}
+        log(f"[bench] mlp: " + ", ".join(f"{k} {v['us_per_layer']:.2f} us/layer" for k, v in mlp.items() if isinstance(v, dict)))
         extra["single_call_16x4096x4096"] = {k: {kk: round(vv, 4) for kk, vv in v.items()}
                                              for k, v in bench_single_call(device).items()}
         mo = bench_moe(device, args.steps, args.warmup)
@@ -644,6 +822,14 @@ def main() -> int:
             k: (round(v, 4) if isinstance(v, float) else v) for k, v in ms.items()}
         rp = bench_replay(device, args.steps, args.warmup)
         extra["gdn_tape_replay"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in rp.items()}
+        rp32 = bench_replay(device, args.steps, args.warmup, tape_dtype="float32")
+        extra["gdn_tape_replay_fp32_tape"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in rp32.items()}
+        for dt in ("float32", "bfloat16"):
+            pl = bench_rollback_per_layer(device, args.steps, args.warmup, tape_dtype=dt)
+            log(f"[bench] rollback through 48 per-layer caches ({dt} tape): {pl['us_per_rollback']:.1f} us on the device, "
+                f"{pl['host_us_per_rollback']:.1f} us on the host")
+            extra[f"gdn_rollback_per_layer_cache_{dt}_tape"] = {
+                k: (round(v, 4) if isinstance(v, float) else v) for k, v in pl.items()}
         fw = bench_gdn_forward(device, args.steps, args.warmup)
         log(f"forward with tape: {fw['us_per_layer']:.3f} us/layer, {fw['gbps']:.0f} GB/s")
         extra["gdn_forward_with_tape"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in fw.items()}
@@ -654,9 +840,10 @@ def main() -> int:
         log(f"[bench] replay: {rp['us_per_layer']:.3f} us/layer, {rp['gbps']:.0f} GB/s")
 
     achieved = main_res["bytes_per_launch"] / (main_res["avg_launch_us"] * 1e-6) / 1e9
+    traffic = None if args.packed_weights else MEASURED_TRAFFIC_BYTES.get(args.workload)
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK / 1e9, unit="GB/s",
                     frac=round(achieved * 1e9 / HBM_PEAK, 4),
-                    traffic=None if args.packed_weights else MEASURED_TRAFFIC_BYTES.get(args.workload),
+                    traffic=traffic, traffic_source=TRAFFIC_SOURCE if traffic is not None else None,
                     kernel="qmm_stream_kernel", bytes_per_launch=round(main_res["bytes_per_launch"]),
                     avg_launch_us=round(main_res["avg_launch_us"], 3))
     cpu = None if args.skip_cpu else bench_cpu_baseline(args.workload)
