@@ -40,6 +40,9 @@ MEASURED_TRAFFIC_BYTES = {"27b": 44.32e6, "9b": None}
 TRAFFIC_SOURCE = "profiles/qmm_stream_kernel_27b_stack_pmc.txt"
 
 
+LEGS = ("other_stack", "gate_up", "packed", "chain", "mlp", "single", "moe", "replay", "forward", "sdpa", "glue")
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -744,6 +747,8 @@ def main() -> int:
     ap.add_argument("--workload", default="27b", choices=["27b", "9b"])
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the cpu_baseline leg")
     ap.add_argument("--skip-extra", action="store_true", help="only the headline stack")
+    ap.add_argument("--legs", default="", help="comma-separated subset of the extra measurements to run "
+                                               f"(default all): {', '.join(LEGS)}")
     ap.add_argument("--packed-weights", action="store_true",
                     help="headline stack through verify_matmul_packed (weights stored in the streaming "
                          "kernel's order); off by default: the headline uses the reference's operands")
@@ -779,65 +784,69 @@ def main() -> int:
     log(f"[bench] {args.workload}: {main_res['ms_per_step']:.3f} ms/step, "
         f"{main_res['weight_gbps']:.0f} GB/s weights, {main_res['avg_launch_us']:.2f} us/launch")
     extra = {}
-    if not args.skip_extra:
+    rnd = lambda d: {k: (round(v, 4) if isinstance(v, float) else v) for k, v in d.items()}  # noqa: E731
+    legs = set() if args.skip_extra else set(args.legs.split(",")) if args.legs else set(LEGS)
+    if legs - set(LEGS):
+        print(f"unknown --legs {sorted(legs - set(LEGS))}; known: {', '.join(LEGS)}", file=sys.stderr)
+        return 2
+    if "other_stack" in legs:
         other = "9b" if args.workload == "27b" else "27b"
         o = bench_qmm_stack(other, args.steps, args.warmup, device)
         extra[f"stack_{other}"] = dict(ms_per_step=round(o["ms_per_step"], 4),
                                        weight_gbps=round(o["weight_gbps"], 1),
                                        frac_hbm=round(o["total_bytes"] / (o["event_ms_per_step"] * 1e-3) / HBM_PEAK, 4))
-        j = bench_qmm_stack(args.workload, args.steps, args.warmup, device, join_gate_up=True)
-        extra[f"stack_{args.workload}_gate_up_in_one_launch"] = dict(
-            calls_per_step=j["calls_per_step"], ms_per_step=round(j["ms_per_step"], 4),
-            weight_gbps=round(j["weight_gbps"], 1), avg_launch_us=round(j["avg_launch_us"], 3),
-            frac_hbm=round(j["total_bytes"] / (j["event_ms_per_step"] * 1e-3) / HBM_PEAK, 4))
-        for label, kw in (("packed_weights", dict(packed=True)),
-                          ("gate_up_in_one_launch_packed_weights", dict(packed=True, join_gate_up=True))):
-            q = bench_qmm_stack(args.workload, args.steps, args.warmup, device, **kw)
-            log(f"[bench] {args.workload} stack, {label}: {q['ms_per_step']:.3f} ms/step")
-            extra[f"stack_{args.workload}_{label}"] = dict(
-                calls_per_step=q["calls_per_step"], ms_per_step=round(q["ms_per_step"], 4),
-                weight_gbps=round(q["weight_gbps"], 1), avg_launch_us=round(q["avg_launch_us"], 3),
-                frac_hbm=round(q["total_bytes"] / (q["event_ms_per_step"] * 1e-3) / HBM_PEAK, 4))
+    stack_variants = []
+    if "gate_up" in legs:
+        stack_variants.append(("gate_up_in_one_launch", dict(join_gate_up=True)))
+    if "packed" in legs:
+        stack_variants += [("packed_weights", dict(packed=True)),
+                           ("gate_up_in_one_launch_packed_weights", dict(packed=True, join_gate_up=True))]
+    for label, kw in stack_variants:
+        q = bench_qmm_stack(args.workload, args.steps, args.warmup, device, **kw)
+        log(f"[bench] {args.workload} stack, {label}: {q['ms_per_step']:.3f} ms/step")
+        extra[f"stack_{args.workload}_{label}"] = dict(
+            calls_per_step=q["calls_per_step"], ms_per_step=round(q["ms_per_step"], 4),
+            weight_gbps=round(q["weight_gbps"], 1), avg_launch_us=round(q["avg_launch_us"], 3),
+            frac_hbm=round(q["total_bytes"] / (q["event_ms_per_step"] * 1e-3) / HBM_PEAK, 4))
+    if "chain" in legs:
         for n_layers in (1, 3):
             ch = bench_qmm_chain_stack(args.workload, args.steps, args.warmup, device, layers_per_launch=n_layers)
             log(f"[bench] {args.workload} stack, {n_layers} layer(s) per chained launch: {ch['ms_per_step']:.3f} ms/step, "
                 f"{ch['us_per_layer']:.2f} us/layer")
-            extra[f"stack_{args.workload}_chained_{n_layers}_layer_per_launch"] = {
-                k: (round(v, 4) if isinstance(v, float) else v) for k, v in ch.items()}
+            extra[f"stack_{args.workload}_chained_{n_layers}_layer_per_launch"] = rnd(ch)
+    if "mlp" in legs:
         mlp = bench_mlp_chain(args.workload, args.steps, args.warmup, device)
-        extra[f"mlp_{args.workload}"] = {k: ({kk: round(vv, 4) for kk, vv in v.items()} if isinstance(v, dict)
-                                            else round(v, 6)) for k, v in mlp.items()}
-        log(f"[bench] mlp: " + ", ".join(f"{k} {v['us_per_layer']:.2f} us/layer" for k, v in mlp.items() if isinstance(v, dict)))
-        extra["single_call_16x4096x4096"] = {k: {kk: round(vv, 4) for kk, vv in v.items()}
-                                             for k, v in bench_single_call(device).items()}
+        extra[f"mlp_{args.workload}"] = {k: (rnd(v) if isinstance(v, dict) else round(v, 6)) for k, v in mlp.items()}
+        log("[bench] mlp: " + ", ".join(f"{k} {v['us_per_layer']:.2f} us/layer" for k, v in mlp.items() if isinstance(v, dict)))
+    if "single" in legs:
+        extra["single_call_16x4096x4096"] = {k: rnd(v) for k, v in bench_single_call(device).items()}
+    if "moe" in legs:
         mo = bench_moe(device, args.steps, args.warmup)
-        extra["moe_35b_a3b_stack"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in mo.items()}
+        extra["moe_35b_a3b_stack"] = rnd(mo)
         log(f"[bench] moe: {mo['ms_per_step']:.3f} ms/step, {mo['weight_gbps']:.0f} GB/s")
-        mj = bench_moe(device, args.steps, args.warmup, join_gate_up=True)
-        extra["moe_35b_a3b_stack_gate_up_in_one_launch"] = {k: (round(v, 4) if isinstance(v, float) else v)
-                                                            for k, v in mj.items()}
+        extra["moe_35b_a3b_stack_gate_up_in_one_launch"] = rnd(bench_moe(device, args.steps, args.warmup, join_gate_up=True))
         ms = bench_moe(device, args.steps, args.warmup, join_gate_up=True, shared_as_expert=True)
         log(f"[bench] moe stack, shared expert stored as expert 256: {ms['ms_per_step']:.3f} ms/step")
-        extra["moe_35b_a3b_stack_shared_expert_in_the_gathered_launch"] = {
-            k: (round(v, 4) if isinstance(v, float) else v) for k, v in ms.items()}
+        extra["moe_35b_a3b_stack_shared_expert_in_the_gathered_launch"] = rnd(ms)
+    if "replay" in legs:
         rp = bench_replay(device, args.steps, args.warmup)
-        extra["gdn_tape_replay"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in rp.items()}
-        rp32 = bench_replay(device, args.steps, args.warmup, tape_dtype="float32")
-        extra["gdn_tape_replay_fp32_tape"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in rp32.items()}
+        extra["gdn_tape_replay"] = rnd(rp)
+        log(f"[bench] replay: {rp['us_per_layer']:.3f} us/layer, {rp['gbps']:.0f} GB/s")
+        extra["gdn_tape_replay_fp32_tape"] = rnd(bench_replay(device, args.steps, args.warmup, tape_dtype="float32"))
         for dt in ("float32", "bfloat16"):
             pl = bench_rollback_per_layer(device, args.steps, args.warmup, tape_dtype=dt)
             log(f"[bench] rollback through 48 per-layer caches ({dt} tape): {pl['us_per_rollback']:.1f} us on the device, "
                 f"{pl['host_us_per_rollback']:.1f} us on the host")
-            extra[f"gdn_rollback_per_layer_cache_{dt}_tape"] = {
-                k: (round(v, 4) if isinstance(v, float) else v) for k, v in pl.items()}
+            extra[f"gdn_rollback_per_layer_cache_{dt}_tape"] = rnd(pl)
+    if "forward" in legs:
         fw = bench_gdn_forward(device, args.steps, args.warmup)
-        log(f"forward with tape: {fw['us_per_layer']:.3f} us/layer, {fw['gbps']:.0f} GB/s")
-        extra["gdn_forward_with_tape"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in fw.items()}
-        sd = bench_sdpa(device, args.steps, args.warmup)
-        extra["sdpa_q16_kv4112"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in sd.items()}
-        gl = bench_gdn_glue(device, args.steps, args.warmup)
-        extra["gdn_layer_glue"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in gl.items()}
-        log(f"[bench] replay: {rp['us_per_layer']:.3f} us/layer, {rp['gbps']:.0f} GB/s")
+        log(f"[bench] forward with tape: {fw['us_per_layer']:.3f} us/layer, {fw['gbps']:.0f} GB/s")
+        extra["gdn_forward_with_tape"] = rnd(fw)
+    if "sdpa" in legs:
+        extra["sdpa_q16_kv4112"] = rnd(bench_sdpa(device, args.steps, args.warmup))
+    if "glue" in legs:
+        extra["gdn_layer_glue"] = {k: (round(v, 3) if isinstance(v, float) else v)
+                                   for k, v in bench_gdn_glue(device, args.steps, args.warmup).items()}
 
     achieved = main_res["bytes_per_launch"] / (main_res["avg_launch_us"] * 1e-6) / 1e9
     traffic = None if args.packed_weights else MEASURED_TRAFFIC_BYTES.get(args.workload)
