@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
@@ -21,6 +21,7 @@ QMM_STATIC_SCRATCH_BYTES = 8 << 20  # DFLASH_QMM_STATIC_SCRATCH_BYTES
 QMM_CHAIN_MAX = 16                       # DFLASH_QMM_CHAIN_MAX
 QMM_CHAIN_ERROR_OFFSET = (16384 - 64 + 1) * 4  # DFLASH_QMM_CHAIN_ERROR_OFFSET
 QMM_EPILOGUE_NONE, QMM_EPILOGUE_SILU_MUL = 0, 1
+OPT_GDN_STEP_BY_STEP, OPT_SDPA_SPLITS = 0, 1  # DFLASH_OPT_*
 
 
 class QmmProblem(ctypes.Structure):
@@ -33,6 +34,8 @@ class QmmProblem(ctypes.Structure):
 EXPORTED_SYMBOLS = (
     "dflash_abi_version",
     "dflash_last_error",
+    "dflash_set_option",
+    "dflash_get_option",
     "dflash_qmm_m16_workspace_bytes",
     "dflash_qmm_m16",
     "dflash_qmm_m16_static",
@@ -67,6 +70,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.dflash_abi_version.argtypes = []
     lib.dflash_last_error.restype = c.c_char_p
     lib.dflash_last_error.argtypes = []
+    lib.dflash_set_option.restype = c.c_int
+    lib.dflash_set_option.argtypes = [c.c_int, c.c_int]
+    lib.dflash_get_option.restype = c.c_int
+    lib.dflash_get_option.argtypes = [c.c_int]
     lib.dflash_qmm_m16_workspace_bytes.restype = c.c_size_t
     lib.dflash_qmm_m16_workspace_bytes.argtypes = [c.c_int] * 6
     lib.dflash_qmm_m16.restype = c.c_int

@@ -18,6 +18,7 @@ import torch.nn.functional as F
 
 from .gdn_layer import rms_norm_ops
 from .kernels import batched_sdpa_2pass_exact
+from .verify_linear import shared_input_outputs
 
 _HYBRID_SDPA_EXACT_KV_THRESHOLD = 1024
 
@@ -141,11 +142,10 @@ def _project(self, x: torch.Tensor, cache: Optional[Any]):
     B, L, _ = x.shape
     num_attention_heads = _attention_num_heads(self)
     num_key_value_heads = _attention_num_kv_heads(self)
-    q_proj_output = self.q_proj(x)
+    # one launch for the three where fuse_shared_input_linears joined them
+    q_proj_output, keys, values = shared_input_outputs(self, ("q_proj", "k_proj", "v_proj"), x)
     queries, gate = torch.chunk(q_proj_output.reshape(B, L, num_attention_heads, -1), 2, dim=-1)
     gate = gate.reshape(B, L, -1)
-    keys = self.k_proj(x)
-    values = self.v_proj(x)
     queries = self.q_norm(queries).transpose(1, 2)
     keys = self.k_norm(keys.reshape(B, L, num_key_value_heads, -1)).transpose(1, 2)
     values = values.reshape(B, L, num_key_value_heads, -1).transpose(1, 2)

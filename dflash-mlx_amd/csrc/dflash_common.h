@@ -10,6 +10,7 @@ namespace dflash {
 
 // printf-style message kept per host thread; returned by dflash_last_error().
 void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+int option(int which);  // dflash_set_option's value for DFLASH_OPT_*
 
 #define DFLASH_REQUIRE(cond, code, ...)  \
   do {                                   \

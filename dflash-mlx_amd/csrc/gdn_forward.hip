@@ -763,9 +763,7 @@ int gdn_forward_launch(const char* who, const void* q, const void* k, const void
   const bool fast = Dk == 128 && Dv == 128 && T >= 1 && smem <= 64 * 1024 &&
                     (state_dtype != DFLASH_FP32 ||
                      (((uintptr_t)state_in % 16) == 0 && ((uintptr_t)state_out % 16) == 0));
-  // DFLASH_GDN_SEQUENTIAL=1 keeps the step-by-step kernel for every shape (read per call: A/B runs)
-  const char* sequential_env = getenv("DFLASH_GDN_SEQUENTIAL");
-  const bool no_chunk = sequential_env && sequential_env[0] == '1';
+  const bool no_chunk = option(DFLASH_OPT_GDN_STEP_BY_STEP) != 0;  // (tests of one kernel against the other)
   const bool aligned16 = (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)y | (uintptr_t)tape |
                            (uintptr_t)z | (uintptr_t)norm_weight) % 16) == 0;
   const bool chunk = fast && !g_per_dk && state_dtype == DFLASH_FP32 && T <= 16 && aligned16 && !no_chunk;

@@ -674,12 +674,8 @@ int qmm_stream_grid() {
 // (5120x7168: 10.7 us with 224 workgroups against 11.8 us with 256; 17408x5120: 15.9 us with 240
 // against 17.2 us), and among such grids with the same longest range the smaller one is faster
 // (5120x5120: 200 workgroups 9.65 us, 240 9.94 us, 256 10.06 us).  Grids are kept multiples of
-// eight, the number of XCDs the ranges are dealt over.  DFLASH_QMM_GRID=n overrides (experiments).
+// eight, the number of XCDs the ranges are dealt over.
 int qmm_stream_pick_grid(int units, int row_blocks, int cus) {
-  if (const char* e = getenv("DFLASH_QMM_GRID")) {
-    const int g = atoi(e);
-    if (g > 0 && g <= cus) return g < units ? g : units;
-  }
   if (cus > units) return units;
   constexpr int kUnalignedPenalty = 2;  // units
   int best = cus;

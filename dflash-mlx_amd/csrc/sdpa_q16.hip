@@ -356,9 +356,8 @@ __global__ __launch_bounds__(256) void sdpa_q16_merge_kernel(SdpaArgs a, int D) 
 int pick_splits(int B, int Hk, int N, int* keys_per_split) {
   // About one workgroup per compute unit, and never less than 128 keys per split: every split
   // adds B * Hq * 16 * (2 D + 8) bytes of partial results, written once and read once.
-  // DFLASH_SDPA_SPLITS=n asks for n ranges instead (read per call: experiments and tests)
-  const char* env = getenv("DFLASH_SDPA_SPLITS");
-  const int forced = env ? atoi(env) : 0;
+  // DFLASH_OPT_SDPA_SPLITS = n asks for n ranges instead (tests)
+  const int forced = option(DFLASH_OPT_SDPA_SPLITS);
   int want = forced > 0 ? forced : (256 + B * Hk - 1) / (B * Hk);
   const int most = (N + 127) / 128;
   if (want > most) want = most;

@@ -30,6 +30,7 @@ import torch.nn as nn
 from . import _native
 from .kernels import _DTYPE_CODE, fused_output_norm_applies, gated_delta_kernel_with_tape
 from .recurrent_rollback_cache import RecurrentRollbackCache
+from .verify_linear import shared_input_outputs
 
 _EXACT_SMALL_PROJ_PAD_M = 16
 
@@ -221,10 +222,9 @@ def _gdn_call(self, inputs: torch.Tensor, mask: Optional[torch.Tensor], cache: O
               record: bool) -> torch.Tensor:
     """The body shared by the plain and the speculative call (dflash_mlx/runtime.py:359-453)."""
     B, S, _ = inputs.shape
-    qkv = self.in_proj_qkv(inputs)
-    z = self.in_proj_z(inputs).reshape(B, S, self.num_v_heads, self.head_v_dim)
-    b = self.in_proj_b(inputs)
-    a = self.in_proj_a(inputs)
+    # one launch for those of the four that fuse_shared_input_linears joined
+    qkv, z, b, a = shared_input_outputs(self, ("in_proj_qkv", "in_proj_z", "in_proj_b", "in_proj_a"), inputs)
+    z = z.reshape(B, S, self.num_v_heads, self.head_v_dim)
 
     conv_state = cache[0] if cache is not None else None
     conv_next, q, k, v, g, beta = gdn_prepare(

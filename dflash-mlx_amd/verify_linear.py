@@ -7,12 +7,15 @@ same install / uninstall entry points (:146-196).  A swapped module shares the
 packed weight, scales and biases tensors with the module it replaces.
 
 ``fuse_shared_input_linears`` has no counterpart in the reference.  A verify call of
-16 x K against N rows costs about 8 us on this part before and after its weights stream
+16 x K against N rows costs about 6 us on this part before and after its weights stream
 (first-access latency, split-K hand-over, the gap to the next launch), whatever N is, so
 projections that read the same activations - gate/up of an MLP, q/k/v of an attention
 layer, the input projections of a linear-attention layer - are cheaper as one launch over
-their rows laid end to end than as one launch each: the module tree, every module's own
-tensors (now views into the shared storage) and all results stay as they were.
+their rows laid end to end than as one launch each.  The joint launch is an explicit call:
+the parent module asks for all of them at once (``shared_input_outputs(parent, names, x)``,
+as the attention and linear-attention layers of this package do).  The module tree and every
+module's own tensors (now views into the shared storage) stay as they were, and a member
+called on its own still answers, from its rows, with a launch of its own.
 """
 from __future__ import annotations
 
@@ -96,17 +99,13 @@ SHARED_INPUT_GROUPS: Tuple[Tuple[str, ...], ...] = (
 )
 
 
-class SharedInputGroup:
-    """Rows of several projections laid end to end: one verify launch serves them all.
+class FusedProjections:
+    """Rows of several projections of one parent module laid end to end: ``group(x)`` is one
+    verify launch, ``x @ [W_0; W_1; ...]^T``, and returns every member's columns of it."""
 
-    The first member asked about an input computes ``x @ [W_0; W_1; ...]^T`` and every member
-    takes its columns of that product, once; a member asking twice, or about another input,
-    starts a new product.  An input is recognised by storage address, shape, strides, dtype and
-    version counter, and the group holds on to it until every member has been served, so that
-    no other live tensor can take its place in between."""
-
-    def __init__(self, members: Sequence["VerifyQuantizedLinear"]):
+    def __init__(self, names: Sequence[str], members: Sequence["VerifyQuantizedLinear"]):
         first = members[0]
+        self.names = tuple(names)
         self.group_size, self.bits = first.group_size, first.bits
         self.weight = torch.cat([m.weight for m in members], dim=0).contiguous()
         self.scales = torch.cat([m.scales for m in members], dim=0).contiguous()
@@ -117,32 +116,45 @@ class SharedInputGroup:
             n = int(m.weight.shape[0])
             self.bounds.append((row, row + n))
             row += n
-        self._key = None
-        self._input: Optional[torch.Tensor] = None
-        self._product: Optional[torch.Tensor] = None
-        self._pending = 0
         self._packed = None  # the joint matrix in the streaming kernel's order (pack_verify_linears)
 
-    @staticmethod
-    def _key_of(x: torch.Tensor):
-        return (x.data_ptr(), tuple(x.shape), tuple(x.stride()), x.dtype, x._version)
+    def applies(self, parent: nn.Module, x: torch.Tensor) -> bool:
+        """The joint launch gives what ``parent``'s members would give one by one: 16 rows on the
+        verify path, on the device the joint matrix lives on, every member still a view into it
+        (a module moved with ``.to()``, or replaced, has left) and behind no wrapper that would
+        pad this input."""
+        m = 1
+        for d in x.shape[:-1]:
+            m *= d
+        if m != 16 or x.device != self.weight.device or not _should_use_verify(x, self.group_size, self.bits, True):
+            return False
+        for index, name in enumerate(self.names):
+            mod = getattr(parent, name, None)
+            if getattr(mod, "_dflash_exact_small_proj_wrapped", False):
+                if x.ndim == 3 and x.shape[1] < mod.pad_m:
+                    return False
+                mod = mod.linear
+            if getattr(mod, "_shared_input", None) != (self, index):
+                return False
+        return True
 
-    def member_output(self, index: int, x: torch.Tensor) -> torch.Tensor:
-        bit = 1 << index
-        if self._product is None or not (self._pending & bit) or self._key != self._key_of(x):
-            if self._packed is not None and x.is_cuda:
-                self._product = verify_matmul_packed(x, self._packed)
-            else:
-                self._product = verify_matmul(x, self.weight, self.scales, self.biases, transpose=True,
-                                              group_size=self.group_size, bits=self.bits)
-            self._key, self._input = self._key_of(x), x
-            self._pending = (1 << len(self.bounds)) - 1
-        lo, hi = self.bounds[index]
-        out = self._product[..., lo:hi]
-        self._pending &= ~bit
-        if not self._pending:
-            self._key = self._input = self._product = None
-        return out
+    def __call__(self, x: torch.Tensor) -> Tuple[torch.Tensor, ...]:
+        if self._packed is not None and x.is_cuda:
+            product = verify_matmul_packed(x, self._packed)
+        else:
+            product = verify_matmul(x, self.weight, self.scales, self.biases, transpose=True,
+                                    group_size=self.group_size, bits=self.bits)
+        return tuple(product[..., lo:hi] for lo, hi in self.bounds)
+
+
+def shared_input_outputs(parent: nn.Module, names: Sequence[str], x: torch.Tensor) -> Tuple[torch.Tensor, ...]:
+    """``tuple(getattr(parent, n)(x) for n in names)``, with the projections that
+    ``fuse_shared_input_linears`` joined under ``parent`` served by their one launch."""
+    outs = {}
+    for group in getattr(parent, "_dflash_fused", ()):
+        if all(n in names for n in group.names) and group.applies(parent, x):
+            outs.update(zip(group.names, group(x)))
+    return tuple(outs[n] if n in outs else getattr(parent, n)(x) for n in names)
 
 
 def _build_dispatch(obj: "VerifyQuantizedLinear"):
@@ -153,16 +165,13 @@ def _build_dispatch(obj: "VerifyQuantizedLinear"):
     bits = obj.bits
     mode = obj.mode
     bias = obj.bias
-    shared = getattr(obj, "_shared_input", None)
     packed = getattr(obj, "_packed", None)
 
     def call(x: torch.Tensor) -> torch.Tensor:
         m = 1
         for d in x.shape[:-1]:
             m *= d
-        if m == 16 and shared is not None and _should_use_verify(x, gs, bits, True):
-            y = shared[0].member_output(shared[1], x)
-        elif m == 16 and packed is not None and x.is_cuda and _should_use_verify(x, gs, bits, True):
+        if m == 16 and packed is not None and x.is_cuda and _should_use_verify(x, gs, bits, True):
             y = verify_matmul_packed(x, packed)
         elif m == 16:
             y = verify_matmul(x, w, s, b, transpose=True, group_size=gs, bits=bits)
@@ -191,7 +200,8 @@ class VerifyQuantizedLinear(QuantizedLinear):
 
     def _apply(self, fn, *args, **kwargs):
         # .to()/.cuda() replace the buffers; re-bind the dispatch closure to the new ones.
-        # The new buffers are no longer views into a shared-input group's storage: leave it.
+        # The new buffers are no longer views into a joint matrix: leave the group (its
+        # ``applies`` sees that and stops serving the parent).
         out = super()._apply(fn, *args, **kwargs)
         object.__setattr__(self, "_shared_input", None)
         object.__setattr__(self, "_packed", None)  # a packed copy stays where it was made
@@ -258,7 +268,8 @@ def fuse_shared_input_linears(model: nn.Module, *,
     """Joins, under every parent module, the swapped projections named by one of ``groups``
     (those present, when at least two of them are and they agree in K, group size, dtype and
     device, K is a multiple of 512, the rows add up to a multiple of 32 and none adds a bias vector)
-    into a ``SharedInputGroup``; narrow projections left out of the swap (N a multiple of 16) join too.  Call it after
+    into a ``FusedProjections`` kept in ``parent._dflash_fused`` for ``shared_input_outputs``; narrow
+    projections left out of the swap (N a multiple of 16) join too.  Call it after
     ``install_verify_linears`` and after the model sits on its device.  Returns the number of
     groups formed.  ``DFLASH_VERIFY_FUSE_SHARED_INPUT=0`` turns it into a no-op."""
     if os.environ.get("DFLASH_VERIFY_FUSE_SHARED_INPUT", "1").strip() == "0":
@@ -282,15 +293,15 @@ def fuse_shared_input_linears(model: nn.Module, *,
 
     for parent in list(model.modules()):
         for names in groups:
-            found = [c for c in (candidate(parent, n) for n in names) if c is not None]
-            if len(found) < 2 or len({id(c[2]) for c in found}) != len(found):
+            found = [(n,) + c for n, c in ((n, candidate(parent, n)) for n in names) if c is not None]
+            if len(found) < 2 or len({id(c[3]) for c in found}) != len(found):
                 continue
-            ref = found[0][2]
+            ref = found[0][3]
             same = all(m.weight.shape[1] == ref.weight.shape[1] and m.group_size == ref.group_size and
                        m.bits == ref.bits and m.mode == ref.mode and m.scales.dtype == ref.scales.dtype and
                        m.weight.dtype == ref.weight.dtype and m.weight.device == ref.weight.device
-                       for _, _, m in found)
-            rows = sum(int(m.weight.shape[0]) for _, _, m in found)
+                       for _, _, _, m in found)
+            rows = sum(int(m.weight.shape[0]) for _, _, _, m in found)
             # K a multiple of 512: no variant's divisibility guard can send the joint product
             # to the stock operator, whose rounding differs between one matrix and several
             k = int(ref.weight.shape[1]) * (32 // ref.bits)
@@ -298,12 +309,13 @@ def fuse_shared_input_linears(model: nn.Module, *,
                     rows >= _env_int("DFLASH_VERIFY_MAX_N", _VERIFY_MAX_N_DEFAULT):
                 continue
             members = []
-            for holder, attr, m in found:
+            for _, holder, attr, m in found:
                 if not isinstance(m, VerifyQuantizedLinear):  # a narrow projection: swapped now that it has a group
                     m = VerifyQuantizedLinear.from_quantized(m)
                     setattr(holder, attr, m)
                 members.append(m)
-            group = SharedInputGroup(members)
+            group = FusedProjections([n for n, _, _, _ in found], members)
+            object.__setattr__(parent, "_dflash_fused", tuple(getattr(parent, "_dflash_fused", ())) + (group,))
             for index, (m, (lo, hi)) in enumerate(zip(members, group.bounds)):
                 # the module's own tensors become views: the stock path and state_dict see the
                 # same values, and the separate copies are released

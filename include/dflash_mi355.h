@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 10
+#define DFLASH_ABI_VERSION 11
 
 enum {
   DFLASH_OK = 0,
@@ -52,6 +52,21 @@ enum { DFLASH_QMM_KERNEL_AUTO = 0, DFLASH_QMM_KERNEL_TILE = 1, DFLASH_QMM_KERNEL
 
 int dflash_abi_version(void);
 const char* dflash_last_error(void);
+
+/*
+ * Process-wide switches for tests and A/B measurements; no counterpart in the reference (whose
+ * kernels have none).  They are plain integers read by the entry points named below, 0 (the
+ * default) meaning "decide as documented"; nothing on a launch path reads the environment.
+ *   DFLASH_OPT_GDN_STEP_BY_STEP  1: dflash_gdn_forward_tape{,_norm} keep the step-by-step kernel
+ *                                where the block kernel would apply
+ *   DFLASH_OPT_SDPA_SPLITS       n > 0: dflash_sdpa_q16 (and its workspace size) cut the keys into
+ *                                n ranges (fewer if a range would fall below one tile)
+ * dflash_set_option returns 0, or DFLASH_ERR_ARG for an unknown option or a negative value;
+ * dflash_get_option returns the value, or DFLASH_ERR_ARG.
+ */
+enum { DFLASH_OPT_GDN_STEP_BY_STEP = 0, DFLASH_OPT_SDPA_SPLITS = 1, DFLASH_OPT_COUNT = 2 };
+int dflash_set_option(int option, int value);
+int dflash_get_option(int option);
 
 /*
  * M=16 int4 affine quantized matmul, y[16,N] = x[16,K] . (scale*q + bias)^T.
@@ -255,8 +270,8 @@ int dflash_tape_replay(const void* tape, const void* k, const void* g, const voi
  *   tape      [slots, T, Hv, Dv]   fp32 (output)
  *   mask      [slots, T] uint8 or NULL
  * 128 x 128 heads take register-resident kernels: one gate per head with an fp32 state and
- * T <= 16 the block kernel on the fp32 matrix cores (closed form of the recurrence; the
- * environment variable DFLASH_GDN_SEQUENTIAL=1 turns it off), the rest a step-by-step kernel
+ * T <= 16 the block kernel on the fp32 matrix cores (closed form of the recurrence; the option
+ * DFLASH_OPT_GDN_STEP_BY_STEP turns it off), the rest a step-by-step kernel
  * while T*(3*128 + (g_per_dk ? 128 : 1) + 2)*4 bytes fit 64 KiB of LDS; every other shape a
  * simple kernel that keeps S in state_out.
  */

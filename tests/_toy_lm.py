@@ -6,6 +6,7 @@ import torch.nn as nn
 
 from dflash_mlx_amd import gdn_layer as G
 from dflash_mlx_amd.quantized import QuantizedLinear
+from dflash_mlx_amd.verify_linear import shared_input_outputs
 
 
 def _qlinear(n_in, n_out, gen, dtype, scale=1.0):
@@ -45,7 +46,8 @@ class MLP(nn.Module):
         self.down_proj = _qlinear(inner, hidden, gen, dtype)
 
     def forward(self, x):
-        return self.down_proj(G.silu_ops(self.gate_proj(x)) * self.up_proj(x))
+        gate, up = shared_input_outputs(self, ("gate_proj", "up_proj"), x)
+        return self.down_proj(G.silu_ops(gate) * up)
 
 
 class Block(nn.Module):

@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 import torch
 
+import dflash_mlx_amd._native as nat
 from dflash_mlx_amd.gdn_layer import gated_norm
 from dflash_mlx_amd.kernels import (_gated_delta_ops_with_tape, fused_output_norm_applies,
                                     gated_delta_kernel_with_tape, tape_replay_kernel)
@@ -160,9 +161,11 @@ def test_closed_form_equals_the_sequential_kernel(native_lib, monkeypatch):
     mask = torch.ones((2, 16), dtype=torch.bool)
     mask[0, 5:8] = False
     block = _run(args, mask)
-    monkeypatch.setenv("DFLASH_GDN_SEQUENTIAL", "1")
-    steps = _run(args, mask)
-    monkeypatch.delenv("DFLASH_GDN_SEQUENTIAL")
+    assert native_lib.dflash_set_option(nat.OPT_GDN_STEP_BY_STEP, 1) == 0
+    try:
+        steps = _run(args, mask)
+    finally:
+        native_lib.dflash_set_option(nat.OPT_GDN_STEP_BY_STEP, 0)
     for a, b in zip(block, steps):
         assert _rel(_f64(a), _f64(b)) <= 2e-5
     assert _rel(_f64(block[2]), _f64(steps[2])) > 0     # two different kernels did run

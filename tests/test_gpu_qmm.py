@@ -358,13 +358,17 @@ def test_shared_input_projections_in_one_launch(verify_env, native_lib, c_oracle
     launches = []
     direct = VL.verify_matmul
     monkeypatch.setattr(VL, "verify_matmul", lambda x, w, *a, **k: (launches.append(int(w.shape[0])), direct(x, w, *a, **k))[1])
-    for mod in (model.mlp.gate_proj, model.mlp.up_proj):
-        object.__setattr__(mod, "_call_fn", VL._build_dispatch(mod))
     x = cases["gate_proj"].x.to(DEV)
-    out = {n: getattr(model.mlp, n)(x) for n in cases}
+    out = dict(zip(cases, VL.shared_input_outputs(model.mlp, tuple(cases), x)))
     torch.cuda.synchronize()
     assert launches == [1536 + 2080]
     group = model.mlp.gate_proj._shared_input[0]
+    # a member asked on its own answers from its rows, with a launch of its own
+    alone = model.mlp.up_proj(x)
+    assert launches == [1536 + 2080, 2080]
+    assert torch.equal(alone, VQ.verify_matmul(x, group.weight[1536:], group.scales[1536:], group.biases[1536:],
+                                               group_size=64, bits=4))
+    del launches[1:]
     joint = VQ.verify_matmul(x, group.weight, group.scales, group.biases, group_size=64, bits=4)
     assert torch.equal(torch.cat([out["gate_proj"], out["up_proj"]], dim=-1), joint)
     for name, c in cases.items():
@@ -397,12 +401,8 @@ def test_input_projections_of_a_linear_attention_layer_in_one_launch(verify_env,
     launches = []
     direct = VL.verify_matmul
     monkeypatch.setattr(VL, "verify_matmul", lambda x, w, *a, **k: (launches.append(int(w.shape[0])), direct(x, w, *a, **k))[1])
-    for name in cases:
-        mod = getattr(model.linear_attn, name)
-        mod = getattr(mod, "linear", mod)
-        object.__setattr__(mod, "_call_fn", VL._build_dispatch(mod))
     x = cases["in_proj_qkv"].x.to(DEV).reshape(1, 16, K)
-    out = {n: getattr(model.linear_attn, n)(x) for n in cases}
+    out = dict(zip(cases, VL.shared_input_outputs(model.linear_attn, tuple(cases), x)))
     torch.cuda.synchronize()
     assert launches == [1024 + 512 + 48 + 48]
     for name, c in cases.items():

@@ -137,18 +137,21 @@ def test_modules_switch_to_their_packed_copy(verify_env, native_lib):
     assert pack_verify_linears(model) == 2 and pack_verify_linears(model) == 0  # down_proj and the gate/up group
     assert model.mlp.down_proj._packed is not None and model.mlp.odd._packed is None
     assert model.mlp.gate_proj._packed is None and group._packed is not None and group._packed.N == 1024
-    assert torch.equal(torch.cat([model.mlp.gate_proj(xg), model.mlp.up_proj(xg)], dim=-1), joint)
-    called = []
     import dflash_mlx_amd.verify_linear as VL
+    called = []
     real = VL.verify_matmul_packed
     try:
         VL.verify_matmul_packed = lambda x, p: (called.append(p.N), real(x, p))[1]
         object.__setattr__(model.mlp.down_proj, "_call_fn", VL._build_dispatch(model.mlp.down_proj))
-        after = {n: getattr(model.mlp, n)(cases[n].x.to(DEV)) for n in cases}
+        both = VL.shared_input_outputs(model.mlp, ("gate_proj", "up_proj"), xg)
+        after = {n: getattr(model.mlp, n)(cases[n].x.to(DEV)) for n in ("down_proj", "odd")}
     finally:
         VL.verify_matmul_packed = real
     torch.cuda.synchronize()
-    assert called == [1024, 1024, 1024]  # the gate/up group for each of the two inputs, then down_proj
+    assert called == [1024, 1024]  # the gate/up group's joint matrix, then down_proj
+    assert torch.equal(torch.cat(both, dim=-1), joint)
+    # members asked one by one: their rows of the row-major joint matrix, the same values
+    assert torch.equal(model.mlp.gate_proj(xg), before["gate_proj"])
     for n in ("down_proj", "odd"):
         assert torch.equal(before[n], after[n])
     x3 = torch.randn(3, 2048, device=DEV).to(torch.bfloat16)

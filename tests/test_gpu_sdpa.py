@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 import torch
 
+import dflash_mlx_amd._native as nat
 from dflash_mlx_amd.kernels import batched_sdpa_2pass_exact
 from oracle import dflash_oracle as O
 
@@ -49,9 +50,12 @@ def test_against_the_oracle(native_lib, name, B, Hq, Hk, N, D):
 @pytest.mark.parametrize("splits", [1, 2, 5, 64])
 def test_any_number_of_key_ranges_gives_the_same_attention(native_lib, monkeypatch, splits):
     q, k, v = _case(1, 4, 2, 700, 128, 77, "bf16")
-    monkeypatch.setenv("DFLASH_SDPA_SPLITS", str(splits))
-    out = batched_sdpa_2pass_exact(_dev(q, "bf16"), _dev(k, "bf16"), _dev(v, "bf16"), 0.1)
-    torch.cuda.synchronize()
+    assert native_lib.dflash_set_option(nat.OPT_SDPA_SPLITS, splits) == 0
+    try:
+        out = batched_sdpa_2pass_exact(_dev(q, "bf16"), _dev(k, "bf16"), _dev(v, "bf16"), 0.1)
+        torch.cuda.synchronize()
+    finally:
+        native_lib.dflash_set_option(nat.OPT_SDPA_SPLITS, 0)
     _check(out, O.sdpa_q16_exact(q, k, v, 0.1), v, "bf16", 4)
 
 

@@ -355,7 +355,8 @@ class _SharedInputToy(nn.Module):
 
 def test_fuse_shared_input_groups_keep_every_result(monkeypatch):
     """Joined projections: the modules keep their values (as views of one storage), the stock
-    path is untouched, and with the verify gate open one product serves all members once."""
+    path is untouched, and with the verify gate open a parent that asks for all members at once
+    (``shared_input_outputs``) gets them from one product."""
     import dflash_mlx_amd.verify_linear as VL
 
     monkeypatch.delenv("DFLASH_VERIFY_QMM", raising=False)
@@ -380,7 +381,7 @@ def test_fuse_shared_input_groups_keep_every_result(monkeypatch):
     assert torch.equal(m.mlp.up_proj(x5), quantized_matmul(x5, before["mlp.up_proj.weight"], before["mlp.up_proj.scales"],
                                                            before["mlp.up_proj.biases"]))
 
-    # gate open, device product replaced by the stock operator: count the joint products
+    # gate open, device product replaced by the stock operator: count the products and their rows
     calls = []
 
     def product(x, w, s, b, **kw):
@@ -389,30 +390,33 @@ def test_fuse_shared_input_groups_keep_every_result(monkeypatch):
 
     monkeypatch.setattr(VL, "verify_matmul", product)
     monkeypatch.setattr(VL, "_should_use_verify", lambda x, gs, bits, tr: True)
-    for mod in (m.mlp.gate_proj, m.mlp.up_proj):
-        object.__setattr__(mod, "_call_fn", VL._build_dispatch(mod))
     full = quantized_matmul(x, group.weight, group.scales, group.biases)
-    g1, u1 = m.mlp.gate_proj(x), m.mlp.up_proj(x)
+    # the parent asks for both at once: one product over the joint rows
+    g1, u1 = VL.shared_input_outputs(m.mlp, ("gate_proj", "up_proj"), x)
     assert calls == [640] and torch.equal(g1, full[:, :256]) and torch.equal(u1, full[:, 256:])
-    assert group._input is None and group._product is None           # all served: nothing held
-    # same member twice, then another input with one member left waiting
-    m.mlp.gate_proj(x)
-    m.mlp.gate_proj(x)
-    assert calls == [640, 640, 640] and group._input is x
-    x2 = torch.randn(16, 512).to(torch.bfloat16)
-    u2 = m.mlp.up_proj(x2)
-    assert calls == [640] * 4 and torch.equal(u2, quantized_matmul(x2, group.weight, group.scales, group.biases)[:, 256:])
-    # an input changed in place is a new input
-    g3 = m.mlp.gate_proj(x2)
-    assert calls == [640] * 4                      # gate of x2 was still pending
-    m.mlp.gate_proj(x2)
-    x2.add_(1.0)
-    u4 = m.mlp.up_proj(x2)
-    assert calls == [640] * 6 and torch.equal(u4, quantized_matmul(x2, group.weight, group.scales, group.biases)[:, 256:])
-    assert g3.shape == (16, 256)
+    # a member on its own answers from its rows with a product of its own; nothing is remembered
+    assert torch.equal(m.mlp.up_proj(x), quantized_matmul(x, group.weight[256:], group.scales[256:], group.biases[256:]))
+    assert calls == [640, 384]
+    x.add_(1.0)   # (an input changed in place is just an input)
+    g2, u2 = VL.shared_input_outputs(m.mlp, ("gate_proj", "up_proj"), x)
+    full2 = quantized_matmul(x, group.weight, group.scales, group.biases)
+    assert calls == [640, 384, 640] and torch.equal(g2, full2[:, :256]) and torch.equal(u2, full2[:, 256:])
+    # names that are only partly joined: q and k by their launch, v (adds a bias) by itself
+    q, k, v = VL.shared_input_outputs(m.attn, ("q_proj", "k_proj", "v_proj"), x)
+    assert calls[3:] == [320, 64] and q.shape == (16, 256) and k.shape == (16, 64)
+    assert torch.equal(v, m.attn.v_proj(x))
+    # a parent without groups, and an input that is not a verify block: every member by itself
+    del calls[:]
+    og, ou = VL.shared_input_outputs(m.odd, ("gate_proj", "up_proj"), torch.randn(16, 384).to(torch.bfloat16))
+    assert calls == [256, 256] and og.shape == ou.shape == (16, 256)
+    g5, u5 = VL.shared_input_outputs(m.mlp, ("gate_proj", "up_proj"), x5)
+    assert calls == [256, 256] and torch.equal(u5, m.mlp.up_proj(x5))
     # moving the module gives it buffers of its own: it leaves the group
     m.mlp.up_proj._apply(lambda t: t.clone())
     assert m.mlp.up_proj._shared_input is None
+    del calls[:]
+    g6, u6 = VL.shared_input_outputs(m.mlp, ("gate_proj", "up_proj"), x)
+    assert calls == [256, 384] and torch.equal(g6, g2) and torch.equal(u6, u2)
     assert uninstall_verify_linears(m) == 8
 
 
@@ -427,6 +431,7 @@ def test_narrow_projections_join_a_shared_input_group(monkeypatch):
     """The 48-row gates of a linear-attention layer are kept out of the swap by the N % 32 rule,
     but join the group of the layer's input projections (behind their pad-to-16 wrappers too);
     without a group they stay what they were."""
+    import dflash_mlx_amd.verify_linear as VL
     from dflash_mlx_amd.gdn_layer import _install_exact_small_proj_hooks
 
     monkeypatch.delenv("DFLASH_VERIFY_QMM", raising=False)
@@ -456,6 +461,14 @@ def test_narrow_projections_join_a_shared_input_group(monkeypatch):
             (0, 256), (256, 384), (384, 432), (432, 480)] and inner._shared_input[1] == 3
         for n, w in want.items():
             assert torch.equal(getattr(m.linear_attn, n)(x), w)
+        group = inner._shared_input[0]
+        assert m.linear_attn._dflash_fused == (group,) and group.names == ("in_proj_qkv", "in_proj_z", "in_proj_b", "in_proj_a")
+        # behind the wrappers a block of 16 is passed through as it is: the joint launch applies
+        monkeypatch.setattr(VL, "_should_use_verify", lambda x, gs, bits, tr: True)
+        x3 = x.reshape(1, 16, 512)
+        assert group.applies(m.linear_attn, x3) and not group.applies(m.linear_attn, x3[:, :5])
+        monkeypatch.undo()
+        monkeypatch.delenv("DFLASH_VERIFY_QMM", raising=False)
     # 256 + 48 rows are not a multiple of 32: no group, and the narrow projection is left alone
     m = layer()
     del m.linear_attn.in_proj_z, m.linear_attn.in_proj_a
