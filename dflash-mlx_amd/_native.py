@@ -21,7 +21,7 @@ QMM_STATIC_SCRATCH_BYTES = 8 << 20  # DFLASH_QMM_STATIC_SCRATCH_BYTES
 QMM_CHAIN_MAX = 16                       # DFLASH_QMM_CHAIN_MAX
 QMM_CHAIN_ERROR_OFFSET = (16384 - 64 + 1) * 4  # DFLASH_QMM_CHAIN_ERROR_OFFSET
 QMM_EPILOGUE_NONE, QMM_EPILOGUE_SILU_MUL = 0, 1
-OPT_GDN_STEP_BY_STEP, OPT_SDPA_SPLITS = 0, 1  # DFLASH_OPT_*
+OPT_GDN_STEP_BY_STEP, OPT_SDPA_SPLITS, OPT_SDPA_STAGED = 0, 1, 2  # DFLASH_OPT_*
 
 
 class QmmProblem(ctypes.Structure):

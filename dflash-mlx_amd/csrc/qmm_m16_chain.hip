@@ -185,6 +185,15 @@ __device__ __forceinline__ void load16_to_lds_coherent(const void* gptr, char* l
 #ifdef DFLASH_CHAIN_STAMPS
 // Experiment builds only: per workgroup, wave 0 (a worker) and wave 8 (a loader) record the
 // constant-rate wall clock at every unit.  [block][role][slot]
+#if DFLASH_CHAIN_STAMPS == 3  // per problem only, every workgroup: [block][problem * 4 + event]
+constexpr int kStampSlots = 64;
+__device__ unsigned long long g_stamps[256][1][kStampSlots];
+#define DFLASH_STAMP(role, idx)                                                          \
+  do {                                                                                   \
+    if (lane == 0 && (role) == 12 && (idx) < kStampSlots && blockIdx.x < 256)            \
+      g_stamps[blockIdx.x][0][idx] = wall_clock64();                                     \
+  } while (0)
+#else
 constexpr int kStampSlots = 512;
 __device__ unsigned long long g_stamps[64][13][kStampSlots];
 #define DFLASH_STAMP(role, idx)                                                          \
@@ -192,6 +201,7 @@ __device__ unsigned long long g_stamps[64][13][kStampSlots];
     if (lane == 0 && (idx) < kStampSlots && blockIdx.x < 64)                             \
       g_stamps[blockIdx.x][role][idx] = wall_clock64();                                  \
   } while (0)
+#endif
 #else
 #define DFLASH_STAMP(role, idx) do {} while (0)
 #endif
@@ -986,7 +996,7 @@ int qmm_chain_launch(const dflash_qmm_problem* problems, int count, void* worksp
 #ifdef DFLASH_CHAIN_STAMPS
 extern "C" int dflash_debug_read_stamps(unsigned long long* out_host) {
   return (int)hipMemcpyFromSymbol(out_host, HIP_SYMBOL(dflash::stream::g_stamps),
-                                  sizeof(unsigned long long) * 64 * 13 * dflash::stream::kStampSlots);
+                                  sizeof(dflash::stream::g_stamps));
 }
 #endif
 

@@ -516,10 +516,13 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       Operands& cur = op[par];
       Operands& nxt = op[par ^ 1];
       asm volatile("s_barrier" ::: "memory");
-      const bool fetch = left > 1;
-      if (fetch) next_addresses();
-      consume_unit<ACT_FP16, SB_FP16, SBROW>(cur, nxt, fetch, rd_x, rd_w, rd_s, acc4, ones, mask, magic);
-      if (fetch) operands_wait(nxt, acc4[0], acc4[1], acc4[2], acc4[3]);
+      // The next unit's operands are read along the way.  After the last unit the same reads
+      // are made once more, of the unit just consumed (valid LDS, results unused): with a
+      // condition around them every tile would be a basic block of its own, and the compiler
+      // could not run one tile's unpacking under another tile's matrix instructions.
+      if (left > 1) next_addresses();
+      consume_unit<ACT_FP16, SB_FP16, SBROW>(cur, nxt, true, rd_x, rd_w, rd_s, acc4, ones, mask, magic);
+      operands_wait(nxt, acc4[0], acc4[1], acc4[2], acc4[3]);
       --left;
       ++in_rb;
       if (--rb_left == 0 || left == 0) {

@@ -61,10 +61,12 @@ const char* dflash_last_error(void);
  *                                where the block kernel would apply
  *   DFLASH_OPT_SDPA_SPLITS       n > 0: dflash_sdpa_q16 (and its workspace size) cut the keys into
  *                                n ranges (fewer if a range would fall below one tile)
+ *   DFLASH_OPT_SDPA_STAGED       1: dflash_sdpa_q16 without a mask keeps the kernel that stages its
+ *                                tiles through registers (the one a mask always takes)
  * dflash_set_option returns 0, or DFLASH_ERR_ARG for an unknown option or a negative value;
  * dflash_get_option returns the value, or DFLASH_ERR_ARG.
  */
-enum { DFLASH_OPT_GDN_STEP_BY_STEP = 0, DFLASH_OPT_SDPA_SPLITS = 1, DFLASH_OPT_COUNT = 2 };
+enum { DFLASH_OPT_GDN_STEP_BY_STEP = 0, DFLASH_OPT_SDPA_SPLITS = 1, DFLASH_OPT_SDPA_STAGED = 2, DFLASH_OPT_COUNT = 3 };
 int dflash_set_option(int option, int value);
 int dflash_get_option(int option);
 
