@@ -286,6 +286,16 @@ __global__ __launch_bounds__(kThreads) void qmm_m16_gather_kernel(
       count += __popcll(m);
     }
     if (lane == 0) n_rows = count;
+  } else if (e == 0) {
+    // A row whose expert id is outside [0, E) belongs to no expert: its output is zero (the
+    // workgroups of expert 0 write it, each for its columns, so that no row of y is left as
+    // it was found).
+    for (int pidx = (int)threadIdx.x - 64; pidx < P; pidx += kThreads - 64) {
+      const int id = expert_ids[pidx];
+      if (id < 0 || id >= (int)gridDim.y) {
+        for (int n = n0; n < n0 + 16 * NT && n < N; ++n) y[(size_t)pidx * N + n] = 0;
+      }
+    }
   }
   __syncthreads();
   const int count = n_rows;

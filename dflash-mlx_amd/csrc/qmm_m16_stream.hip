@@ -198,6 +198,11 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
     }
     __syncthreads();
     units = (int)*t_total * RB * p.stages;
+    // A row whose expert id is outside [0, E) belongs to no entry: its output is zero (written
+    // here, by the first workgroup, so that no row of y is left as it was found).
+    if (blockIdx.x == 0 && tid < p.P && my_e < 0) {
+      for (int n = 0; n < p.N; ++n) p.y[(size_t)tid * p.N + n] = 0;
+    }
   }
 
   // Workgroups beyond the number of units leave; the others divide the units among

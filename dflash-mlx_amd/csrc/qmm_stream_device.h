@@ -194,30 +194,13 @@ __device__ __forceinline__ void consume_unit(const Operands& cur, Operands& nxt,
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     f32x4_t c = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#if defined(DFLASH_X_NOUNPACK)  // (timing experiments; results are wrong)
-    c = A::mfma(a0, make_uint4(cur.wq[j].x, cur.wq[j].x, cur.wq[j].x, cur.wq[j].x), c);
-    c = A::mfma(a1, make_uint4(cur.wq[j].y, cur.wq[j].y, cur.wq[j].y, cur.wq[j].y), c);
-#elif defined(DFLASH_X_NOMFMA)
-    {
-      const uint4 u0 = unpack_codes(cur.wq[j].x, mask, magic), u1 = unpack_codes(cur.wq[j].y, mask, magic);
-      c[0] = __builtin_bit_cast(float, u0.x ^ u1.x ^ a0.x); c[1] = __builtin_bit_cast(float, u0.y ^ u1.y ^ a1.x);
-      c[2] = __builtin_bit_cast(float, u0.z ^ u1.z); c[3] = __builtin_bit_cast(float, u0.w ^ u1.w);
-    }
-#else
     c = A::mfma(a0, unpack_codes(cur.wq[j].x, mask, magic), c);
     c = A::mfma(a1, unpack_codes(cur.wq[j].y, mask, magic), c);
-#endif
-#if defined(DFLASH_X_NOFMA)
-    (void)xs;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) acc[j][r] += c[r];
-#else
     const float s = SB::to_f32(cur.sv[j]);
     const float b = SB::to_f32(cur.bv[j]);
     const float bb = __builtin_fmaf(-A::kOffset, s, b);
 #pragma unroll
     for (int r = 0; r < 4; ++r) acc[j][r] = __builtin_fmaf(bb, xs[r], __builtin_fmaf(s, c[r], acc[j][r]));
-#endif
     if (fetch) {
       if (j == 0) operands_issue_piece<1, SBROW>(xaddr, waddr, saddr, nxt, acc[0]);
       if (j == 1) operands_issue_piece<2, SBROW>(xaddr, waddr, saddr, nxt, acc[1]);

@@ -214,7 +214,7 @@ int dflash_qmm_m16_packed(const void* x, const void* codes, const void* scales, 
  *                           dense form.  Without one, or for other shapes, one workgroup per
  *                           (32 columns, expert) reads its weights directly.
  * Requirements: P <= 2048, group_size in {32,64,128}, N % 16 == 0, K % group_size == 0.
- * Rows whose expert id is outside [0, E) are left unwritten.  Deterministic.
+ * Rows whose expert id is outside [0, E) give zeros.  Deterministic.
  */
 size_t dflash_qmm_m16_gather_workspace_bytes(int P, int K, int N, int E, int group_size);
 
