@@ -207,10 +207,35 @@ def replay_launch(tape: torch.Tensor, k: torch.Tensor, g: torch.Tensor, state_in
 
 
 def tape_replay_kernel(tape: torch.Tensor, k: torch.Tensor, g: torch.Tensor, state: torch.Tensor,
-                       mask: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Replay all ``tape.shape[1]`` steps onto ``state``; returns a new state tensor."""
+                       mask: Optional[torch.Tensor] = None, steps: Optional[int] = None) -> torch.Tensor:
+    """Replay all ``tape.shape[1]`` steps onto ``state``; returns a new state tensor.  ``steps``
+    (no counterpart in the reference, which slices) replays only the first ``steps`` of them:
+    the same as passing ``tape[:, :steps]``, ``k[:, :steps]``, ``g[:, :steps]`` (and the mask's
+    first ``steps`` columns), without making the three views."""
+    if steps is not None and (not state.is_cuda or steps >= tape.shape[1] or steps < 0):
+        n = max(0, min(int(steps), int(tape.shape[1])))
+        tape, k, g = tape[:, :n], k[:, :n], g[:, :n]
+        mask = None if mask is None else mask.reshape(mask.shape[0], -1)[:, :n]
+        steps = None
     if not state.is_cuda:
         return _tape_replay_ops(tape, k, g, state, mask)
+    if steps is not None:
+        # device tensors, fewer steps than rows: the rows are read in place where the kernel can
+        # stage all of them, else through the sliced form
+        bsz, rows, hk, dk = k.shape
+        hv, dv = tape.shape[2:]
+        direct = (dk >= 32 and dk % 32 == 0 and g.ndim == 3 and hv % hk == 0 and mask is None and
+                  tape.is_contiguous() and k.is_contiguous() and g.is_contiguous() and
+                  all(t.dtype in _DTYPE_CODE for t in (tape, k, g, state)) and
+                  rows * (dv + 2 * dk + 1) * 4 + dk * 4 <= 64 * 1024)
+        if not direct:
+            n = int(steps)
+            return tape_replay_kernel(tape[:, :n], k[:, :n], g[:, :n], state,
+                                      None if mask is None else mask.reshape(mask.shape[0], -1)[:, :n])
+        state_c = state.contiguous()
+        state_out = torch.empty_like(state_c)
+        replay_launch(tape, k, g, state_c, state_out, steps=int(steps), T_alloc=rows, slots=bsz)
+        return state_out
 
     bsz, steps, hk, dk = k.shape
     hv, dv = tape.shape[2:]

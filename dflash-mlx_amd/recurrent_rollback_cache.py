@@ -154,13 +154,9 @@ class RecurrentRollbackCache:
             if self._arena is not None:
                 state = self._arena._replay_layer(self._layer, self.cache[1], accepted_steps)
             else:
-                state = tape_replay_kernel(
-                    self._tape[:, :accepted_steps],
-                    self._tape_k[:, :accepted_steps],
-                    self._tape_g[:, :accepted_steps],
-                    self.cache[1],
-                    None,
-                )
+                # (the first accepted_steps rows of the three tapes, read in place)
+                state = tape_replay_kernel(self._tape, self._tape_k, self._tape_g, self.cache[1], None,
+                                           steps=accepted_steps)
             self.cache[1] = state
             self.cache[0] = self._rebuild_conv_state(accepted_steps)
 

@@ -189,10 +189,15 @@ def test_functional_form_and_prefix_slices(native_lib):
         want = _tape_replay_ops(tape[:, :a].double(), k[:, :a].double(), g[:, :a].double(), st.double())
         assert got.dtype == st.dtype and got.data_ptr() != st.data_ptr()
         assert _rel_l2(_np(got), want.cpu().numpy()) <= TOL
+        # the step count instead of the three views: the same launch, the same bits
+        assert torch.equal(tape_replay_kernel(tape, k, g, st, steps=a), got)
+    assert torch.equal(tape_replay_kernel(tape, k, g, st, steps=0), st)
+    assert torch.equal(tape_replay_kernel(tape, k, g, st, steps=99), tape_replay_kernel(tape, k, g, st))
     mask = torch.rand(3, 16, device=DEV) > 0.4
     got = tape_replay_kernel(tape, k, g, st, mask)
     want = _tape_replay_ops(tape.double(), k.double(), g.double(), st.double(), mask)
     assert _rel_l2(_np(got), want.cpu().numpy()) <= TOL
+    assert torch.equal(tape_replay_kernel(tape, k, g, st, mask, steps=7), tape_replay_kernel(tape[:, :7], k[:, :7], g[:, :7], st, mask[:, :7]))
     # Dk not a multiple of 32 takes the array-op route, as in the reference (kernels.py:374-375)
     odd = make_replay_case(1, batch=2, Hk=2, Hv=2, Dk=48, Dv=8, steps=4, T=4, seed=84).to(DEV)
     got = tape_replay_kernel(odd.tape[0], odd.k[0], odd.g[0], odd.state[0])
