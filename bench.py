@@ -204,10 +204,11 @@ def bench_qmm_chain_stack(stack: str, steps: int, warmup: int, device: str, laye
 
 
 def bench_mlp_chain(stack: str, steps: int, warmup: int, device: str):
-    """The MLP of every layer of the stack, three ways: (a) gate, up, silu * mul (array
+    """The MLP of every layer of the stack, four ways: (a) gate, up, silu * mul (array
     operators), down as four separate steps; (b) gate and up in one launch, silu * mul, down;
-    (c) one launch per layer: gate/up with the silu * mul epilogue, and down, which waits
-    inside the launch for the hidden activation while its weights already stream."""
+    (c) gate/up with the silu * mul epilogue as one chained launch of a single problem, then down
+    as a launch of its own; (d) one launch per layer: gate/up with the epilogue, and down, which
+    waits inside the launch for the hidden activation while its weights already stream."""
     import torch
 
     from dflash_mlx_amd.verify_qmm import ChainProblem, QmmChain, verify_matmul
@@ -250,6 +251,11 @@ def bench_mlp_chain(stack: str, steps: int, warmup: int, device: str):
     def chained():
         return [chain()[1] for chain in chains]
 
+    hidden_only = [QmmChain([ChainProblem(g.x, *gu, epilogue="silu_mul")]) for g, u, d, gu in mlps]
+
+    def epilogue_then_down():
+        return [verify_matmul(chain()[0], d.w, d.scales, d.biases) for chain, (g, u, d, gu) in zip(hidden_only, mlps)]
+
     res = {}
     ref = joined()
     got = chained()
@@ -262,7 +268,8 @@ def bench_mlp_chain(stack: str, steps: int, warmup: int, device: str):
     if rel > 2e-2:
         raise RuntimeError(f"chained MLP differs from the separate launches (relative {rel:.3g})")
     res["rel_diff_chained_vs_joined"] = rel
-    for name, fn in (("separate_launches", separate), ("gate_up_in_one_launch", joined), ("one_launch_per_layer", chained)):
+    for name, fn in (("separate_launches", separate), ("gate_up_in_one_launch", joined),
+                     ("gate_up_with_epilogue_then_down", epilogue_then_down), ("one_launch_per_layer", chained)):
         fn()
         graph, _ = capture(fn)
         for _ in range(warmup):

@@ -26,7 +26,8 @@ import torch
 import torch.nn as nn
 
 from .quantized import QuantizedLinear, stock_matmul
-from .verify_qmm import _should_use_verify, pack_weights, packable, verify_matmul, verify_matmul_packed
+from .verify_qmm import (ChainProblem, QmmChain, _should_use_verify, pack_weights, packable, verify_matmul,
+                         verify_matmul_packed)
 
 _VERIFY_MAX_N_DEFAULT = 100_000
 
@@ -117,6 +118,7 @@ class FusedProjections:
             self.bounds.append((row, row + n))
             row += n
         self._packed = None  # the joint matrix in the streaming kernel's order (pack_verify_linears)
+        self._silu_chain = None  # the planned launch of silu_mul(), made on first use
 
     def applies(self, parent: nn.Module, x: torch.Tensor) -> bool:
         """The joint launch gives what ``parent``'s members would give one by one: 16 rows on the
@@ -138,6 +140,28 @@ class FusedProjections:
                 return False
         return True
 
+    def silu_mul_ready(self, x: torch.Tensor) -> bool:
+        """Two members of equal height in a shape the chained kernel's epilogue covers."""
+        if len(self.bounds) != 2 or not x.is_cuda or self.bits != 4 or self.group_size != 64:
+            return False
+        rows = self.bounds[0][1]
+        k = int(self.weight.shape[1]) * 8
+        return self.bounds[1] == (rows, 2 * rows) and rows % 64 == 0 and k % 1024 == 0 and x.is_contiguous()
+
+    def silu_mul(self, x: torch.Tensor) -> torch.Tensor:
+        """``silu(x @ W_0^T) * (x @ W_1^T)`` in one launch; a new tensor per call."""
+        rows = self.bounds[0][1]
+        out = torch.empty((*x.shape[:-1], rows), dtype=x.dtype, device=x.device)
+        chain = self._silu_chain
+        if chain is None:
+            chain = QmmChain([ChainProblem(x.reshape(16, -1), self.weight, self.scales, self.biases,
+                                           epilogue="silu_mul", out=out.view(16, rows))])
+            self._silu_chain = chain
+        else:
+            chain.rebind(0, x=x.reshape(16, -1), out=out.view(16, rows))
+        chain()
+        return out
+
     def __call__(self, x: torch.Tensor) -> Tuple[torch.Tensor, ...]:
         if self._packed is not None and x.is_cuda:
             product = verify_matmul_packed(x, self._packed)
@@ -145,6 +169,26 @@ class FusedProjections:
             product = verify_matmul(x, self.weight, self.scales, self.biases, transpose=True,
                                     group_size=self.group_size, bits=self.bits)
         return tuple(product[..., lo:hi] for lo, hi in self.bounds)
+
+
+def silu_gate_up(parent: nn.Module, x: torch.Tensor, names: Tuple[str, str] = ("gate_proj", "up_proj")) -> torch.Tensor:
+    """``silu(parent.gate_proj(x)) * parent.up_proj(x)``, the hidden activation of a gated MLP.
+
+    Where ``fuse_shared_input_linears`` joined the two projections, they have the same number of
+    rows and the chained kernel covers the shape (group 64, K a multiple of 1024, rows a multiple
+    of 64), a 16-row block on the verify path takes ONE launch: the joint product with the
+    activation and the product applied before anything is stored (``dflash_qmm_m16_chain`` with
+    its silu-mul epilogue; every operator's rounding to the activation dtype is kept, the split
+    of K between workgroups differs from the separate projections', so single results may
+    differ by one rounding of the array dtype).  Everything else goes through
+    ``shared_input_outputs`` and the array operators.  No counterpart in the reference, whose MLP
+    is mlx-lm's ``down_proj(swiglu(gate_proj(x), up_proj(x)))``; 27B shape: gate/up/activation
+    48 us with ``down_proj`` against 60 us for the four separate steps."""
+    for group in getattr(parent, "_dflash_fused", ()):
+        if group.names == tuple(names) and group.applies(parent, x) and group.silu_mul_ready(x):
+            return group.silu_mul(x)
+    gate, up = shared_input_outputs(parent, names, x)
+    return torch.nn.functional.silu(gate) * up
 
 
 def shared_input_outputs(parent: nn.Module, names: Sequence[str], x: torch.Tensor) -> Tuple[torch.Tensor, ...]:

@@ -253,6 +253,31 @@ class QmmChain:
         _native.check(rc, "dflash_qmm_m16_chain")
         return self.outputs
 
+    def rebind(self, index: int, *, x: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> None:
+        """Points projection ``index`` at another input and/or output of the same shape and dtype
+        for the launches that follow (a projection that reads another one keeps doing so; outputs
+        that a later projection reads cannot be moved)."""
+        t = self._table[index]
+        x_old, w, s, b = self._keep[index]
+        if x is not None:
+            if t.wait_for >= 0:
+                raise ValueError("QmmChain.rebind: this projection reads another projection's output")
+            x2 = x.reshape(16, x.shape[-1]) if x.numel() == x_old.numel() else x
+            if tuple(x2.shape) != tuple(x_old.shape) or x2.dtype != x_old.dtype or x2.device != x_old.device \
+                    or not x2.is_contiguous():
+                raise ValueError(f"QmmChain.rebind: x must be a contiguous {tuple(x_old.shape)} tensor of {x_old.dtype}")
+            t.x = x2.data_ptr()
+            self._keep[index] = (x2, w, s, b)
+        if out is not None:
+            y_old = self.outputs[index]
+            if any(self._table[j].wait_for == index for j in range(self._count)):
+                raise ValueError("QmmChain.rebind: another projection of the chain reads this output")
+            if tuple(out.shape) != tuple(y_old.shape) or out.dtype != y_old.dtype or out.device != y_old.device \
+                    or not out.is_contiguous():
+                raise ValueError(f"QmmChain.rebind: out must be a contiguous {tuple(y_old.shape)} tensor of {y_old.dtype}")
+            t.y = out.data_ptr()
+            self.outputs[index] = out
+
     def error_word(self) -> int:
         """0, or 1 + the index of a projection whose wait for its input was given up (read back
         from the workspace of the last launch; synchronises with the device)."""

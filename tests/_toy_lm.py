@@ -6,7 +6,7 @@ import torch.nn as nn
 
 from dflash_mlx_amd import gdn_layer as G
 from dflash_mlx_amd.quantized import QuantizedLinear
-from dflash_mlx_amd.verify_linear import shared_input_outputs
+from dflash_mlx_amd.verify_linear import silu_gate_up
 
 
 def _qlinear(n_in, n_out, gen, dtype, scale=1.0):
@@ -46,8 +46,7 @@ class MLP(nn.Module):
         self.down_proj = _qlinear(inner, hidden, gen, dtype)
 
     def forward(self, x):
-        gate, up = shared_input_outputs(self, ("gate_proj", "up_proj"), x)
-        return self.down_proj(G.silu_ops(gate) * up)
+        return self.down_proj(silu_gate_up(self, x))
 
 
 class Block(nn.Module):

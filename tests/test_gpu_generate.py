@@ -153,3 +153,33 @@ def test_device_tokens_against_the_host_run_of_the_same_model(native_lib, monkey
         top = torch.topk(logits, 2)
         assert float(top.values[0] - top.values[1]) < 0.05 * float(logits.std()), (at, top.values)
         assert {int(a[at]), int(b[at])} == set(top.indices.tolist())
+
+
+def test_speculative_decoding_with_the_mlp_activation_in_the_projection_launch(native_lib, monkeypatch):
+    """hidden = 1024: gate/up of every MLP are joined and their silu * up comes out of one chained
+    launch with the epilogue (verify_linear.silu_gate_up); drafts of any quality commit the same
+    tokens, and plain decoding agrees up to near-ties."""
+    from dflash_mlx_amd import verify_qmm as VQ
+
+    monkeypatch.setenv("DFLASH_VERIFY_QMM", "1")
+    model = ToyHybridLM(seed=17, hidden=1024, Hk=2, Hv=4, D=128, dtype=torch.bfloat16).to(DEV)
+    assert install_verify_linears(model) > 0 and fuse_shared_input_linears(model) == 2 * len(model.layers)
+    model.install_hooks()
+    chained = []
+    real = VQ.QmmChain.__call__
+    monkeypatch.setattr(VQ.QmmChain, "__call__", lambda self: (chained.append(1), real(self))[1])
+    target = lambda ids, cache: model(ids, cache)
+    prompt = torch.randint(0, 384, (9,), generator=torch.Generator().manual_seed(6)).to(DEV)
+    n_new = 48
+    greedy = generate_greedy(target, _cache(model, True), prompt, n_new)
+    assert not chained                                   # one-token steps: no verify block
+    spec = generate_speculative(target, drafts(greedy.cpu(), 384, seed=3)["random"], _cache(model, True), prompt, n_new,
+                                block_tokens=16)
+    blocks = len(chained) // len(model.layers)
+    assert blocks >= n_new // 2 and len(chained) == blocks * len(model.layers)   # every MLP of every verify block
+    again = generate_speculative(target, drafts(spec.cpu(), 384, seed=3)["perfect"], _cache(model, True), prompt, n_new,
+                                 block_tokens=16)
+    torch.cuda.synchronize()
+    assert torch.equal(again, spec)
+    _same_or_parting_at_a_near_tie(model, prompt, spec, greedy, True)
+

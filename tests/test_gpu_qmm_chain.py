@@ -207,3 +207,71 @@ def test_argument_errors(native_lib):
     assert L.dflash_qmm_m16_chain(tab, 2, None, 0, 64, 0, 0, 0, None) == -3
     assert L.dflash_qmm_m16_chain_workspace_bytes(tab, 2, 64) >= 64 * 1024 + 2 * 2 * 8192
     assert L.dflash_qmm_m16_chain_workspace_bytes(tab, 2, 32) == 0
+
+
+def test_hidden_activation_of_a_gated_mlp_in_one_launch(native_lib, c_oracle, monkeypatch):
+    """verify_linear.silu_gate_up on joined gate/up projections: one chained launch with the
+    silu-mul epilogue per call, a new output tensor per call, inputs rebound per call; within
+    the north-star bar of the exact activation, and nearly everywhere the bits of the joint
+    product followed by the array operators."""
+    import dflash_mlx_amd.verify_linear as VL
+    from dflash_mlx_amd.quantized import QuantizedLinear
+
+    monkeypatch.setenv("DFLASH_VERIFY_QMM", "1")
+    K, I = 1024, 1536
+    gate, up = _cases([(K, I), (K, I)], 880)
+    for c in (gate, up):
+        c.scales.mul_(0.05); c.biases.mul_(0.05)
+    mlp = torch.nn.Module()
+    mlp.gate_proj = QuantizedLinear(gate.w.clone(), gate.scales.clone(), gate.biases.clone(), group_size=64, bits=4)
+    mlp.up_proj = QuantizedLinear(up.w.clone(), up.scales.clone(), up.biases.clone(), group_size=64, bits=4)
+    model = torch.nn.Module()
+    model.mlp = mlp
+    assert VL.install_verify_linears(model) == 2 and VL.fuse_shared_input_linears(model) == 1
+    group = model.mlp.gate_proj._shared_input[0]
+    launches = []
+    real = VQ.QmmChain.__call__
+    monkeypatch.setattr(VQ.QmmChain, "__call__", lambda self: (launches.append(self._count), real(self))[1])
+    outs = []
+    for seed in (1, 2, 3):
+        x = (torch.randn(16, K, generator=torch.Generator().manual_seed(seed)) * 0.5).to(torch.bfloat16).to(DEV)
+        assert group.silu_mul_ready(x)
+        h = VL.silu_gate_up(model.mlp, x.reshape(1, 16, K))
+        torch.cuda.synchronize()
+        assert h.shape == (1, 16, I) and all(h.data_ptr() != o.data_ptr() for o in outs)
+        outs.append(h)
+        g, u = VL.shared_input_outputs(model.mlp, ("gate_proj", "up_proj"), x)
+        ops = torch.nn.functional.silu(g) * u
+        assert float((h.reshape(16, I) != ops).float().mean()) <= 2e-3
+        ge, ue = (_exact(c_oracle, c, x).astype(np.float64) for c in (gate, up))
+        exact = ge / (1.0 + np.exp(-ge)) * ue
+        got = h.reshape(16, I).float().cpu().numpy().astype(np.float64)
+        assert np.all(np.abs(got - exact) <= 2e-2 * np.abs(exact).max(axis=1, keepdims=True))
+    assert launches == [1, 1, 1]
+    # a block that is not a verify block: array operators on the members' own outputs
+    x5 = torch.randn(5, K).to(torch.bfloat16).to(DEV)
+    assert torch.equal(VL.silu_gate_up(model.mlp, x5),
+                       torch.nn.functional.silu(model.mlp.gate_proj(x5)) * model.mlp.up_proj(x5))
+    assert launches == [1, 1, 1]
+    # rebinding is refused where it would break the chain, or where the tensor does not fit
+    small = _cases([(1024, 64), (64, 32)], 881)[0]
+    first = VQ.ChainProblem(small.x, small.w, small.scales, small.biases)
+    w2 = torch.zeros((32, 64 // 8), dtype=small.w.dtype, device=DEV)
+    with pytest.raises(ValueError):
+        VQ.QmmChain([first, VQ.ChainProblem(first, w2, small.scales[:32, :1], small.biases[:32, :1])])   # K = 64
+    two = _cases([(1024, 1024), (1024, 64)], 882)
+    a = VQ.ChainProblem(two[0].x, two[0].w, two[0].scales, two[0].biases)
+    b = VQ.ChainProblem(a, two[1].w, two[1].scales, two[1].biases)
+    chain = VQ.QmmChain([a, b])
+    with pytest.raises(ValueError, match="reads another"):
+        chain.rebind(1, x=two[1].x)
+    with pytest.raises(ValueError, match="reads this output"):
+        chain.rebind(0, out=torch.empty_like(chain.outputs[0]))
+    with pytest.raises(ValueError, match="contiguous"):
+        chain.rebind(0, x=two[0].x.float())
+    fresh = torch.empty_like(chain.outputs[1])
+    chain.rebind(0, x=two[0].x.clone())
+    chain.rebind(1, out=fresh)
+    ys = chain()
+    torch.cuda.synchronize()
+    assert ys[1] is fresh and torch.equal(fresh, _separate(_separate(two[0].x, two[0]), two[1]))

@@ -420,6 +420,26 @@ def test_fuse_shared_input_groups_keep_every_result(monkeypatch):
     assert uninstall_verify_linears(m) == 8
 
 
+def test_silu_gate_up_on_the_host_is_the_array_operators(monkeypatch):
+    """No device, or no group: the hidden activation of a gated MLP from its two projections."""
+    import dflash_mlx_amd.verify_linear as VL
+
+    monkeypatch.delenv("DFLASH_VERIFY_QMM", raising=False)
+    m = _SharedInputToy()
+    install_verify_linears(m)
+    x = torch.randn(16, 512).to(torch.bfloat16)
+    m.mlp.up_proj = VerifyQuantizedLinear.from_quantized(QuantizedLinear.from_linear(_mk_linear(512, 256), 64, 4))
+    want = torch.nn.functional.silu(m.mlp.gate_proj(x)) * m.mlp.up_proj(x)
+    assert torch.equal(VL.silu_gate_up(m.mlp, x), want)
+    assert fuse_shared_input_linears(m) >= 1
+    group = m.mlp.gate_proj._shared_input[0]
+    assert group.bounds == [(0, 256), (256, 512)] and not group.silu_mul_ready(x)      # host tensor
+    assert torch.equal(VL.silu_gate_up(m.mlp, x), want)
+    assert torch.equal(VL.silu_gate_up(m.odd, torch.ones(3, 384).to(torch.bfloat16)),
+                       torch.nn.functional.silu(m.odd.gate_proj(torch.ones(3, 384).to(torch.bfloat16))) *
+                       m.odd.up_proj(torch.ones(3, 384).to(torch.bfloat16)))
+
+
 def test_fuse_shared_input_switch(monkeypatch):
     m = _SharedInputToy()
     install_verify_linears(m)
