@@ -325,6 +325,48 @@ __device__ __forceinline__ void store4_rounded(void* p, size_t i, f32x4_t v, int
     store4_from_f32(p, i, v, dt);
   }
 }
+// ---- exact products on the 16-bit matrix cores ---------------------------------------------
+// An fp32 value is the sum of three bf16 values (its leading 8 significant bits, the next 8 of
+// what is left, and the rest: 24 bits in all, each piece cut off, not rounded, so every
+// difference is exact), and a bf16 times a bf16 is exact in fp32.  A product of an fp32 matrix
+// with a matrix whose entries are bf16 numbers can therefore run as three passes of
+// v_mfma_f32_16x16x32_bf16 (9 ns for 32 steps of the sum) instead of eight of
+// v_mfma_f32_16x16x4_f32 (16 ns for 4 steps): the same products, summed in fp32 in another order.
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+// the upper halves of a and b (a in the low half): two bf16 numbers, cut off
+__device__ __forceinline__ uint32_t upper_halves(float a, float b) {
+  return __builtin_amdgcn_perm(__float_as_uint(b), __float_as_uint(a), 0x07060302u);
+}
+__device__ __forceinline__ float below_bf16(float v) {  // v minus its leading 8 significant bits
+  return v - __uint_as_float(__float_as_uint(v) & 0xffff0000u);
+}
+template <int N>
+struct Pieces {  // three bf16 pieces of N fp32 values, packed in pairs
+  uint32_t hi[N / 2], mid[N / 2], lo[N / 2];
+};
+template <int N>
+__device__ __forceinline__ Pieces<N> split_bf16(const float (&f)[N]) {
+  Pieces<N> p;
+  float r1[N], r2[N];
+#pragma unroll
+  for (int j = 0; j < N; ++j) r1[j] = below_bf16(f[j]), r2[j] = below_bf16(r1[j]);
+#pragma unroll
+  for (int j = 0; j < N / 2; ++j) {
+    p.hi[j] = upper_halves(f[2 * j], f[2 * j + 1]);
+    p.mid[j] = upper_halves(r1[2 * j], r1[2 * j + 1]);
+    p.lo[j] = upper_halves(r2[2 * j], r2[2 * j + 1]);
+  }
+  return p;
+}
+__device__ __forceinline__ f32x4_t mfma32_bf16(const uint32_t (&a)[4], const uint32_t (&b)[4], f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, uint4{a[0], a[1], a[2], a[3]}),
+                                                 __builtin_bit_cast(bf16x8_t, uint4{b[0], b[1], b[2], b[3]}), c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4_t mfma16_bf16(const uint32_t (&a)[2], const uint32_t (&b)[2], f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, uint2{a[0], a[1]}),
+                                                   __builtin_bit_cast(s16x4_t, uint2{b[0], b[1]}), c, 0, 0, 0);
+}
+
 // What one (slot, head) item brings in from memory, as it sits in registers while in flight.
 template <bool WIDE>
 struct Incoming {
@@ -405,7 +447,9 @@ __device__ __forceinline__ float bits_as_f32(uint32_t bits, int dt) {
 }
 
 // One workgroup per (slot, head); the register cap keeps at least three on a compute unit.
-template <bool WIDE, bool NORM>
+// SPLIT: q and k are bf16 arrays; the products with S0 and the state update run on the bf16
+// matrix cores with the fp32 factor in three exact pieces (see split_bf16).
+template <bool WIDE, bool NORM, bool SPLIT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void gdn_forward_chunk_128(GdnArgs a) {
   extern __shared__ __align__(16) float smem[];
   float* sK = smem + kOffK;
@@ -473,21 +517,51 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
   f32x4_t U[2], W[2], X = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int t2 = 0; t2 < 2; ++t2) U[t2] = f32x4_t{0.f, 0.f, 0.f, 0.f}, W[t2] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  if constexpr (SPLIT) {
+    // Element j = 4h + e (h = 0, 1) of a lane's operand is column 16 (2C + h) + 4kq + e: the 32
+    // columns 32C .. 32C + 31 over the four lane groups, the same on both sides of a product.
 #pragma unroll
-  for (int c = 0; c < 8; ++c) {
-    const float4 kf4 = *reinterpret_cast<const float4*>(sK + li * kKPad + 16 * c + 4 * kq);
-    const float4 qf4 = *reinterpret_cast<const float4*>(sQ + li * kKPad + 16 * c + 4 * kq);
-    const float kf[4] = {kf4.x, kf4.y, kf4.z, kf4.w};
-    const float qf[4] = {qf4.x, qf4.y, qf4.z, qf4.w};
+    for (int C = 0; C < 4; ++C) {
+      uint32_t kb[4], qb[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+      for (int h = 0; h < 2; ++h) {
+        const float4 kf4 = *reinterpret_cast<const float4*>(sK + li * kKPad + 16 * (2 * C + h) + 4 * kq);
+        const float4 qf4 = *reinterpret_cast<const float4*>(sQ + li * kKPad + 16 * (2 * C + h) + 4 * kq);
+        kb[2 * h] = upper_halves(kf4.x, kf4.y), kb[2 * h + 1] = upper_halves(kf4.z, kf4.w);
+        qb[2 * h] = upper_halves(qf4.x, qf4.y), qb[2 * h + 1] = upper_halves(qf4.z, qf4.w);
+      }
 #pragma unroll
       for (int t2 = 0; t2 < 2; ++t2) {
-        U[t2] = mfma4(st[t2][c][e], kf[e], U[t2]);
-        W[t2] = mfma4(st[t2][c][e], qf[e], W[t2]);
+        const float f[8] = {st[t2][2 * C][0],     st[t2][2 * C][1],     st[t2][2 * C][2],     st[t2][2 * C][3],
+                            st[t2][2 * C + 1][0], st[t2][2 * C + 1][1], st[t2][2 * C + 1][2], st[t2][2 * C + 1][3]};
+        const Pieces<8> sp = split_bf16(f);
+        U[t2] = mfma32_bf16(sp.lo, kb, U[t2]);
+        W[t2] = mfma32_bf16(sp.lo, qb, W[t2]);
+        U[t2] = mfma32_bf16(sp.mid, kb, U[t2]);
+        W[t2] = mfma32_bf16(sp.mid, qb, W[t2]);
+        U[t2] = mfma32_bf16(sp.hi, kb, U[t2]);
+        W[t2] = mfma32_bf16(sp.hi, qb, W[t2]);
       }
-      if (wave == 1) X = mfma4(kf[e], kf[e], X);  // [s][t] = k_s . k_t
-      if (wave == 2) X = mfma4(kf[e], qf[e], X);  // [s][t] = k_s . q_t
+      if (wave == 1) X = mfma32_bf16(kb, kb, X);  // [s][t] = k_s . k_t
+      if (wave == 2) X = mfma32_bf16(kb, qb, X);  // [s][t] = k_s . q_t
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const float4 kf4 = *reinterpret_cast<const float4*>(sK + li * kKPad + 16 * c + 4 * kq);
+      const float4 qf4 = *reinterpret_cast<const float4*>(sQ + li * kKPad + 16 * c + 4 * kq);
+      const float kf[4] = {kf4.x, kf4.y, kf4.z, kf4.w};
+      const float qf[4] = {qf4.x, qf4.y, qf4.z, qf4.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+          U[t2] = mfma4(st[t2][c][e], kf[e], U[t2]);
+          W[t2] = mfma4(st[t2][c][e], qf[e], W[t2]);
+        }
+        if (wave == 1) X = mfma4(kf[e], kf[e], X);  // [s][t] = k_s . k_t
+        if (wave == 2) X = mfma4(kf[e], qf[e], X);  // [s][t] = k_s . q_t
+      }
     }
   }
   {
@@ -601,16 +675,28 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
       dA[0][j] *= cf;
       dA[1][j] *= cf;
     }
+    Pieces<4> dp[2];  // SPLIT: the scaled Delta in pieces; element j of a lane's operand is step 4j + kq
+    if constexpr (SPLIT) {
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2) dp[t2] = split_bf16(dA[t2]);
+    }
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
       float kA[4];  // K[s = 4j + kq][16c + li]
 #pragma unroll
       for (int j = 0; j < 4; ++j) kA[j] = sK[(4 * j + kq) * kKPad + 16 * c + li];
+      const uint32_t ka[2] = {upper_halves(kA[0], kA[1]), upper_halves(kA[2], kA[3])};
 #pragma unroll
       for (int t2 = 0; t2 < 2; ++t2) {
         f32x4_t acc = st[t2][c] * cT;
+        if constexpr (SPLIT) {
+          acc = mfma16_bf16(ka, dp[t2].lo, acc);
+          acc = mfma16_bf16(ka, dp[t2].mid, acc);
+          acc = mfma16_bf16(ka, dp[t2].hi, acc);
+        } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc = mfma4(kA[j], dA[t2][j], acc);
+          for (int j = 0; j < 4; ++j) acc = mfma4(kA[j], dA[t2][j], acc);
+        }
         st[t2][c] = acc;
       }
     }
@@ -771,13 +857,16 @@ int gdn_forward_launch(const char* who, const void* q, const void* k, const void
   if (chunk) {
     const size_t lds = kChunkLdsFloats * sizeof(float);
     const bool wide = in_dtype == DFLASH_FP32;
+    const bool split = in_dtype == DFLASH_BF16;  // q and k are bf16 numbers: exact products on the bf16 matrix cores
     if (z) {
-      if (wide) hipLaunchKernelGGL((gdn_forward_chunk_128<true, true>), grid, block, lds, s, a);
-      else hipLaunchKernelGGL((gdn_forward_chunk_128<false, true>), grid, block, lds, s, a);
+      if (wide) hipLaunchKernelGGL((gdn_forward_chunk_128<true, true, false>), grid, block, lds, s, a);
+      else if (split) hipLaunchKernelGGL((gdn_forward_chunk_128<false, true, true>), grid, block, lds, s, a);
+      else hipLaunchKernelGGL((gdn_forward_chunk_128<false, true, false>), grid, block, lds, s, a);
       norm_done = true;
     } else {
-      if (wide) hipLaunchKernelGGL((gdn_forward_chunk_128<true, false>), grid, block, lds, s, a);
-      else hipLaunchKernelGGL((gdn_forward_chunk_128<false, false>), grid, block, lds, s, a);
+      if (wide) hipLaunchKernelGGL((gdn_forward_chunk_128<true, false, false>), grid, block, lds, s, a);
+      else if (split) hipLaunchKernelGGL((gdn_forward_chunk_128<false, false, true>), grid, block, lds, s, a);
+      else hipLaunchKernelGGL((gdn_forward_chunk_128<false, false, false>), grid, block, lds, s, a);
     }
   } else if (fast) {
     if (g_per_dk) {

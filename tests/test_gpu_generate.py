@@ -180,6 +180,8 @@ def test_speculative_decoding_with_the_mlp_activation_in_the_projection_launch(n
     again = generate_speculative(target, drafts(spec.cpu(), 384, seed=3)["perfect"], _cache(model, True), prompt, n_new,
                                  block_tokens=16)
     torch.cuda.synchronize()
-    assert torch.equal(again, spec)
+    # block boundaries fall differently in the two runs: the fp32 states agree to ~1e-7, which a
+    # bf16 rounding further down may turn into the decision of a near-tie
+    _same_or_parting_at_a_near_tie(model, prompt, again, spec, True)
     _same_or_parting_at_a_near_tie(model, prompt, spec, greedy, True)
 
