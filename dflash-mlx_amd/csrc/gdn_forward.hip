@@ -274,7 +274,8 @@ __global__ __launch_bounds__(kThreads) void gdn_forward_128(GdnArgs a) {
 // s < t and Lq[t][s] = (c_t/c_s)(k_s.q_t) for s <= t:
 //     Delta = R (I + L)^-T with R[dv][t] = beta_t (v_t[dv] - c_t U[dv][t]),
 //     Y = c W + Delta Lq^T,     S_T^T = c_T S0^T + K^T diag(c_T/c_s) Delta^T.
-// Every product runs on the fp32 matrix cores (v_mfma_f32_16x16x4_f32); the only serial part
+// Every product runs on the matrix cores (v_mfma_f32_16x16x4_f32; with bf16 q and k the three
+// big ones on the bf16 matrix cores, see split_bf16); the only serial part
 // is the inverse of the T x T unit triangular matrix, once per head.  The arithmetic per
 // state element drops from ~5 T vector operations to ~1.5 T matrix-core operations, which
 // leaves the kernel bound by the state traffic.
