@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
@@ -54,6 +54,7 @@ EXPORTED_SYMBOLS = (
     "dflash_sdpa_q16_workspace_bytes",
     "dflash_sdpa_q16",
     "dflash_conv_state_rebuild",
+    "dflash_rollback_layer",
 )
 
 
@@ -119,6 +120,8 @@ def _declare(lib: ctypes.CDLL) -> None:
 
     lib.dflash_conv_state_rebuild.restype = c.c_int
     lib.dflash_conv_state_rebuild.argtypes = [c.c_void_p] * 4 + [c.c_int] * 6 + [c.c_void_p]
+    lib.dflash_rollback_layer.restype = c.c_int
+    lib.dflash_rollback_layer.argtypes = [c.c_void_p] * 9 + [c.c_int] * 16 + [c.c_void_p]
 
 
 def lib() -> ctypes.CDLL:

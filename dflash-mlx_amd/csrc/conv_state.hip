@@ -67,3 +67,17 @@ extern "C" int dflash_conv_state_rebuild(const void* conv_prev, const void* qkv,
   DFLASH_HIP_OK(hipGetLastError());
   return DFLASH_OK;
 }
+
+extern "C" int dflash_rollback_layer(const void* tape, const void* k, const void* g, const void* state_in,
+                                     void* state_out, const void* conv_prev, const void* qkv, void* conv_out,
+                                     const int32_t* steps_dev, int steps_host, int slots, int T, int Hk,
+                                     int Hv, int Dk, int Dv, int state_dtype, int tape_dtype, int k_dtype,
+                                     int g_dtype, int g_per_dk, int exact_order, int keep, int C,
+                                     int qkv_elem_bytes, void* stream) {
+  const int rc = dflash_tape_replay(tape, k, g, state_in, state_out, steps_dev, steps_host, nullptr, slots, T, Hk,
+                                    Hv, Dk, Dv, state_dtype, tape_dtype, k_dtype, g_dtype, g_per_dk, exact_order,
+                                    stream);
+  if (rc != DFLASH_OK || qkv == nullptr || keep <= 0) return rc;
+  return dflash_conv_state_rebuild(conv_prev, qkv, conv_out, steps_dev, steps_host, slots, T, keep, C,
+                                   qkv_elem_bytes, stream);
+}

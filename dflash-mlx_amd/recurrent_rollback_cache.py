@@ -22,7 +22,7 @@ from typing import Any, List, Optional, Union
 import torch
 
 from . import _native
-from .kernels import replay_launch, tape_replay_kernel
+from .kernels import _DTYPE_CODE, _exact_order, replay_launch, tape_replay_kernel
 
 
 def conv_state_rebuild(conv_prev: Optional[torch.Tensor], qkv: torch.Tensor,
@@ -142,6 +142,42 @@ class RecurrentRollbackCache:
         end = min(start + keep, int(conv_input.shape[1]))
         return conv_input[:, start:end, :].contiguous()
 
+    def _rollback_in_one_call(self, accepted_steps: int) -> bool:
+        """Replay and conv-window rebuild of this layer through one library call
+        (``dflash_rollback_layer``): the common case of device tensors as ``record_tape`` keeps
+        them.  False (nothing done) for anything else, which takes the two wrappers below."""
+        tape, k, g, qkv, state = self._tape, self._tape_k, self._tape_g, self._tape_qkv, self.cache[1]
+        keep = self.conv_kernel_size - 1
+        if qkv is None or keep <= 0 or not (state.is_cuda and qkv.is_cuda) or tape.ndim != 4 or g.ndim != 3:
+            return False
+        bsz, rows, hv, dv = tape.shape
+        hk, dk = k.shape[2], k.shape[3]
+        if not (0 <= accepted_steps <= rows == qkv.shape[1] and k.shape[1] == rows and g.shape[1] == rows
+                and dk >= 32 and dk % 32 == 0 and hv % hk == 0 and state.shape == (bsz, hv, dv, dk)
+                and rows * (dv + 2 * dk + 1) * 4 + dk * 4 <= 64 * 1024
+                and state.is_contiguous() and qkv.is_contiguous()):
+            return False
+        codes = _DTYPE_CODE
+        if tape.dtype not in codes or k.dtype not in codes or g.dtype not in codes or state.dtype not in codes:
+            return False
+        prev = self._snapshot[0]
+        prev_ptr = None
+        if prev is not None:
+            if not (prev.is_cuda and prev.is_contiguous() and prev.dtype == qkv.dtype
+                    and prev.shape == (bsz, keep, qkv.shape[2])):
+                return False
+            prev_ptr = prev.data_ptr()
+        state_out = torch.empty_like(state)
+        conv_out = torch.empty((bsz, keep, qkv.shape[2]), dtype=qkv.dtype, device=qkv.device)
+        rc = _native.lib().dflash_rollback_layer(
+            tape.data_ptr(), k.data_ptr(), g.data_ptr(), state.data_ptr(), state_out.data_ptr(), prev_ptr,
+            qkv.data_ptr(), conv_out.data_ptr(), None, accepted_steps, bsz, rows, hk, hv, dk, dv,
+            codes[state.dtype], codes[tape.dtype], codes[k.dtype], codes[g.dtype], 0,
+            1 if _exact_order() else 0, keep, qkv.shape[2], qkv.element_size(), _native.raw_stream(state.device))
+        _native.check(rc, "dflash_rollback_layer")
+        self.cache[1], self.cache[0] = state_out, conv_out
+        return True
+
     def rollback(self, n_accepted: int) -> None:
         if self._snapshot is None:
             self.clear_transients()
@@ -151,6 +187,9 @@ class RecurrentRollbackCache:
         if (self._tape is not None and self._tape_k is not None and self._tape_g is not None
                 and self.cache[1] is not None):
             accepted_steps = int(n_accepted) + 1
+            if self._arena is None and self._rollback_in_one_call(accepted_steps):
+                self.clear_transients()
+                return
             if self._arena is not None:
                 state = self._arena._replay_layer(self._layer, self.cache[1], accepted_steps)
             else:

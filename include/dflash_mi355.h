@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 11
+#define DFLASH_ABI_VERSION 12
 
 enum {
   DFLASH_OK = 0,
@@ -367,6 +367,21 @@ int dflash_sdpa_q16(const void* q, const void* k, const void* v, const void* mas
 int dflash_conv_state_rebuild(const void* conv_prev, const void* qkv, void* conv_out,
                               const int32_t* steps_dev, int steps_host, int slots, int T, int keep,
                               int C, int elem_bytes, void* stream);
+
+/*
+ * Rollback of one GatedDeltaNet layer in one call: dflash_tape_replay (no mask) followed by
+ * dflash_conv_state_rebuild on the same stream - what `RecurrentRollbackCache.rollback`
+ * (dflash_mlx/recurrent_rollback_cache.py:149-171) does with its snapshot, its three tapes and
+ * the recorded qkv rows.  Operands, dtypes and requirements as for the two calls; qkv NULL (or
+ * keep == 0) skips the conv window.  Saves a caller that rolls back layer by layer one trip
+ * through its foreign-function interface per layer.
+ */
+int dflash_rollback_layer(const void* tape, const void* k, const void* g, const void* state_in,
+                          void* state_out, const void* conv_prev, const void* qkv, void* conv_out,
+                          const int32_t* steps_dev, int steps_host, int slots, int T, int Hk,
+                          int Hv, int Dk, int Dv, int state_dtype, int tape_dtype, int k_dtype,
+                          int g_dtype, int g_per_dk, int exact_order, int keep, int C,
+                          int qkv_elem_bytes, void* stream);
 
 #ifdef __cplusplus
 }

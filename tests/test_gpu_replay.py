@@ -253,6 +253,58 @@ def test_rollback_cache_on_device_matches_oracle_model(native_lib):
         assert cache._snapshot is None and cache._tape is None and not cache._armed
 
 
+@pytest.mark.parametrize("batch,with_window", [(1, True), (3, True), (2, False)])
+def test_rollback_in_one_library_call_equals_the_two_wrappers(native_lib, monkeypatch, batch, with_window):
+    """``rollback`` of a cache outside an arena makes one ``dflash_rollback_layer`` call; with that
+    path switched off it goes through ``tape_replay_kernel`` and ``conv_state_rebuild``.  Same
+    state and conv window bit for bit, for every accepted length, several batch rows and a cache
+    that had no conv window when it was armed."""
+    case, qkv, conv0 = _gdn_cycle_inputs(91, L=1, B=batch)
+    used = []
+    real = RecurrentRollbackCache._rollback_in_one_call
+
+    def run(acc, one_call):
+        cache = RecurrentRollbackCache(size=2, conv_kernel_size=4)
+        cache[0], cache[1] = (conv0[0].to(DEV) if with_window else None), case.state[0].to(DEV)
+        cache.arm_rollback(prefix_len=7)
+        cache.record_tape(tape=case.tape[0].to(DEV), k=case.k[0].to(DEV), g=case.g[0].to(DEV), qkv=qkv[0].to(DEV))
+        monkeypatch.setattr(RecurrentRollbackCache, "_rollback_in_one_call",
+                            (lambda self, n: used.append(n) or real(self, n)) if one_call else (lambda self, n: False))
+        cache.rollback(acc)
+        torch.cuda.synchronize()
+        return cache[0], cache[1]
+
+    for acc in (0, 1, 6, 14, 15):
+        used.clear()
+        conv_a, state_a = run(acc, True)
+        assert used == [acc + 1]
+        conv_b, state_b = run(acc, False)
+        assert torch.equal(state_a, state_b) and torch.equal(conv_a, conv_b)
+        assert state_a.data_ptr() != state_b.data_ptr()
+
+
+def test_rollback_outside_the_one_call_case_takes_the_wrappers(native_lib):
+    """Per-element gates are not what the one-call path takes: it declines, and the result is
+    the oracle model's all the same."""
+    case = make_replay_case(1, batch=1, T=8, Hk=2, Hv=4, Dk=128, Dv=128, steps=8, seed=93, g_per_dk=True)
+    g = torch.Generator().manual_seed(94)
+    qkv = torch.randn((1, 8, 64), generator=g).to(torch.bfloat16)
+    conv0 = torch.randn((1, 3, 64), generator=g).to(torch.bfloat16)
+    model = O.RollbackCacheModel()
+    model.cache = [conv0.float().numpy(), _np(case.state[0]).astype(np.float64)]
+    cache = RecurrentRollbackCache(size=2, conv_kernel_size=4)
+    cache[0], cache[1] = conv0.to(DEV), case.state[0].to(DEV)
+    model.arm_rollback(); cache.arm_rollback()
+    model.record_tape(tape=_np(case.tape[0]).astype(np.float64), k=_np(case.k[0]).astype(np.float64),
+                      g=_np(case.g[0]).astype(np.float64), qkv=qkv.float().numpy())
+    cache.record_tape(tape=case.tape[0].to(DEV), k=case.k[0].to(DEV), g=case.g[0].to(DEV), qkv=qkv.to(DEV))
+    assert cache._rollback_in_one_call(4) is False and cache._tape is not None
+    model.rollback(3); cache.rollback(3)
+    torch.cuda.synchronize()
+    assert _rel_l2(_np(cache[1]), model.cache[1]) <= TOL
+    assert np.array_equal(cache[0].cpu().float().numpy(), model.cache[0])
+
+
 def test_arena_batched_rollback_equals_per_layer(native_lib):
     L, B, T, Hk, Hv, Dk, Dv, C = 4, 1, 16, 4, 8, 128, 128, 96
     case, qkv, conv0 = _gdn_cycle_inputs(91, L=L, C=C)
