@@ -435,8 +435,8 @@ def bench_replay(device: str, steps: int, warmup: int, tape_dtype: str = "bfloat
 
 def bench_rollback_per_layer(device: str, steps: int, warmup: int, tape_dtype: str = "float32"):
     """The same rollback as the engine makes it without an arena: 48 ``RecurrentRollbackCache``
-    objects, each armed, handed its tape and rolled back on its own (one replay launch and one
-    conv-state rebuild per layer; dflash_mlx/recurrent_rollback_cache.py:149-171).  Arming and
+    objects, each armed, handed its tape and rolled back on its own (one launch per layer: the
+    replay with the conv-state rebuild riding along; dflash_mlx/recurrent_rollback_cache.py:149-171).  Arming and
     recording are reference bookkeeping (no device work) and are left out of the timed region."""
     import torch
 
@@ -476,7 +476,7 @@ def bench_rollback_per_layer(device: str, steps: int, warmup: int, tape_dtype: s
         wall_us += (time.perf_counter() - t0) * 1e6
         ev_us += start.elapsed_time(stop) * 1e3
     total = replay_algorithmic_bytes(D, D, T, tape_bytes=dt.itemsize) * L * H
-    return dict(tape_dtype=tape_dtype, launches_per_rollback=2 * L, us_per_rollback=ev_us / n,
+    return dict(tape_dtype=tape_dtype, launches_per_rollback=L, us_per_rollback=ev_us / n,
                 us_per_layer=ev_us / n / L, host_us_per_rollback=wall_us / n,
                 frac_hbm=total / (ev_us / n * 1e-6) / HBM_PEAK, bytes=total)
 

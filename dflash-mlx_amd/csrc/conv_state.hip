@@ -19,24 +19,7 @@ __global__ __launch_bounds__(256) void conv_rebuild_kernel(
     const char* __restrict__ prev, const char* __restrict__ qkv, char* __restrict__ out,
     const int32_t* __restrict__ steps_dev, int steps_host, int T, int keep, size_t row_bytes) {
   const int slot = blockIdx.x / keep, j = blockIdx.x % keep;
-  int steps = steps_dev ? steps_dev[slot] : steps_host;
-  steps = steps < 0 ? 0 : (steps > T ? T : steps);
-  const int src = steps + j;  // row of concat([prev, qkv]); always < keep + T
-  const V* from = nullptr;
-  if (src >= keep) {
-    from = reinterpret_cast<const V*>(qkv + ((size_t)slot * T + (src - keep)) * row_bytes);
-  } else if (prev != nullptr) {
-    from = reinterpret_cast<const V*>(prev + ((size_t)slot * keep + src) * row_bytes);
-  }
-  V* to = reinterpret_cast<V*>(out + ((size_t)slot * keep + j) * row_bytes);
-  const size_t n = row_bytes / sizeof(V);
-  if (from != nullptr) {
-    for (size_t i = threadIdx.x; i < n; i += blockDim.x) to[i] = from[i];
-  } else {
-    V zero;
-    __builtin_memset(&zero, 0, sizeof(V));
-    for (size_t i = threadIdx.x; i < n; i += blockDim.x) to[i] = zero;
-  }
+  conv_rebuild_row<V>(prev, qkv, out, steps_dev ? steps_dev[slot] : steps_host, T, keep, row_bytes, slot, j);
 }
 
 }  // namespace
@@ -66,18 +49,4 @@ extern "C" int dflash_conv_state_rebuild(const void* conv_prev, const void* qkv,
   }
   DFLASH_HIP_OK(hipGetLastError());
   return DFLASH_OK;
-}
-
-extern "C" int dflash_rollback_layer(const void* tape, const void* k, const void* g, const void* state_in,
-                                     void* state_out, const void* conv_prev, const void* qkv, void* conv_out,
-                                     const int32_t* steps_dev, int steps_host, int slots, int T, int Hk,
-                                     int Hv, int Dk, int Dv, int state_dtype, int tape_dtype, int k_dtype,
-                                     int g_dtype, int g_per_dk, int exact_order, int keep, int C,
-                                     int qkv_elem_bytes, void* stream) {
-  const int rc = dflash_tape_replay(tape, k, g, state_in, state_out, steps_dev, steps_host, nullptr, slots, T, Hk,
-                                    Hv, Dk, Dv, state_dtype, tape_dtype, k_dtype, g_dtype, g_per_dk, exact_order,
-                                    stream);
-  if (rc != DFLASH_OK || qkv == nullptr || keep <= 0) return rc;
-  return dflash_conv_state_rebuild(conv_prev, qkv, conv_out, steps_dev, steps_host, slots, T, keep, C,
-                                   qkv_elem_bytes, stream);
 }

@@ -157,4 +157,31 @@ __device__ __forceinline__ void swap_row_bit(f32x4_t& even, f32x4_t& odd) {
   }
 }
 
+// One output row of the conv-window rebuild (dflash_mlx/recurrent_rollback_cache.py:129-146):
+// row j of `slot` is row steps + j of concat([prev or zeros, qkv]), copied by a workgroup in
+// pieces of type V.  Shared by the kernel of its own and by the replay launches that carry the
+// conv window along.
+template <typename V>
+__device__ __forceinline__ void conv_rebuild_row(const char* __restrict__ prev, const char* __restrict__ qkv,
+                                                 char* __restrict__ out, int steps, int T, int keep,
+                                                 size_t row_bytes, int slot, int j) {
+  steps = steps < 0 ? 0 : (steps > T ? T : steps);
+  const int src = steps + j;  // row of concat([prev, qkv]); always < keep + T
+  const V* from = nullptr;
+  if (src >= keep) {
+    from = reinterpret_cast<const V*>(qkv + ((size_t)slot * T + (src - keep)) * row_bytes);
+  } else if (prev != nullptr) {
+    from = reinterpret_cast<const V*>(prev + ((size_t)slot * keep + src) * row_bytes);
+  }
+  V* to = reinterpret_cast<V*>(out + ((size_t)slot * keep + j) * row_bytes);
+  const size_t n = row_bytes / sizeof(V);
+  if (from != nullptr) {
+    for (size_t i = threadIdx.x; i < n; i += blockDim.x) to[i] = from[i];
+  } else {
+    V zero;
+    __builtin_memset(&zero, 0, sizeof(V));
+    for (size_t i = threadIdx.x; i < n; i += blockDim.x) to[i] = zero;
+  }
+}
+
 }  // namespace dflash

@@ -38,6 +38,13 @@ struct ReplayArgs {
   int steps_host;
   int T, Hk, Hv, Dk, Dv;
   int state_dtype, tape_dtype, k_dtype, g_dtype, g_per_dk;
+  // the conv window of the same layer, rebuilt by workgroups behind the replay's (none: conv_keep 0)
+  const char* conv_prev;
+  const char* conv_qkv;
+  char* conv_out;
+  size_t conv_row_bytes;
+  int conv_keep, conv_vec16;
+  int replay_blocks;  // slots * Hv
 };
 
 // LDS layout (floats): sA[Dv][T] (delta, t contiguous) | sK[T][Dk] | sG[T][Dk or 1] | sGt[Dk]
@@ -115,6 +122,18 @@ __device__ __forceinline__ int slot_steps(const ReplayArgs& a, int slot) {
   return n > a.T ? a.T : n;
 }
 
+// Workgroups beyond the replay's own rebuild the conv window, one output row each.  True if this
+// workgroup was one of them (and is done).
+__device__ __forceinline__ bool conv_window_workgroup(const ReplayArgs& a) {
+  if ((int)blockIdx.x < a.replay_blocks) return false;
+  const int b = (int)blockIdx.x - a.replay_blocks;
+  const int slot = b / a.conv_keep, j = b % a.conv_keep;
+  const int steps = a.steps_dev ? a.steps_dev[slot] : a.steps_host;
+  if (a.conv_vec16) conv_rebuild_row<uint4>(a.conv_prev, a.conv_qkv, a.conv_out, steps, a.T, a.conv_keep, a.conv_row_bytes, slot, j);
+  else conv_rebuild_row<unsigned char>(a.conv_prev, a.conv_qkv, a.conv_out, steps, a.T, a.conv_keep, a.conv_row_bytes, slot, j);
+  return true;
+}
+
 // ---------------------------------------------------------------------------
 // fp32 state, Dk = Dv = 128, T <= 16: the folded sweep as a rank-16 update on the matrix cores.
 //   S_out^T = diag(prod g) S_in^T + K'^T Delta,   K'[t][dk] = c_t[dk] k_t[dk]  (16 steps = 4 MFMAs
@@ -163,6 +182,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
   float* sD = sK + 16 * kPad;
   float* sG = sD + 16 * kPad;
   float* sGt = sG + (a.g_per_dk ? 16 * 128 : 16);
+  if (conv_window_workgroup(a)) return;
   const int slot = blockIdx.x / a.Hv, hv = blockIdx.x % a.Hv;
   const int n = slot_steps(a, slot);
   const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kq = lane >> 4;
@@ -311,6 +331,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
 template <bool EXACT>
 __global__ __launch_bounds__(kThreads) void replay_generic(ReplayArgs a) {
   extern __shared__ float smem[];
+  if (conv_window_workgroup(a)) return;
   const Smem s = carve(smem, a, a.T);
   const int slot = blockIdx.x / a.Hv, hv = blockIdx.x % a.Hv;
   const int n = slot_steps(a, slot);
@@ -374,13 +395,15 @@ bool valid_dtype(int dt) { return dt == DFLASH_BF16 || dt == DFLASH_FP16 || dt =
 }  // namespace
 }  // namespace dflash
 
-extern "C" int dflash_tape_replay(const void* tape, const void* k, const void* g,
-                                  const void* state_in, void* state_out, const int32_t* steps_dev,
-                                  int steps_host, const uint8_t* mask, int slots, int T, int Hk,
-                                  int Hv, int Dk, int Dv, int state_dtype, int tape_dtype,
-                                  int k_dtype, int g_dtype, int g_per_dk, int exact_order,
-                                  void* stream) {
-  using namespace dflash;
+namespace dflash {
+namespace {
+// The replay launch; with qkv != nullptr the conv window of the same slots rides along
+// (conv_prev [slots, keep, C] or NULL, qkv [slots, T, C], conv_out [slots, keep, C]).
+int replay_launch(const void* tape, const void* k, const void* g, const void* state_in, void* state_out,
+                  const int32_t* steps_dev, int steps_host, const uint8_t* mask, int slots, int T, int Hk,
+                  int Hv, int Dk, int Dv, int state_dtype, int tape_dtype, int k_dtype, int g_dtype,
+                  int g_per_dk, int exact_order, const void* conv_prev, const void* qkv, void* conv_out,
+                  int keep, int C, int qkv_elem_bytes, void* stream) {
   DFLASH_REQUIRE(state_in && state_out, DFLASH_ERR_ARG, "dflash_tape_replay: null state");
   DFLASH_REQUIRE(state_in != state_out, DFLASH_ERR_ARG,
                  "dflash_tape_replay: state_out must not alias state_in");
@@ -418,8 +441,25 @@ extern "C" int dflash_tape_replay(const void* tape, const void* k, const void* g
   a.T = T; a.Hk = Hk; a.Hv = Hv; a.Dk = Dk; a.Dv = Dv;
   a.state_dtype = state_dtype; a.tape_dtype = tape_dtype; a.k_dtype = k_dtype;
   a.g_dtype = g_dtype; a.g_per_dk = g_per_dk ? 1 : 0;
+  a.replay_blocks = slots * Hv;
+  a.conv_prev = a.conv_qkv = nullptr; a.conv_out = nullptr; a.conv_row_bytes = 0; a.conv_keep = a.conv_vec16 = 0;
+  long long conv_blocks = 0;
+  if (qkv != nullptr) {
+    DFLASH_REQUIRE(conv_out && conv_out != conv_prev, DFLASH_ERR_ARG,
+                   "dflash_rollback_layer: conv_out must be given and must not alias conv_prev");
+    DFLASH_REQUIRE(T > 0 && keep > 0 && C > 0 && qkv_elem_bytes > 0, DFLASH_ERR_SHAPE,
+                   "dflash_rollback_layer: non-positive dimension of the conv window");
+    a.conv_prev = (const char*)conv_prev; a.conv_qkv = (const char*)qkv; a.conv_out = (char*)conv_out;
+    a.conv_row_bytes = (size_t)C * qkv_elem_bytes;
+    a.conv_keep = keep;
+    a.conv_vec16 = a.conv_row_bytes % 16 == 0 && (uintptr_t)qkv % 16 == 0 && (uintptr_t)conv_out % 16 == 0 &&
+                   (uintptr_t)conv_prev % 16 == 0;
+    conv_blocks = (long long)slots * keep;
+    DFLASH_REQUIRE((long long)slots * Hv + conv_blocks < (1ll << 31), DFLASH_ERR_SHAPE,
+                   "dflash_rollback_layer: too many workgroups");
+  }
 
-  const dim3 grid((unsigned)(slots * Hv)), block(kThreads);
+  const dim3 grid((unsigned)(slots * Hv + conv_blocks)), block(kThreads);
   hipStream_t s = (hipStream_t)stream;
   if (exact) {
     hipLaunchKernelGGL(replay_generic<true>, grid, block, smem, s, a);
@@ -434,4 +474,30 @@ extern "C" int dflash_tape_replay(const void* tape, const void* k, const void* g
   }
   DFLASH_HIP_OK(hipGetLastError());
   return DFLASH_OK;
+}
+}  // namespace
+}  // namespace dflash
+
+extern "C" int dflash_tape_replay(const void* tape, const void* k, const void* g,
+                                  const void* state_in, void* state_out, const int32_t* steps_dev,
+                                  int steps_host, const uint8_t* mask, int slots, int T, int Hk,
+                                  int Hv, int Dk, int Dv, int state_dtype, int tape_dtype,
+                                  int k_dtype, int g_dtype, int g_per_dk, int exact_order,
+                                  void* stream) {
+  return dflash::replay_launch(tape, k, g, state_in, state_out, steps_dev, steps_host, mask, slots, T, Hk, Hv, Dk,
+                               Dv, state_dtype, tape_dtype, k_dtype, g_dtype, g_per_dk, exact_order, nullptr,
+                               nullptr, nullptr, 0, 0, 0, stream);
+}
+
+extern "C" int dflash_rollback_layer(const void* tape, const void* k, const void* g, const void* state_in,
+                                     void* state_out, const void* conv_prev, const void* qkv, void* conv_out,
+                                     const int32_t* steps_dev, int steps_host, int slots, int T, int Hk,
+                                     int Hv, int Dk, int Dv, int state_dtype, int tape_dtype, int k_dtype,
+                                     int g_dtype, int g_per_dk, int exact_order, int keep, int C,
+                                     int qkv_elem_bytes, void* stream) {
+  const bool window = qkv != nullptr && keep > 0;
+  return dflash::replay_launch(tape, k, g, state_in, state_out, steps_dev, steps_host, nullptr, slots, T, Hk, Hv, Dk,
+                               Dv, state_dtype, tape_dtype, k_dtype, g_dtype, g_per_dk, exact_order,
+                               window ? conv_prev : nullptr, window ? qkv : nullptr, window ? conv_out : nullptr,
+                               window ? keep : 0, window ? C : 0, window ? qkv_elem_bytes : 0, stream);
 }

@@ -170,13 +170,17 @@ def _slot_major(t: torch.Tensor, inner: int) -> tuple:
 def replay_launch(tape: torch.Tensor, k: torch.Tensor, g: torch.Tensor, state_in: torch.Tensor,
                   state_out: torch.Tensor, *, steps: Union[int, torch.Tensor], T_alloc: int,
                   mask: Optional[torch.Tensor] = None, slots: Optional[int] = None,
-                  exact_order: Optional[bool] = None) -> None:
+                  exact_order: Optional[bool] = None,
+                  conv: Optional[tuple] = None) -> None:
     """Enqueue one ``dflash_tape_replay`` on the current stream.
 
     The leading dimension(s) of every operand are flattened into ``slots``
     independent problems; ``steps`` is a host int applied to every slot or an int32
     device tensor with one entry per slot.  ``T_alloc`` is the number of step rows
-    each slot's tape/k/g storage holds (>= any step count used)."""
+    each slot's tape/k/g storage holds (>= any step count used).
+
+    ``conv = (conv_prev or None, qkv, conv_out)`` (contiguous, ``[slots.., keep | T_alloc, C]``, no
+    mask): the same launch also rebuilds the conv windows (``dflash_rollback_layer``)."""
     lib = _native.lib()
     if not state_in.is_cuda:
         raise _native.NativeLibraryError("tape replay kernel needs device tensors")
@@ -197,12 +201,27 @@ def replay_launch(tape: torch.Tensor, k: torch.Tensor, g: torch.Tensor, state_in
         mask = mask.to(torch.uint8).contiguous()
         mask_ptr = mask.data_ptr()
     stream = _native.raw_stream(state_in.device)
+    exact = 1 if (_exact_order() if exact_order is None else exact_order) else 0
+    if conv is not None:
+        conv_prev, qkv, conv_out = conv
+        if mask is not None or not (qkv.is_contiguous() and conv_out.is_contiguous()) or int(qkv.shape[-2]) != T_alloc:
+            raise ValueError("conv windows ride along only without a mask, contiguous, with the tape's row count")
+        if conv_prev is not None and not (conv_prev.is_contiguous() and conv_prev.dtype == qkv.dtype
+                                          and conv_prev.shape[-2:] == conv_out.shape[-2:]):
+            raise ValueError("conv_prev must be contiguous, [.., keep, C], in the dtype of qkv")
+        rc = lib.dflash_rollback_layer(
+            tape.data_ptr(), k.data_ptr(), g.data_ptr(), state_in.data_ptr(), state_out.data_ptr(),
+            None if conv_prev is None else conv_prev.data_ptr(), qkv.data_ptr(), conv_out.data_ptr(),
+            steps_dev, steps_host, slots, T_alloc, Hk, Hv, Dk, Dv,
+            _DTYPE_CODE[state_in.dtype], _DTYPE_CODE[tape.dtype], _DTYPE_CODE[k.dtype], _DTYPE_CODE[g.dtype],
+            g_per_dk, exact, int(conv_out.shape[-2]), int(qkv.shape[-1]), qkv.element_size(), stream)
+        _native.check(rc, "dflash_rollback_layer")
+        return
     rc = lib.dflash_tape_replay(
         tape.data_ptr(), k.data_ptr(), g.data_ptr(), state_in.data_ptr(), state_out.data_ptr(),
         steps_dev, steps_host, mask_ptr, slots, T_alloc, Hk, Hv, Dk, Dv,
         _DTYPE_CODE[state_in.dtype], _DTYPE_CODE[tape.dtype], _DTYPE_CODE[k.dtype],
-        _DTYPE_CODE[g.dtype], g_per_dk, 1 if (_exact_order() if exact_order is None else exact_order) else 0,
-        stream)
+        _DTYPE_CODE[g.dtype], g_per_dk, exact, stream)
     _native.check(rc, "dflash_tape_replay")
 
 

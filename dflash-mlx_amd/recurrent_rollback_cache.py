@@ -12,8 +12,8 @@ tape must assign a *new* tensor to ``cache[1]`` rather than update it in place.
 
 ``RollbackArena`` is the batched form for a whole model: one allocation holds the
 states (double-buffered), tapes and conv windows of all GDN layers, so that a
-rollback of every layer is a single replay launch plus a single conv-rebuild
-launch whose accepted length may live on the device.
+rollback of every layer is a single launch (replay and conv-window rebuild together)
+whose accepted length may live on the device.
 """
 from __future__ import annotations
 
@@ -356,10 +356,10 @@ class RollbackArena:
                                  f"batch row) or {self.L * self.B} (one per layer and batch row)")
             self.steps.copy_(acc)
             steps = self.steps
+        # every layer's state and conv window in one launch
         replay_launch(self.tape, self.k, self.g, self.state[snap], self.state[nxt], steps=steps,
-                      T_alloc=self.T, slots=self.L * self.B)
-        if self.keep > 0:
-            conv_state_rebuild(self.conv[snap], self.qkv, steps, self.keep, out=self.conv[nxt])
+                      T_alloc=self.T, slots=self.L * self.B,
+                      conv=(self.conv[snap], self.qkv, self.conv[nxt]) if self.keep > 0 else None)
         for layer, c in enumerate(self._caches):
             c.cache = [self.conv[nxt, layer], self.state[nxt, layer]]
             c.clear_transients()

@@ -369,12 +369,13 @@ int dflash_conv_state_rebuild(const void* conv_prev, const void* qkv, void* conv
                               int C, int elem_bytes, void* stream);
 
 /*
- * Rollback of one GatedDeltaNet layer in one call: dflash_tape_replay (no mask) followed by
- * dflash_conv_state_rebuild on the same stream - what `RecurrentRollbackCache.rollback`
- * (dflash_mlx/recurrent_rollback_cache.py:149-171) does with its snapshot, its three tapes and
- * the recorded qkv rows.  Operands, dtypes and requirements as for the two calls; qkv NULL (or
- * keep == 0) skips the conv window.  Saves a caller that rolls back layer by layer one trip
- * through its foreign-function interface per layer.
+ * Rollback of GatedDeltaNet layers in one launch: what dflash_tape_replay (no mask) and
+ * dflash_conv_state_rebuild do, by one kernel whose trailing workgroups copy the conv-window
+ * rows - what `RecurrentRollbackCache.rollback` (dflash_mlx/recurrent_rollback_cache.py:149-171)
+ * does with its snapshot, its three tapes and the recorded qkv rows.  Operands, dtypes,
+ * requirements and results (bit for bit) as for the two calls, with qkv [slots, T, C] holding
+ * the same T rows per slot as the tapes; qkv NULL (or keep == 0) leaves the conv window out.
+ * One launch and one trip through the caller's foreign-function interface per rollback.
  */
 int dflash_rollback_layer(const void* tape, const void* k, const void* g, const void* state_in,
                           void* state_out, const void* conv_prev, const void* qkv, void* conv_out,
