@@ -148,14 +148,19 @@ class RecurrentRollbackCache:
         them.  False (nothing done) for anything else, which takes the two wrappers below."""
         tape, k, g, qkv, state = self._tape, self._tape_k, self._tape_g, self._tape_qkv, self.cache[1]
         keep = self.conv_kernel_size - 1
-        if qkv is None or keep <= 0 or not (state.is_cuda and qkv.is_cuda) or tape.ndim != 4 or g.ndim != 3:
+        if (qkv is None or keep <= 0 or not (state.is_cuda and qkv.is_cuda) or tape.ndim != 4 or k.ndim != 4
+                or g.ndim != 3 or qkv.ndim != 3):
             return False
         bsz, rows, hv, dv = tape.shape
         hk, dk = k.shape[2], k.shape[3]
-        if not (0 <= accepted_steps <= rows == qkv.shape[1] and k.shape[1] == rows and g.shape[1] == rows
-                and dk >= 32 and dk % 32 == 0 and hv % hk == 0 and state.shape == (bsz, hv, dv, dk)
+        # every extent the kernel indexes with is checked here: it reads what these numbers say
+        if not (0 <= accepted_steps <= rows and k.shape[:2] == (bsz, rows) and g.shape == (bsz, rows, hv)
+                and qkv.shape[:2] == (bsz, rows) and state.shape == (bsz, hv, dv, dk)
+                and dk >= 32 and dk % 32 == 0 and hv % hk == 0
                 and rows * (dv + 2 * dk + 1) * 4 + dk * 4 <= 64 * 1024
-                and state.is_contiguous() and qkv.is_contiguous()):
+                and state.is_contiguous() and qkv.is_contiguous() and tape.is_contiguous()
+                and k.is_contiguous() and g.is_contiguous()
+                and tape.device == k.device == g.device == qkv.device == state.device):
             return False
         codes = _DTYPE_CODE
         if tape.dtype not in codes or k.dtype not in codes or g.dtype not in codes or state.dtype not in codes:
@@ -163,7 +168,7 @@ class RecurrentRollbackCache:
         prev = self._snapshot[0]
         prev_ptr = None
         if prev is not None:
-            if not (prev.is_cuda and prev.is_contiguous() and prev.dtype == qkv.dtype
+            if not (prev.device == qkv.device and prev.is_contiguous() and prev.dtype == qkv.dtype
                     and prev.shape == (bsz, keep, qkv.shape[2])):
                 return False
             prev_ptr = prev.data_ptr()
