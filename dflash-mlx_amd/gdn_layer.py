@@ -116,6 +116,17 @@ def gdn_prepare(qkv: torch.Tensor, conv_state: Optional[torch.Tensor], conv_w: t
                                Hk=Hk, Hv=Hv, Dk=Dk, Dv=Dv, eps=eps)
     lib = _native.lib()
     dev, dt = qkv.device, qkv.dtype
+    # the kernel indexes with B, S, C, K and the head counts: every operand must have the extents
+    # that follow from them, on qkv's device
+    expect = dict(a=(a, (B, S, Hv)), b=(b, (B, S, Hv)), A_log=(A_log, (Hv,)), dt_bias=(dt_bias, (Hv,)),
+                  conv_w=(conv_w, (C, K)))
+    if conv_state is not None:
+        expect["conv_state"] = (conv_state, (B, K - 1, C))
+    for name, (t, shape) in expect.items():
+        if tuple(t.shape) != shape or t.device != dev:
+            raise ValueError(f"gdn_prepare: {name} must be {list(shape)} on {dev}, got {list(t.shape)} on {t.device}")
+    if mask is not None and (mask.numel() != B * S or mask.device != dev):
+        raise ValueError(f"gdn_prepare: mask must hold {B} x {S} entries on {dev}")
     qkv_c, w_c, a_c, b_c = qkv.contiguous(), conv_w.contiguous(), a.contiguous(), b.contiguous()
     cs = None if conv_state is None else conv_state.contiguous()
     mask_c = None if mask is None else mask.to(torch.uint8).contiguous()
@@ -138,7 +149,8 @@ def gdn_prepare(qkv: torch.Tensor, conv_state: Optional[torch.Tensor], conv_w: t
 def gated_norm(x: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
     """silu(z) * rms_norm(x, weight, eps) over the last axis."""
     D = int(x.shape[-1])
-    if not (_kernel_covers(x, D) and z.dtype == x.dtype and z.shape == x.shape and weight.dtype in _DTYPE_CODE):
+    if not (_kernel_covers(x, D) and z.dtype == x.dtype and z.shape == x.shape and weight.dtype in _DTYPE_CODE
+            and tuple(weight.shape) == (D,) and z.device == x.device == weight.device):
         return gated_norm_ops(x, z, weight, eps)
     lib = _native.lib()
     x_c, z_c, w_c = x.contiguous(), z.contiguous(), weight.contiguous()

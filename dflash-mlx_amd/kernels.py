@@ -22,6 +22,15 @@ from . import _native
 _DTYPE_CODE = {torch.bfloat16: _native.BF16, torch.float16: _native.FP16, torch.float32: _native.FP32}
 
 
+def _require_extents(who: str, device: torch.device, **operands) -> None:
+    """``name=(tensor, shape)`` pairs: the kernels index with the extents the caller derived from
+    one operand, so every other operand must have exactly the extents that follow from them, and
+    live on the same device.  Anything else is an error here instead of a stray access there."""
+    for name, (t, shape) in operands.items():
+        if tuple(t.shape) != tuple(shape) or t.device != device:
+            raise ValueError(f"{who}: {name} must be {list(shape)} on {device}, got {list(t.shape)} on {t.device}")
+
+
 def _expand_heads(x: torch.Tensor, hv: int, what: str) -> torch.Tensor:
     hk = int(x.shape[2])
     if hv % hk != 0:
@@ -82,7 +91,8 @@ def fused_output_norm_applies(q: torch.Tensor, v: torch.Tensor, state: torch.Ten
     """Whether ``gated_delta_kernel_with_tape(..., output_norm=...)`` can be asked for: device
     tensors of the kernels' dtypes, z shaped like v, rows of a multiple of 64 up to 256."""
     dv = int(v.shape[-1])
-    return (state.is_cuda and z.shape == v.shape and z.dtype == q.dtype == v.dtype and weight.dtype in _DTYPE_CODE and
+    return (state.is_cuda and z.shape == v.shape and z.device == weight.device == state.device and
+            z.dtype == q.dtype == v.dtype and weight.dtype in _DTYPE_CODE and
             q.dtype in _DTYPE_CODE and int(weight.numel()) == dv and dv % 64 == 0 and dv <= 256 and
             int(q.shape[-1]) >= 32 and int(q.shape[-1]) % 32 == 0 and int(q.shape[1]) > 0)
 
@@ -112,6 +122,11 @@ def gated_delta_kernel_with_tape(q: torch.Tensor, k: torch.Tensor, v: torch.Tens
     if not state.is_cuda or dk < 32 or dk % 32 != 0 or not dtypes_ok or T == 0:
         return _gated_delta_ops_with_tape(q, k, v, g, beta, state, mask)
     lib = _native.lib()
+    _require_extents("gated_delta_kernel_with_tape", state.device, q=(q, (B, T, hk, dk)), k=(k, (B, T, hk, dk)),
+                     v=(v, (B, T, hv, dv)), g=(g, (B, T, hv) + ((dk,) if g.ndim == 4 else ())),
+                     beta=(beta, (B, T, hv)), state=(state, (B, hv, dv, dk)))
+    if mask is not None and (mask.numel() != B * T or mask.device != state.device):
+        raise ValueError(f"gated_delta_kernel_with_tape: mask must hold {B} x {T} entries on {state.device}")
     q_c, k_c, v_c, g_c, beta_c = (t.contiguous() for t in (q, k, v, g, beta))
     state_c = state.contiguous()
     y = torch.empty((B, T, hv, dv), dtype=q.dtype, device=q.device)
@@ -251,6 +266,8 @@ def tape_replay_kernel(tape: torch.Tensor, k: torch.Tensor, g: torch.Tensor, sta
             n = int(steps)
             return tape_replay_kernel(tape[:, :n], k[:, :n], g[:, :n], state,
                                       None if mask is None else mask.reshape(mask.shape[0], -1)[:, :n])
+        _require_extents("tape_replay_kernel", state.device, tape=(tape, (bsz, rows, hv, dv)), k=(k, (bsz, rows, hk, dk)),
+                         g=(g, (bsz, rows, hv)), state=(state, (bsz, hv, dv, dk)))
         state_c = state.contiguous()
         state_out = torch.empty_like(state_c)
         replay_launch(tape, k, g, state_c, state_out, steps=int(steps), T_alloc=rows, slots=bsz)
@@ -271,6 +288,10 @@ def tape_replay_kernel(tape: torch.Tensor, k: torch.Tensor, g: torch.Tensor, sta
 
     if not fits_lds(steps):
         return _tape_replay_ops(tape, k, g, state, mask)
+    _require_extents("tape_replay_kernel", state.device, tape=(tape, (bsz, steps, hv, dv)), k=(k, (bsz, steps, hk, dk)),
+                     g=(g, (bsz, steps, hv) + ((dk,) if g.ndim == 4 else ())), state=(state, (bsz, hv, dv, dk)))
+    if mask is not None and (mask.numel() != bsz * steps or mask.device != state.device):
+        raise ValueError(f"tape_replay_kernel: mask must hold {bsz} x {steps} entries on {state.device}")
 
     state_c = state.contiguous()
     tape_c, T_tape = _slot_major(tape, hv * dv)
@@ -323,7 +344,10 @@ def batched_sdpa_2pass_exact(queries: torch.Tensor, keys: torch.Tensor, values: 
         return None
     if d not in (128, 256) or d != vdim or hk <= 0 or hq % hk != 0 or hq // hk > 8 or n_kv < 16:
         return None
-    if keys.dtype != queries.dtype or values.dtype != queries.dtype or tuple(values.shape[:3]) != tuple(keys.shape[:3]):
+    if keys.dtype != queries.dtype or values.dtype != queries.dtype:
+        return None
+    if (tuple(keys.shape) != (bsz, hk, n_kv, d) or tuple(values.shape) != (bsz, hk, n_kv, d)
+            or not (keys.device == values.device == queries.device)):
         return None
 
     def in_place(t: torch.Tensor) -> torch.Tensor:
@@ -340,7 +364,7 @@ def batched_sdpa_2pass_exact(queries: torch.Tensor, keys: torch.Tensor, values: 
                                                  device=mask.device))
         else:
             mask_tensor = mask.to(queries.dtype)
-        mask_tensor = torch.broadcast_to(mask_tensor, (bsz, hq, q_len, n_kv)).contiguous()
+        mask_tensor = torch.broadcast_to(mask_tensor.to(queries.device), (bsz, hq, q_len, n_kv)).contiguous()
 
     lib = _native.lib()
     out = torch.empty_like(queries)

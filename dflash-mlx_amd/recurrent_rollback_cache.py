@@ -39,12 +39,19 @@ def conv_state_rebuild(conv_prev: Optional[torch.Tensor], qkv: torch.Tensor,
         out = torch.empty((*lead, keep, C), dtype=qkv.dtype, device=qkv.device)
     if not qkv.is_cuda:
         raise _native.NativeLibraryError("conv_state_rebuild needs device tensors")
+    if (tuple(out.shape) != (*lead, keep, C) or out.dtype != qkv.dtype or out.device != qkv.device
+            or not out.is_contiguous()):
+        raise ValueError("out must be a contiguous [.., keep, C] tensor in the dtype of qkv, on its device")
+    if isinstance(steps, torch.Tensor) and (steps.dtype != torch.int32 or steps.device != qkv.device
+                                            or steps.numel() != slots or not steps.is_contiguous()):
+        raise ValueError("steps tensor must be int32, on the device, one entry per slot")
     qkv = qkv.contiguous()
     prev_ptr = None
     if conv_prev is not None:
         conv_prev = conv_prev.contiguous()
-        if conv_prev.dtype != qkv.dtype or conv_prev.shape[-2] != keep:
-            raise ValueError("conv_prev must be [.., keep, C] in the dtype of qkv")
+        if (conv_prev.dtype != qkv.dtype or tuple(conv_prev.shape) != (*lead, keep, C)
+                or conv_prev.device != qkv.device):
+            raise ValueError("conv_prev must be [.., keep, C] in the dtype of qkv, on its device")
         prev_ptr = conv_prev.data_ptr()
     steps_dev, steps_host = None, 0
     if isinstance(steps, torch.Tensor):

@@ -88,6 +88,20 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
     return ws
 
 
+def _require_operands(who: str, K: int, N: int, group_size: int, w: torch.Tensor, scales: torch.Tensor,
+                      biases: torch.Tensor, device: torch.device, lead: Tuple[int, ...] = ()) -> None:
+    """The kernels read what K, N and the group size say: weights of any other extent, word size
+    or device must not reach them (``lead``: leading extents, the experts of the gathered form)."""
+    groups = lead + (N, K // group_size)
+    if (tuple(w.shape) != lead + (N, K // 8) or w.element_size() != 4 or tuple(scales.shape) != groups
+            or tuple(biases.shape) != groups or scales.dtype not in _DTYPE_CODE or biases.dtype != scales.dtype
+            or not (w.device == scales.device == biases.device == device)):
+        raise ValueError(f"{who}: K={K}, N={N} need w {list(lead + (N, K // 8))} of 32-bit words and bf16/fp16 scales, "
+                         f"biases {list(groups)} on {device}; got {tuple(w.shape)} {w.dtype}, {tuple(scales.shape)} "
+                         f"{scales.dtype}, {tuple(biases.shape)} {biases.dtype} on {w.device}, {scales.device}, "
+                         f"{biases.device}")
+
+
 def _launch(x2: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
             K: int, N: int, group_size: int, variant: str, k_parts: int) -> torch.Tensor:
     if not x2.is_cuda:
@@ -97,6 +111,7 @@ def _launch(x2: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: tor
     lib = _native.lib()
     if scales.dtype not in _DTYPE_CODE or biases.dtype != scales.dtype:
         raise TypeError(f"scales/biases must both be bf16 or fp16, got {scales.dtype}/{biases.dtype}")
+    _require_operands("verify_matmul", K, N, group_size, w, scales, biases, x2.device)
     y = torch.empty((16, N), dtype=x2.dtype, device=x2.device)
     stream = _native.raw_stream(x2.device)
     vcode = _VARIANT_CODE[variant]
@@ -220,6 +235,7 @@ class QmmChain:
             K, N = int(w.shape[1]) * 8, int(w.shape[0])
             if int(x2.shape[1]) != K or s.dtype not in _DTYPE_CODE or b.dtype != s.dtype or N % 32 != 0:
                 raise ValueError(f"QmmChain: operands of projection {i} do not fit together (K={K}, N={N})")
+            _require_operands(f"QmmChain, projection {i}", K, N, group_size, w, s, b, x2.device)
             act = x2.dtype if act is None else act
             sb = s.dtype if sb is None else sb
             device = x2.device if device is None else device
@@ -411,6 +427,9 @@ def gather_qmm(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: t
     E, N = int(w_q.shape[0]), int(w_q.shape[1])
     if ids.numel() != P:
         raise ValueError("one expert id per row of x is required")
+    if w_q.ndim != 3 or x2.dtype not in _DTYPE_CODE or ids.device != x2.device:
+        raise ValueError("gather_qmm: w [E, N, K/8], bf16/fp16 x and the expert ids on x's device are required")
+    _require_operands("gather_qmm", K, N, group_size, w_q, scales, biases, x2.device, lead=(E,))
     y = torch.empty((P, N), dtype=x2.dtype, device=x2.device)
     stream = _native.raw_stream(x2.device)
     # DFLASH_QMM_KERNEL=tile keeps the streaming kernel out of the gathered form as well
