@@ -161,23 +161,29 @@ def bench_qmm_stack(stack: str, steps: int, warmup: int, device: str, join_gate_
     return res
 
 
-def bench_qmm_chain_stack(stack: str, steps: int, warmup: int, device: str, layers_per_launch: int = 1):
+def bench_qmm_chain_stack(stack: str, steps: int, warmup: int, device: str, layers_per_launch: int = 1,
+                          join_gate_up: bool = False):
     """The same stack with the projections of ``layers_per_launch`` layers handed over as one list
     per launch (``QmmChain``, dflash_qmm_m16_chain): one persistent grid runs them back to back,
     each divided among the workgroups as a launch of its own would be.  Every projection has an
     input of its own here, as in the headline (no dependencies between them), and the outputs
-    must equal those of the separate launches bit for bit."""
+    must equal those of the separate launches bit for bit.  ``join_gate_up``: gate_proj and
+    up_proj as one problem of both matrices' rows (see ``build_stack``)."""
     import torch
 
     from dflash_mlx_amd._native import QMM_CHAIN_MAX
     from dflash_mlx_amd.verify_qmm import ChainProblem, QmmChain
     from dflash_mlx_amd.workloads import stack_bytes, stack_linears
 
-    calls = build_stack(stack, device)
-    per_layer = len(stack_linears(stack)[0])
+    calls = build_stack(stack, device, join_gate_up)
+    per_layer = len(stack_linears(stack)[0]) - (1 if join_gate_up else 0)
     per_chain = per_layer * layers_per_launch
     assert per_chain <= QMM_CHAIN_MAX
     _, total_bytes = stack_bytes(stack)
+    if join_gate_up:  # x is shared: count what the problems handed over here move
+        from dflash_mlx_amd.workloads import qmm_algorithmic_bytes
+
+        total_bytes = sum(qmm_algorithmic_bytes(c.K, c.N)[1] for c in calls)
     chains = [QmmChain([ChainProblem(c.x, c.w, c.scales, c.biases) for c in calls[i:i + per_chain]])
               for i in range(0, len(calls), per_chain)]
 
@@ -821,6 +827,12 @@ def main() -> int:
             log(f"[bench] {args.workload} stack, {n_layers} layer(s) per chained launch: {ch['ms_per_step']:.3f} ms/step, "
                 f"{ch['us_per_layer']:.2f} us/layer")
             extra[f"stack_{args.workload}_chained_{n_layers}_layer_per_launch"] = rnd(ch)
+        for n_layers in (1, 4):
+            ch = bench_qmm_chain_stack(args.workload, args.steps, args.warmup, device, layers_per_launch=n_layers,
+                                       join_gate_up=True)
+            log(f"[bench] {args.workload} stack, {n_layers} layer(s) per chained launch, gate/up as one problem: "
+                f"{ch['ms_per_step']:.3f} ms/step, {ch['us_per_layer']:.2f} us/layer")
+            extra[f"stack_{args.workload}_chained_{n_layers}_layer_per_launch_gate_up_as_one_problem"] = rnd(ch)
     if "mlp" in legs:
         mlp = bench_mlp_chain(args.workload, args.steps, args.warmup, device)
         extra[f"mlp_{args.workload}"] = {k: (rnd(v) if isinstance(v, dict) else round(v, 6)) for k, v in mlp.items()}
