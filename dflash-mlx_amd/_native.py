@@ -12,14 +12,15 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
 QMM_KERNEL_AUTO, QMM_KERNEL_TILE, QMM_KERNEL_STREAM = 0, 1, 2
 QMM_STATIC_SCRATCH_BYTES = 8 << 20  # DFLASH_QMM_STATIC_SCRATCH_BYTES
 QMM_CHAIN_MAX = 16                       # DFLASH_QMM_CHAIN_MAX
-QMM_CHAIN_ERROR_OFFSET = (16384 - 64 + 1) * 4  # DFLASH_QMM_CHAIN_ERROR_OFFSET
+QMM_ERROR_OFFSET = (16384 - 64 + 1) * 4        # DFLASH_QMM_ERROR_OFFSET
+QMM_CHAIN_ERROR_OFFSET = QMM_ERROR_OFFSET      # DFLASH_QMM_CHAIN_ERROR_OFFSET
 QMM_EPILOGUE_NONE, QMM_EPILOGUE_SILU_MUL = 0, 1
 OPT_GDN_STEP_BY_STEP, OPT_SDPA_SPLITS, OPT_SDPA_STAGED = 0, 1, 2  # DFLASH_OPT_*
 
@@ -38,6 +39,7 @@ EXPORTED_SYMBOLS = (
     "dflash_get_option",
     "dflash_qmm_m16_workspace_bytes",
     "dflash_qmm_m16",
+    "dflash_qmm_error",
     "dflash_qmm_m16_static",
     "dflash_qmm_m16_chain_workspace_bytes",
     "dflash_qmm_m16_chain",
@@ -81,6 +83,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.dflash_qmm_m16.argtypes = (
         [c.c_void_p] * 6 + [c.c_size_t] + [c.c_int] * 8 + [c.c_void_p]
     )
+    lib.dflash_qmm_error.restype = c.c_int
+    lib.dflash_qmm_error.argtypes = [c.c_void_p, c.POINTER(c.c_uint32), c.c_void_p]
     lib.dflash_qmm_m16_static.restype = c.c_int
     lib.dflash_qmm_m16_static.argtypes = [c.c_void_p] * 5 + [c.c_int] * 8 + [c.c_void_p]
     lib.dflash_qmm_m16_chain_workspace_bytes.restype = c.c_size_t

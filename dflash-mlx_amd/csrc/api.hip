@@ -37,3 +37,11 @@ extern "C" int dflash_get_option(int option) {
   DFLASH_REQUIRE(option >= 0 && option < DFLASH_OPT_COUNT, DFLASH_ERR_ARG, "dflash_get_option: option %d", option);
   return dflash::option(option);
 }
+
+extern "C" int dflash_qmm_error(const void* workspace, uint32_t* word_host, void* stream) {
+  DFLASH_REQUIRE(workspace && word_host, DFLASH_ERR_ARG, "dflash_qmm_error: null argument");
+  DFLASH_HIP_OK(hipStreamSynchronize((hipStream_t)stream));
+  DFLASH_HIP_OK(hipMemcpy(word_host, (const char*)workspace + DFLASH_QMM_ERROR_OFFSET, sizeof(uint32_t),
+                          hipMemcpyDeviceToHost));
+  return DFLASH_OK;
+}

@@ -211,8 +211,11 @@ __global__ __launch_bounds__(kThreads) void qmm_m16_kernel(
   for (int t = 0; t < NT; ++t) {
     float sum = 0.f;
     for (int p = 0; p < k_parts; ++p) {
-      sum += __hip_atomic_load(&partials[((size_t)p * 16 + m) * N + n0 + 16 * t + col],
-                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      float* slot = &partials[((size_t)p * 16 + m) * N + n0 + 16 * t + col];
+      sum += __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // the workspace is left zero-filled: the streaming kernel, which may share it, takes a
+      // non-zero word in a slot of its own for a partial tile that has arrived
+      __hip_atomic_store(slot, 0.f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     y[(size_t)m * N + n0 + 16 * t + col] = (uint16_t)A::from_f32(sum);
   }
@@ -403,7 +406,8 @@ int launch_gather_gs(int act_dtype, int sb_dtype, const void* x, const int32_t* 
 // Layout of the workspace: [arrival counters, fixed 64 KiB][partials: k_parts*16*N fp32].
 // The counter block has the same size for every shape so that calls of different
 // shapes sharing one workspace never put partial sums where another call keeps its
-// counters (counters must read zero when a call starts; partials may hold anything).
+// counters (counters must read zero when a call starts; so must the partials, for the sake
+// of the streaming kernel, and every kernel leaves them so).
 constexpr size_t kCounterBytes = 64 * 1024;
 constexpr int kMaxCounterTiles = (int)(kCounterBytes / sizeof(uint32_t));
 
@@ -514,30 +518,21 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace dflash {
 namespace {
-// zero-fills the counter block (16 bytes per thread)
-__global__ __launch_bounds__(256) void scratch_clear_kernel(uint4* p, int n16) {
-  const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
-  if (i < n16) p[i] = make_uint4(0u, 0u, 0u, 0u);
-}
-
 // Device address of `scratch` on the current device.  In host code the array's name is only
 // a handle for the runtime, never an address a kernel could use: the address is asked for
-// once per device (each device has its own copy at its own address) and kept.  The first
-// use on a device also puts the counter block to zero on `stream`, ahead of the caller's
-// kernel; from then on every call leaves the counters at zero.
-int static_scratch(void** out, hipStream_t stream) {
+// once per device (each device has its own copy at its own address) and kept.  Nothing is
+// enqueued: the array reads zero when the image is loaded, which is the state a workspace
+// starts from, and every call leaves it zero-filled where the next one needs it.
+int static_scratch(void** out) {
   static std::mutex mu;
   static void* ptrs[kMaxDevices] = {};
   const int slot = current_device_slot();
   std::lock_guard<std::mutex> lock(mu);
-  // devices beyond the table share its last entry: looked up (and cleared) on every call
+  // devices beyond the table share its last entry: looked up on every call
   if (ptrs[slot] == nullptr || slot == kMaxDevices - 1) {
     void* ptr = nullptr;
     DFLASH_HIP_OK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
     DFLASH_REQUIRE(ptr != nullptr, DFLASH_ERR_HIP, "dflash_qmm_m16_static: no device address for the scratch array");
-    const int n16 = (int)(kCounterBytes / 16);
-    hipLaunchKernelGGL(scratch_clear_kernel, dim3((n16 + 255) / 256), dim3(256), 0, stream, (uint4*)ptr, n16);
-    DFLASH_HIP_OK(hipGetLastError());
     ptrs[slot] = ptr;
   }
   *out = ptrs[slot];
@@ -558,7 +553,7 @@ extern "C" int dflash_qmm_m16_static(const void* x, const uint32_t* w_q, const v
                  "array holds %zu; use dflash_qmm_m16 with a workspace of the caller's",
                  need, kStaticScratchBytes);
   void* ptr = nullptr;
-  const int rc = static_scratch(&ptr, (hipStream_t)stream);
+  const int rc = static_scratch(&ptr);
   if (rc != DFLASH_OK) return rc;
   return dflash_qmm_m16(x, w_q, scales, biases, y, ptr, kStaticScratchBytes, K, N, group_size,
                         act_dtype, sb_dtype, variant, k_parts, kernel, stream);

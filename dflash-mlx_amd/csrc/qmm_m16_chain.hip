@@ -687,6 +687,9 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
           if (wg0 + j <= hi_wg) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) sum[i][r] += v[j][r];
+            // the workspace is left zero-filled: the streaming kernel, which may share it, takes
+            // a non-zero word in a slot of its own for a partial tile that has arrived
+            store_partial(const_cast<float*>(src[j]), f32x4_t{0.f, 0.f, 0.f, 0.f});
           }
         }
       }

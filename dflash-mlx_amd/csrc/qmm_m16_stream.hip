@@ -29,11 +29,18 @@
 //    the same rows add their accumulators through LDS only when a row block ends; after
 //    that worker w holds tile w.
 //  * A workgroup whose range covers all of K for a row block writes y directly.  Row
-//    blocks shared between workgroups go through fp32 partial tiles in the workspace; a
-//    workgroup announces its tiles once, after its last unit (wrapping agent-scope
-//    counter per row block), and the last contributor to arrive adds them in contributor
-//    order and rounds once - deterministic, no spinning.  Partials are written through to
-//    / read from the level all XCDs share (sc1): no L2 write-back fence is ever issued.
+//    blocks shared between workgroups go through fp32 partial tiles in the workspace, in
+//    ONE memory round trip: a partial tile is its own "ready" flag.  Slots read zero
+//    between calls; a contributor stores its tile with every +0.0 written as -0.0, so that
+//    no word of a stored tile has the bit pattern zero, and leaves.  One fixed contributor
+//    per row block - the one with the highest block index, so that everything it waits for
+//    was dispatched before it - keeps its own tile in registers, reads the others' slots
+//    until every word is non-zero, adds the tiles in contributor order, rounds once, and
+//    puts the slots back to zero.  Deterministic; the wait is bounded (a workgroup that
+//    gives up records an error word in the workspace and the launch still ends).  Partials
+//    are written through to / read from the level all XCDs share (sc1): no L2 write-back
+//    fence is ever issued, nobody waits for a store to be acknowledged, and there is no
+//    arrival counter whose answer somebody would have to wait for.
 //
 // The compiler orders every LDS access it can see behind ALL outstanding direct-to-LDS
 // loads (s_waitcnt vmcnt(0)), and __syncthreads() carries a fence with the same effect;
@@ -58,8 +65,12 @@ struct Params {
   const uint16_t* scales;
   const uint16_t* biases;
   uint16_t* y;
-  float* partials;     // [2 * grid][wave][lane][4] fp32
-  uint32_t* counters;  // [row blocks of all entries]
+  float* partials;     // [2 * grid][wave][lane][4] fp32; all zero between calls
+  uint32_t* status;    // the 64 KiB block ahead of the partial tiles: [kErrorWord] is set when a wait gives up
+  int spin_limit;      // polls of a row block's partial tiles before the adding workgroup gives up
+#ifdef DFLASH_STREAM_STAMPS
+  int stamp_slot;
+#endif
   int K, N;
   int stages;          // K / 256
   int units;           // row blocks * stages (dense form; the gathered form counts its own)
@@ -113,6 +124,19 @@ __global__ __launch_bounds__(256) void qmm_pack_kernel(const uint32_t* __restric
   }
 }
 
+#ifdef DFLASH_STREAM_STAMPS
+// Experiment builds only: wall-clock stamps of wave 0 (a worker) and wave 8 (a loader) of every
+// workgroup, for the last 64 launches.  [launch % 64][block][event]
+__device__ unsigned long long g_sstamps[64][256][16];
+#define DFLASH_SSTAMP(ev)                                                                     \
+  do {                                                                                        \
+    if (lane == 0 && (wave == 0 || wave == kWaves) && blockIdx.x < 256)                       \
+      g_sstamps[p.stamp_slot & 63][blockIdx.x][ev] = wall_clock64();                         \
+  } while (0)
+#else
+#define DFLASH_SSTAMP(ev) do {} while (0)
+#endif
+
 // CHUNK: units per scale/bias chunk (4, or 2 when K is a multiple of 512 only).
 // GATHER: per-expert form.  Rows of x that share an expert are taken 16 at a time as one
 // "entry"; an entry is a matrix problem of its own, [rows, K] x [N, K]^T, and the unit
@@ -137,6 +161,8 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t lds0 = lds_address(lds);
+  if (wave == 0) DFLASH_SSTAMP(0);
+  if (wave == kWaves) DFLASH_SSTAMP(8);
   const int RB = (p.N + kRows - 1) / kRows;  // row blocks of one matrix
   // bytes from one unit's codes to the next unit's of the same rows, and from chunk to chunk
   const bool packed = !GATHER && CHUNK == 4 && p.packed;
@@ -245,8 +271,8 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
   //     slot of unit u is free),
   //   when a row block ends with unit u: one more (the slot of unit u carries the cross-wave
   //     sum),
-  //   after the last unit, if a row block was shared with other workgroups: two more (partial
-  //     tiles stored / arrival counters bumped).
+  // (the hand-over of shared row blocks after the last unit involves the worker waves only,
+  // each on its own: no barrier).
 
   if (wave >= kWaves) {
     // ================================ loader waves ====================================
@@ -363,12 +389,13 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
     };
 
     const int ahead = units < 4 * grid ? kAheadShort : kAhead;
+    DFLASH_SSTAMP(9);
     for (int i = kFirst; i < ahead && issued < u1; ++i) issue_next();
     if (!kFirst) wait_unit(u0);
+    DFLASH_SSTAMP(10);
     asm volatile("s_barrier" ::: "memory");
+    DFLASH_SSTAMP(11);
     int rb_left = p.stages - st0;  // units of the current row block from unit u on
-    int in_rb = 0;                 // units of the current row block this workgroup has done
-    bool any_shared = false;       // a row block ended that other workgroups share
 #pragma unroll 1
     for (int u = u0; u < u1; ++u) {
       const bool rb_ends = rb_left == 1 || u + 1 == u1;
@@ -379,18 +406,11 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       // refilled kDepth - kAhead units later
       const int limit = u + ahead;
       while (issued <= limit && issued < u1) issue_next();
-      ++in_rb;
       --rb_left;
       if (rb_ends) {
         asm volatile("s_barrier" ::: "memory");
-        if (in_rb != p.stages) any_shared = true;
-        in_rb = 0;
         rb_left = p.stages;
       }
-    }
-    if (any_shared) {
-      asm volatile("s_barrier" ::: "memory");
-      asm volatile("s_barrier" ::: "memory");
     }
     return;
   }
@@ -498,8 +518,11 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
     }
   };
 
+  DFLASH_SSTAMP(1);
   if (kWorkersFetchFirstChunk) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  DFLASH_SSTAMP(2);
   asm volatile("s_barrier" ::: "memory");
+  DFLASH_SSTAMP(3);
   next_addresses();
   operands_issue_piece<0, SBROW>(rd_x, rd_w, rd_s, op[0], acc4[0]);
   operands_issue_piece<1, SBROW>(rd_x, rd_w, rd_s, op[0], acc4[0]);
@@ -512,7 +535,35 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
   int in_rb = 0;                 // units of the current row block this workgroup has done
   int rb = rb0;
   int cur_slot = 0;              // byte offset of the current unit's ring slot
-  int shared_rb[2] = {-1, -1};   // row blocks whose partial tiles I have stored
+  int mine_rb[2] = {-1, -1};     // shared row blocks whose tiles I add (slot 0: the one my range starts in)
+  f32x4_t mine0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, mine1 = mine0;  // my own tiles of those row blocks
+
+  // contributors of a row block: the workgroups whose ranges intersect [lo, lo+stages);
+  // owner(v) = ceil((v+1)*grid/units) - 1 is the workgroup whose range holds unit v
+  auto contributors = [&](int vrb, int& lo_wg, int& hi_wg) __attribute__((always_inline)) {
+    const int lo = vrb * p.stages;
+    lo_wg = (int)((((unsigned)lo + 1u) * (unsigned)grid + units - 1) / (unsigned)units) - 1;
+    hi_wg = (int)((((unsigned)(lo + p.stages)) * (unsigned)grid + units - 1) / (unsigned)units) - 1;
+  };
+  // Who adds the tiles of a row block with contributors lo_wg..hi_wg: the one with the highest
+  // block index.  Workgroups are dispatched in the order of their block indices, so all the
+  // others are running or have finished when it starts: its wait cannot keep a workgroup it
+  // waits for off the device.  Unit ranges in block order: the last contributor.  In the
+  // XCD-major order (block = (wg % per) * 8 + wg / per, per = grid / 8) the block index grows
+  // with wg inside a chunk of `per` ranges, and the last range of a chunk has the highest index
+  // of all: the last contributor if the contributors sit in one chunk or end on its last range,
+  // else the last range of the chunk before.
+  const bool xcd_major = grid == (int)gridDim.x && grid % xcds == 0;
+  auto adder_of = [&](int lo_wg, int hi_wg) __attribute__((always_inline)) -> int {
+    if (!xcd_major) return hi_wg;
+    const int per = grid / xcds;
+    const int chunk = hi_wg / per;
+    if (lo_wg / per == chunk || hi_wg - chunk * per == per - 1) return hi_wg;
+    return chunk * per - 1;
+  };
+  auto slot_of = [&](int w, int which) __attribute__((always_inline)) -> float* {
+    return p.partials + ((size_t)w * 2 + which) * kPartialFloats + tid * 4;
+  };
 
 #pragma unroll 1
   while (true) {
@@ -530,6 +581,9 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       operands_wait(nxt, acc4[0], acc4[1], acc4[2], acc4[3]);
       --left;
       ++in_rb;
+#ifdef DFLASH_STREAM_STAMPS
+      if (left + 1 == u1 - u0) DFLASH_SSTAMP(4);
+#endif
       if (--rb_left == 0 || left == 0) {
         // ---- a row block ends inside my range ---------------------------------------------
         const uint32_t sbase = lds0 + cur_slot;
@@ -543,11 +597,18 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
         } else {
           // Other workgroups hold the rest of this row block.  A workgroup shares at most two
           // row blocks: the one its range starts in (partial slot 0) and the one it ends in
-          // (slot 1); partial tiles are kept in accumulator layout.  The store is not awaited
-          // here: arrival is announced once, after the last unit.
+          // (slot 1); partial tiles are kept in accumulator layout.  The workgroup that adds
+          // keeps its tile; every other one stores it and is done with the row block.
           const int which = rb == rb0 ? 0 : 1;
-          store_partial(p.partials + ((size_t)wg * 2 + which) * kPartialFloats + tid * 4, acc);
-          shared_rb[which] = rb;
+          int lo_wg, hi_wg;
+          contributors(rb, lo_wg, hi_wg);
+          if (adder_of(lo_wg, hi_wg) == wg) {
+            mine_rb[which] = rb;
+            if (which == 0) mine0 = acc;
+            else mine1 = acc;
+          } else {
+            store_partial(slot_of(wg, which), nonzero_words(acc));
+          }
         }
         ++rb;
         in_rb = 0;
@@ -555,102 +616,67 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_stream_kernel(Params p) {
       }
       cur_slot += kSlotBytes;
       if (cur_slot == kDepth * kSlotBytes) cur_slot = 0;
-      if (left == 0) goto arrive;
+      if (left == 0) goto hand_over;
     }
   }
-arrive:
-  if (shared_rb[0] < 0 && shared_rb[1] < 0) return;
-  // ---- arrival at the shared row blocks ---------------------------------------------------
-  // Every worker's partial stores have been acknowledged before the barrier, hence before
-  // thread 0 bumps the counters; a release fence here would write back the whole L2.
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  asm volatile("s_barrier" ::: "memory");
-  int wg_lo[2], wg_hi[2];
+hand_over:
+  DFLASH_SSTAMP(5);
+  // ---- the row blocks whose tiles I add -----------------------------------------------------
+  // Every wave on its own (its 1 KiB of every tile): read the other contributors' slots, eight
+  // tiles at a time, until no word is zero; add in contributor order, my own tile in its place;
+  // store the result; put the slots back to zero for the next call.
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
-    // contributors of a row block: the workgroups whose ranges intersect [lo, lo+stages);
-    // owner(v) = ceil((v+1)*grid/units) - 1 is the workgroup whose range holds unit v
-    const int lo = shared_rb[i] * p.stages;
-    wg_lo[i] = (int)((((unsigned)lo + 1u) * (unsigned)grid + units - 1) / (unsigned)units) - 1;
-    wg_hi[i] = (int)((((unsigned)(lo + p.stages)) * (unsigned)grid + units - 1) / (unsigned)units) - 1;
-  }
-  if (tid == 0) {
-    uint32_t prev[2] = {0u, 0u}, flag[2];
+    if (mine_rb[i] < 0) continue;
+    int lo_wg, hi_wg;
+    contributors(mine_rb[i], lo_wg, hi_wg);
+    // Only the first contributor can have started before the row block (then the block is the
+    // one its range ends in, slot 1); every later one starts inside it (slot 0).
+    const int which_first = range_begin(units, lo_wg, grid) < mine_rb[i] * p.stages ? 1 : 0;
+    const f32x4_t own = i == 0 ? mine0 : mine1;
+    f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int wg0 = lo_wg; wg0 <= hi_wg; wg0 += 8) {  // more than eight contributors: long K, few rows
+      const float* src[8];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      // wrapping increment: the last arrival sees n-1 and leaves 0 behind for the next call
-      if (shared_rb[i] >= 0) prev[i] = atomicInc(&p.counters[shared_rb[i]], (uint32_t)(wg_hi[i] - wg_lo[i]));
-    }
+      for (int j = 0; j < 8; ++j) {
+        const int w = wg0 + j <= hi_wg ? wg0 + j : hi_wg;  // surplus slots re-read the last tile
+        src[j] = slot_of(w, w == lo_wg ? which_first : 0);
+      }
+      f32x4_t v[8];
+      int polls = 0;
+      while (true) {
+        load_partials8(src, v);
+        uint32_t present = 1u;  // stays non-zero while no word of a tile I wait for is zero
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-      flag[i] = (shared_rb[i] >= 0 && prev[i] == (uint32_t)(wg_hi[i] - wg_lo[i])) ? 1u : 0u;
-    asm volatile("ds_write_b32 %0, %1\n ds_write_b32 %0, %2 offset:4\n s_waitcnt lgkmcnt(0)"
-                 :
-                 : "v"(lds0), "v"(flag[0]), "v"(flag[1])
-                 : "memory");
-  }
-  asm volatile("s_barrier" ::: "memory");
-  uint32_t last0, last1;
-  asm volatile("ds_read_b32 %0, %2\n ds_read_b32 %1, %2 offset:4\n s_waitcnt lgkmcnt(0)"
-               : "=&v"(last0), "=&v"(last1)
-               : "v"(lds0)
-               : "memory");
-  const bool is_last[2] = {__builtin_amdgcn_readfirstlane(last0) != 0,
-                           __builtin_amdgcn_readfirstlane(last1) != 0};
-  // The last contributor to arrive adds the partial tiles in contributor order.  Only the
-  // first contributor can have started before a row block (then the block is the one its range
-  // ends in, slot 1); every later one starts inside it (slot 0).  A workgroup that is last at
-  // both of its row blocks asks for the tiles of both before it adds any: the two answers take
-  // as long as one.
-  auto sources = [&](int i, int wg0, const float* (&src)[8]) __attribute__((always_inline)) {
-    const int lo = shared_rb[i] * p.stages;
-    const int which_first = range_begin(units, wg_lo[i], grid) < lo ? 1 : 0;
+        for (int j = 0; j < 8; ++j) {
+          if (wg0 + j <= hi_wg && wg0 + j != wg) {
+            const u32x4_t bits = __builtin_bit_cast(u32x4_t, v[j]);
+            present = min(present, min(min(bits.x, bits.y), min(bits.z, bits.w)));
+          }
+        }
+        if (__builtin_amdgcn_ballot_w64(present == 0u) == 0ull) break;
+        if (++polls > p.spin_limit) {
+          // gives up: the launch ends, this row block's output is wrong, and the caller can tell
+          if (lane == 0) __hip_atomic_store(&p.status[kErrorWord], 0x80000000u | (uint32_t)mine_rb[i],
+                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(2);
+      }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int w = wg0 + j <= wg_hi[i] ? wg0 + j : wg_hi[i];  // surplus slots re-read the last tile
-      src[j] = p.partials + ((size_t)w * 2 + (w == wg_lo[i] ? which_first : 0)) * kPartialFloats + tid * 4;
-    }
-  };
-  auto add_round = [&](int i, int wg0, const f32x4_t (&v)[8], f32x4_t& acc) __attribute__((always_inline)) {
+      for (int j = 0; j < 8; ++j) {
+        if (wg0 + j <= hi_wg) {
+          const bool me = wg0 + j == wg;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      if (wg0 + j <= wg_hi[i]) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) acc[r] += v[j][r];
+          for (int r = 0; r < 4; ++r) acc[r] += me ? own[r] : v[j][r];
+          if (!me) store_partial(const_cast<float*>(src[j]), f32x4_t{0.f, 0.f, 0.f, 0.f});
+        }
       }
     }
-  };
-  f32x4_t first[2][8];
-  if (is_last[0] && is_last[1]) {
-    const float* src0[8];
-    const float* src1[8];
-    sources(0, wg_lo[0], src0);
-    sources(1, wg_lo[1], src1);
-    issue_partials8(src0, first[0]);
-    join_partials8(src1, first[1], first[0]);
-  } else {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      if (!is_last[i]) continue;
-      const float* src[8];
-      sources(i, wg_lo[i], src);
-      load_partials8(src, first[i]);
-    }
+    DFLASH_SSTAMP(6);
+    emit(mine_rb[i], acc);
   }
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    if (!is_last[i]) continue;
-    f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    add_round(i, wg_lo[i], first[i], acc);
-    for (int wg0 = wg_lo[i] + 8; wg0 <= wg_hi[i]; wg0 += 8) {  // more than eight contributors: long K, few rows
-      const float* src[8];
-      sources(i, wg0, src);
-      f32x4_t v[8];
-      load_partials8(src, v);
-      add_round(i, wg0, v, acc);
-    }
-    emit(shared_rb[i], acc);
-  }
+  DFLASH_SSTAMP(7);
 }
 
 }  // namespace stream
@@ -754,6 +780,10 @@ int launch_stream(stream::Params& p, bool gather, int grid, int act_dtype, int s
     DFLASH_HIP_OK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
     attr_set[slot][idx] = true;
   }
+#ifdef DFLASH_STREAM_STAMPS
+  static int launches = 0;
+  p.stamp_slot = launches++;
+#endif
   void* args[] = {&p};
   DFLASH_HIP_OK(hipLaunchKernel(fn, dim3(grid), dim3(kThreads), args, lds_bytes, stream));
   return DFLASH_OK;
@@ -779,8 +809,9 @@ int qmm_stream_launch(const void* x, const uint32_t* w, const void* scales, cons
   DFLASH_REQUIRE(workspace && workspace_bytes >= need, DFLASH_ERR_WORKSPACE,
                  "dflash_qmm_m16: workspace of %zu bytes needed, %zu given", need,
                  workspace ? workspace_bytes : (size_t)0);
-  p.counters = (uint32_t*)workspace;
+  p.status = (uint32_t*)workspace;
   p.partials = (float*)((char*)workspace + 64 * 1024);
+  p.spin_limit = kSpinLimit;
   return launch_stream(p, false, grid, act_dtype, sb_dtype, stream);
 }
 
@@ -826,8 +857,9 @@ int qmm_stream_packed_launch(const void* x, const void* w_img, const void* s_img
   DFLASH_REQUIRE(workspace && workspace_bytes >= need, DFLASH_ERR_WORKSPACE,
                  "dflash_qmm_m16_packed: workspace of %zu bytes needed, %zu given", need,
                  workspace ? workspace_bytes : (size_t)0);
-  p.counters = (uint32_t*)workspace;
+  p.status = (uint32_t*)workspace;
   p.partials = (float*)((char*)workspace + 64 * 1024);
+  p.spin_limit = kSpinLimit;
   return launch_stream(p, false, grid, act_dtype, sb_dtype, stream);
 }
 
@@ -855,9 +887,16 @@ int qmm_stream_gather_launch(const void* x, const int32_t* expert_ids, const uin
   DFLASH_REQUIRE(workspace && workspace_bytes >= need, DFLASH_ERR_WORKSPACE,
                  "dflash_qmm_m16_gather: workspace of %zu bytes needed, %zu given", need,
                  workspace ? workspace_bytes : (size_t)0);
-  p.counters = (uint32_t*)workspace;
+  p.status = (uint32_t*)workspace;
   p.partials = (float*)((char*)workspace + 64 * 1024);
+  p.spin_limit = kSpinLimit;
   return launch_stream(p, true, grid, act_dtype, sb_dtype, stream);
 }
 
 }  // namespace dflash
+
+#ifdef DFLASH_STREAM_STAMPS
+extern "C" int dflash_debug_read_stream_stamps(unsigned long long* out_host) {
+  return (int)hipMemcpyFromSymbol(out_host, HIP_SYMBOL(dflash::stream::g_sstamps), sizeof(dflash::stream::g_sstamps));
+}
+#endif

@@ -244,9 +244,28 @@ __device__ __forceinline__ f32x4_t reduce_groups_read(uint32_t base, const f32x4
   return own;
 }
 
+// Word of the workspace's first 64 KiB that a workgroup sets when a bounded wait gives up
+// (DFLASH_QMM_ERROR_OFFSET / 4 of the C interface).
+constexpr int kErrorWord = 16384 - 64 + 1;
+// Polls of a row block's partial tiles (about a microsecond each) before the adding workgroup
+// gives up.
+constexpr int kSpinLimit = 1 << 18;
+
+// A partial tile on its way through memory doubles as its own "ready" flag: +0.0 travels as
+// -0.0 (the sum starts from +0.0, and +0.0 + -0.0 = +0.0, x + -0.0 = x: nothing changes), so
+// no word of a stored tile is all zero bits, which is what an empty slot holds.
+__device__ __forceinline__ f32x4_t nonzero_words(f32x4_t v) {
+#pragma unroll
+  for (int r = 0; r < 4; ++r) v[r] = v[r] == 0.0f ? -0.0f : v[r];
+  return v;
+}
+
 // Partial accumulator tiles cross XCDs: stored and loaded at agent scope (sc1).
 __device__ __forceinline__ void store_partial(float* p, f32x4_t v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1\n" : : "v"(p), "v"(v) : "memory");
+  // A store of more than 64 bits reads the upper half of its data a cycle after it has been
+  // issued, and the compiler, which inserts the wait states such hazards need, cannot see
+  // inside this block: the next instruction it places may write those registers.
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n s_nop 1\n" : : "v"(p), "v"(v) : "memory");
 }
 // eight tiles at once, so that their latencies overlap
 __device__ __forceinline__ void load_partials8(const float* const (&p)[8], f32x4_t (&v)[8]) {
@@ -262,43 +281,6 @@ __device__ __forceinline__ void load_partials8(const float* const (&p)[8], f32x4
       "s_waitcnt vmcnt(0)\n"
       : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]),
         "=&v"(v[7])
-      : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7])
-      : "memory");
-}
-
-// The same loads for two row blocks at once: issue_partials8() only asks, and join_partials8()
-// asks for the second block's tiles and waits for both; it names the first block's registers
-// as operands of its own, so that nothing can be placed between the two that touches them
-// while they are being written.
-__device__ __forceinline__ void issue_partials8(const float* const (&p)[8], f32x4_t (&v)[8]) {
-  asm volatile(
-      "global_load_dwordx4 %0, %8, off sc1\n"
-      "global_load_dwordx4 %1, %9, off sc1\n"
-      "global_load_dwordx4 %2, %10, off sc1\n"
-      "global_load_dwordx4 %3, %11, off sc1\n"
-      "global_load_dwordx4 %4, %12, off sc1\n"
-      "global_load_dwordx4 %5, %13, off sc1\n"
-      "global_load_dwordx4 %6, %14, off sc1\n"
-      "global_load_dwordx4 %7, %15, off sc1\n"
-      : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]),
-        "=&v"(v[7])
-      : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7])
-      : "memory");
-}
-__device__ __forceinline__ void join_partials8(const float* const (&p)[8], f32x4_t (&v)[8], f32x4_t (&first)[8]) {
-  asm volatile(
-      "global_load_dwordx4 %0, %16, off sc1\n"
-      "global_load_dwordx4 %1, %17, off sc1\n"
-      "global_load_dwordx4 %2, %18, off sc1\n"
-      "global_load_dwordx4 %3, %19, off sc1\n"
-      "global_load_dwordx4 %4, %20, off sc1\n"
-      "global_load_dwordx4 %5, %21, off sc1\n"
-      "global_load_dwordx4 %6, %22, off sc1\n"
-      "global_load_dwordx4 %7, %23, off sc1\n"
-      "s_waitcnt vmcnt(0)\n"
-      : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]),
-        "=&v"(v[7]), "+v"(first[0]), "+v"(first[1]), "+v"(first[2]), "+v"(first[3]), "+v"(first[4]),
-        "+v"(first[5]), "+v"(first[6]), "+v"(first[7])
       : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7])
       : "memory");
 }

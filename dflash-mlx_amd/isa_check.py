@@ -9,6 +9,11 @@ instantiation of its kernel and also refuses spills to scratch memory (a loader 
 memory operations would break its count of loads in flight).  ``check_arrivals``: between the
 last store before a bump of an arrival counter and the bump itself the code must wait for all
 of the wave's memory operations - nothing else keeps the counter from overtaking the stores.
+``check_wide_stores``: a global store of more than 64 bits reads the upper half of its data a
+cycle after it has been issued; where the compiler places such a store it also places the wait
+states, but it cannot see one inside a hand-written block, so every such store in a block must
+be followed by wait states of its own (seen on the device as partial tiles whose upper two
+words were those of whatever the next instruction wrote).
 """
 from __future__ import annotations
 
@@ -30,7 +35,7 @@ KERNELS = (
     ("sdpa_q16.hip", "_ZN6dflash12_GLOBAL__N_124sdpa_q16_resident_kernel", 24, 60),
 )
 # source, number of counter bumps (arrival counters; the chained kernel's per-problem and exit counters too)
-ARRIVALS = (("qmm_m16.hip", 24), ("qmm_m16_stream.hip", 32), ("qmm_m16_chain.hip", 32))
+ARRIVALS = (("qmm_m16.hip", 24), ("qmm_m16_stream.hip", 0), ("qmm_m16_chain.hip", 32))
 
 
 def _regs(text: str) -> set:
@@ -129,6 +134,24 @@ def check_arrivals(text: str, source: str, arrivals: int) -> None:
         raise AssertionError(f"{source}: {found} counter bumps, expected {arrivals}")
 
 
+def check_wide_stores(text: str, source: str) -> int:
+    """Every 96/128-bit global store inside a hand-written block is followed by s_nop; returns how many."""
+    lines = text.split("\n")
+    in_block, found = False, 0
+    for i, line in enumerate(lines):
+        t = line.strip()
+        if t.startswith(";;#ASMSTART"):
+            in_block = True
+        elif t.startswith(";;#ASMEND"):
+            in_block = False
+        elif in_block and re.match(r"(global|flat|buffer)_store_dwordx[34]\b", t):
+            found += 1
+            nxt = next((l.strip() for l in lines[i + 1:] if l.strip()), "")
+            if not nxt.startswith("s_nop"):
+                raise AssertionError(f"{source}: wide store at line {i + 1} of the assembly is not followed by wait states")
+    return found
+
+
 def check_all() -> None:
     """Every check on every source; raises AssertionError on the first finding."""
     from concurrent.futures import ThreadPoolExecutor
@@ -140,3 +163,6 @@ def check_all() -> None:
         check_kernels(isa[source], prefix, count, min_reads)
     for source, arrivals in ARRIVALS:
         check_arrivals(isa[source], source, arrivals)
+    for source in ("qmm_m16_stream.hip", "qmm_m16_chain.hip"):
+        if check_wide_stores(isa[source], source) == 0:
+            raise AssertionError(f"{source}: no partial-tile store found")

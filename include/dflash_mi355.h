@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 12
+#define DFLASH_ABI_VERSION 13
 
 enum {
   DFLASH_OK = 0,
@@ -84,14 +84,28 @@ int dflash_get_option(int option);
  *   biases   [N, K/group_size]  sb_dtype
  *   y        [16, N]            act_dtype
  *   workspace                   >= dflash_qmm_m16_workspace_bytes(...) bytes, 256-byte
- *                               aligned, ZERO-FILLED ONCE by the caller before its first
- *                               use; the kernel leaves it zero-filled where it must be,
- *                               so it can be reused by later calls on the same stream.
+ *                               aligned, ZERO-FILLED ONCE (all of it) by the caller before
+ *                               its first use; every qmm kernel leaves it zero-filled, so
+ *                               it can be reused by later calls on the same stream.
  *                               Calls that share a workspace must not overlap in time.
  * Requirements: group_size in {32,64,128}; N % 16 == 0; K % group_size == 0;
  * for the pipe variant K % (32*k_parts) == 0.  Results are deterministic
  * (bit-identical from run to run for identical inputs).
+ *
+ * The streaming kernel hands partial sums of row blocks that several workgroups share to one
+ * of them through the workspace; that workgroup waits for the others' partial tiles (they
+ * were dispatched before it, so they are running or done).  The wait is bounded: a workgroup
+ * that gives up - which takes a device that stops running resident workgroups for about a
+ * second - stores 0x80000000 | row block into the 32-bit word at byte offset
+ * DFLASH_QMM_ERROR_OFFSET of the workspace, the launch ends normally, and y is then
+ * undefined.  The word stays set until the caller zero-fills the workspace again, which it
+ * must do before the next call; dflash_qmm_error() reads it.
  */
+#define DFLASH_QMM_ERROR_OFFSET ((16384 - 64 + 1) * 4)
+/* Copies the error word of a qmm workspace to *word_host (0: no wait has given up) after waiting
+ * for the work enqueued on `stream`. */
+int dflash_qmm_error(const void* workspace, uint32_t* word_host, void* stream);
+
 size_t dflash_qmm_m16_workspace_bytes(int K, int N, int group_size, int variant, int k_parts,
                                       int kernel);
 
@@ -110,8 +124,9 @@ int dflash_qmm_m16(const void* x, const uint32_t* w_q, const void* scales, const
  * projections of the verify stacks need about 4 MiB; a pipe call served by the tile kernel
  * needs 64 KiB + k_parts * 64 * N bytes.  All calls on one GPU share that GPU's array:
  * calls that overlap in time on one GPU (two streams, two threads) race, as they would on a
- * shared workspace.  The first call on a GPU also enqueues a small kernel on `stream` that
- * zero-fills the array's counter block.
+ * shared workspace.  Nothing but the product's own kernel is enqueued, also by the first call
+ * on a GPU (the array reads zero when the library's image is loaded), so every call may be
+ * made under stream capture.
  */
 #define DFLASH_QMM_STATIC_SCRATCH_BYTES ((size_t)8 << 20)
 
@@ -148,7 +163,7 @@ int dflash_qmm_m16_static(const void* x, const uint32_t* w_q, const void* scales
  * which must be resident at once: the device must not be shared with other long-running kernels.
  */
 #define DFLASH_QMM_CHAIN_MAX 16
-#define DFLASH_QMM_CHAIN_ERROR_OFFSET ((16384 - 64 + 1) * 4)
+#define DFLASH_QMM_CHAIN_ERROR_OFFSET DFLASH_QMM_ERROR_OFFSET
 enum { DFLASH_QMM_EPILOGUE_NONE = 0, DFLASH_QMM_EPILOGUE_SILU_MUL = 1 };
 
 typedef struct dflash_qmm_problem {

@@ -6,6 +6,8 @@ Tolerances:
   reference's own  max_abs <= 8e-3 (bf16) / 4e-3 (fp16), max_abs/(max|y_ref|+1e-3) <= 2e-2
                    on x, w ~ N(0,1)/sqrt(K)   (tests/test_verify_qmm_parity.py:83-109)
 """
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -210,6 +212,41 @@ def test_deterministic_and_workspace_reuse(verify_env, native_lib, c_oracle):
     for y in ya[1:]:
         assert torch.equal(y, ya[0])
     _check_north_star(_f32(yb).astype(np.float64), _oracle_exact(c_oracle, b.to("cpu")))
+
+
+def test_every_kernel_hands_the_shared_workspace_back_zero_filled(verify_env, native_lib, c_oracle):
+    """The streaming kernel takes a non-zero word in a partial-tile slot for a tile that has
+    arrived, so every kernel that writes partial tiles puts them back to zero: the streaming
+    kernel itself, the tile kernel's split-K form, the chained and the gathered form.  One
+    workspace through all of them, checked after each, with the streaming kernel's result still
+    right (and the same bits as with a workspace of its own) at the end."""
+    verify_env.setenv("DFLASH_QMM_KERNEL", "auto")
+    ws = VQ._workspace(torch.device(DEV), nat.raw_stream(torch.device(DEV)), 1)
+
+    def clean():
+        torch.cuda.synchronize()
+        word = ctypes.c_uint32(7)
+        assert native_lib.dflash_qmm_error(ws.data_ptr(), ctypes.byref(word), None) == 0 and word.value == 0
+        return int((ws != 0).sum()) == 0
+
+    a = make_qmm_case(5120, 7168, 31).to(DEV)       # streaming kernel, four workgroups per row block
+    b = make_qmm_case(4096, 1536, 32).to(DEV)       # row blocks that straddle unit ranges
+    ya = VQ.verify_matmul(a.x, a.w, a.scales, a.biases)
+    yb = VQ.verify_matmul(b.x, b.w, b.scales, b.biases)
+    assert clean()
+    verify_env.setenv("DFLASH_QMM_KERNEL", "tile")  # split-K form of the tile kernel (K >= 8192 -> pipe x 8)
+    c = make_qmm_case(8192, 512, 33).to(DEV)
+    yc = VQ.verify_matmul(c.x, c.w, c.scales, c.biases)
+    verify_env.setenv("DFLASH_QMM_KERNEL", "auto")
+    assert clean()
+    chain = VQ.QmmChain([VQ.ChainProblem(a.x, a.w, a.scales, a.biases), VQ.ChainProblem(b.x, b.w, b.scales, b.biases)])
+    chained = chain()
+    assert clean()
+    assert torch.equal(chained[0], ya) and torch.equal(chained[1], yb)
+    ya2 = VQ.verify_matmul(a.x, a.w, a.scales, a.biases)
+    assert clean() and torch.equal(ya2, ya)
+    _check_north_star(_f32(ya2).astype(np.float64), _oracle_exact(c_oracle, a.to("cpu")))
+    _check_north_star(_f32(yc).astype(np.float64), _oracle_exact(c_oracle, c.to("cpu")))
 
 
 def test_n_tiles_are_independent_full_size(verify_env, native_lib, kernel_mode):

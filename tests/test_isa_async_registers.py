@@ -44,6 +44,12 @@ def test_checks_flag_what_they_are_for():
     isa_check.check_arrivals(patient, "x.hip", 1)
     with pytest.raises(AssertionError, match="expected 2"):
         isa_check.check_arrivals(patient, "x.hip", 2)
+    bare = ";;#ASMSTART\nglobal_store_dwordx4 v[2:3], v[4:7], off sc1\n;;#ASMEND\nv_mov_b32 v6, v9\n"
+    with pytest.raises(AssertionError, match="wait states"):
+        isa_check.check_wide_stores(bare, "x.hip")
+    padded = bare.replace("off sc1\n", "off sc1\ns_nop 1\n")
+    assert isa_check.check_wide_stores(padded, "x.hip") == 1
+    assert isa_check.check_wide_stores("global_store_dwordx4 v[2:3], v[4:7], off\nv_mov_b32 v6, v9\n", "x.hip") == 0
 
 
 @needs_hipcc
@@ -60,3 +66,11 @@ def test_partial_tiles_are_acknowledged_before_the_arrival_counter(source, arriv
     acknowledgement keeps the counter from overtaking them (a workgroup barrier does not wait
     for global stores on this target)."""
     isa_check.check_arrivals(_text(source), source, arrivals)
+
+
+@needs_hipcc
+@pytest.mark.parametrize("source", ["qmm_m16_stream.hip", "qmm_m16_chain.hip"])
+def test_hand_written_wide_stores_carry_their_wait_states(source):
+    """A 128-bit global store reads the upper half of its data a cycle after issue; inside a
+    hand-written block the compiler does not add the wait states that protect those registers."""
+    assert isa_check.check_wide_stores(_text(source), source) > 0

@@ -70,3 +70,35 @@ def test_static_scratch_rejects_what_does_not_fit(native_lib):
                                    nat.QMM_MMA2BIG_PIPE, 8, nat.QMM_KERNEL_TILE, None)
     assert rc == -3
     assert b"scratch" in lib.dflash_last_error()
+
+
+def test_static_scratch_under_stream_capture(native_lib):
+    """The entry point enqueues nothing but the product's kernel, so it can be captured - also as
+    the first call of a process - and replayed; every replay equals the eager result."""
+    lib = native_lib
+    K, N = 5120, 5120
+    d = make_qmm_case(K, N, 4200).to("cuda:0")
+    ws = torch.zeros(nat.QMM_STATIC_SCRATCH_BYTES, dtype=torch.uint8, device="cuda:0")
+    y_ref = torch.empty((16, N), dtype=torch.bfloat16, device="cuda:0")
+    y_cap = torch.empty((16, N), dtype=torch.bfloat16, device="cuda:0")
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rc = lib.dflash_qmm_m16_static(_ptr(d.x), _ptr(d.w), _ptr(d.scales), _ptr(d.biases), _ptr(y_cap), K, N, 64,
+                                           nat.BF16, nat.BF16, nat.QMM_MMA2BIG_PIPE, 8, nat.QMM_KERNEL_AUTO,
+                                           ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+            nat.check(rc, "dflash_qmm_m16_static under capture")
+    torch.cuda.current_stream().wait_stream(side)
+    rc = lib.dflash_qmm_m16(_ptr(d.x), _ptr(d.w), _ptr(d.scales), _ptr(d.biases), _ptr(y_ref), _ptr(ws), ws.numel(),
+                            K, N, 64, nat.BF16, nat.BF16, nat.QMM_MMA2BIG_PIPE, 8, nat.QMM_KERNEL_AUTO,
+                            ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    nat.check(rc, "dflash_qmm_m16")
+    torch.cuda.synchronize()
+    for replay in range(3):
+        y_cap.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_cap.view(torch.int16), y_ref.view(torch.int16)), replay
