@@ -20,8 +20,9 @@
 //    whatever x holds, and the launch ends normally.
 //  * an epilogue turns a gate/up pair into the MLP's hidden activation inside the launch:
 //    the matrix holds gate rows then up rows, a row block takes 64 rows of each, and the
-//    workgroup that finishes it stores silu(gate) * up (each factor rounded to the activation
-//    type first, as separate operators would) - which the down projection then waits for.
+//    workgroup that finishes it stores silu(gate) * up (every operator of x * sigmoid(x) * up
+//    rounded to the activation type, as separate operators would) - which the down projection
+//    then waits for.
 //
 // Everything else - units of 128 rows x 256 k, 8 worker + 4 loader waves, direct-to-LDS loads
 // into a ring, hand-written LDS reads, bare barriers - is the streaming kernel's, see there.
@@ -209,10 +210,14 @@ __device__ unsigned long long g_stamps[64][13][kStampSlots];
 template <bool FP16>
 __device__ __forceinline__ float silu_mul(float g, float u) {
   using A = Act<FP16>;
-  // each factor as the activation type would hold it between separate operators
+  // silu(g) * u as the array operators x * sigmoid(x) and * give it: the factors as the
+  // activation type holds them between the projections and the activation, then the sigmoid,
+  // its product with g and the product with u each rounded to that type (the last one by the
+  // store).  Same form as the GatedDeltaNet glue kernels use.
   g = A::to_f32(A::from_f32(g));
   u = A::to_f32(A::from_f32(u));
-  const float s = A::to_f32(A::from_f32(g / (1.0f + __expf(-g))));
+  const float sig = A::to_f32(A::from_f32(1.0f / (1.0f + expf(-g))));
+  const float s = A::to_f32(A::from_f32(g * sig));
   return s * u;
 }
 

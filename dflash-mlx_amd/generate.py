@@ -21,6 +21,7 @@ import torch
 
 from .engine import HybridGDNEngine, _BaseEngine
 from .runtime import _match_acceptance_length
+from .verify_qmm import raise_on_device_errors
 
 TargetFn = Callable[[torch.Tensor, List[Any]], torch.Tensor]
 DraftFn = Callable[[torch.Tensor, int, torch.Tensor], torch.Tensor]
@@ -67,6 +68,8 @@ def generate_speculative(target: TargetFn, draft: DraftFn, target_cache: List[An
         verify_logits = target(verify_token_ids[None], target_cache)
         posterior = greedy_tokens(verify_logits[0])
         acceptance_len = int(_match_acceptance_length(verify_token_ids[1:], posterior[:-1]).item())
+        if device.type == "cuda":
+            raise_on_device_errors(device)  # the cycle's one wait for the device: a kernel that gave up a wait says so here
         if acceptance_history is not None:
             acceptance_history.append(acceptance_len)
         commit_count = 1 + acceptance_len

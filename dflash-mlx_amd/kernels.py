@@ -221,9 +221,27 @@ def replay_launch(tape: torch.Tensor, k: torch.Tensor, g: torch.Tensor, state_in
         conv_prev, qkv, conv_out = conv
         if mask is not None or not (qkv.is_contiguous() and conv_out.is_contiguous()) or int(qkv.shape[-2]) != T_alloc:
             raise ValueError("conv windows ride along only without a mask, contiguous, with the tape's row count")
+        # The kernel writes slots * keep rows of C elements into conv_out and reads slots * T_alloc
+        # rows of qkv (and slots * keep of conv_prev): every one of those extents, the element
+        # type and the device are checked here, since nothing behind this point can.
+        keep, C = int(conv_out.shape[-2]), int(qkv.shape[-1])
+
+        def leading(t: torch.Tensor) -> int:
+            n = 1
+            for d in t.shape[:-2]:
+                n *= int(d)
+            return n
+
+        if (qkv.ndim < 3 or conv_out.ndim < 3 or int(conv_out.shape[-1]) != C or conv_out.dtype != qkv.dtype
+                or leading(qkv) != slots or leading(conv_out) != slots
+                or not (qkv.device == conv_out.device == state_in.device)):
+            raise ValueError(f"conv windows: qkv must be [slots.., {T_alloc}, C] and conv_out [slots.., keep, C] with "
+                             f"{slots} slots, one element type, on {state_in.device}; got {tuple(qkv.shape)} {qkv.dtype} "
+                             f"on {qkv.device} and {tuple(conv_out.shape)} {conv_out.dtype} on {conv_out.device}")
         if conv_prev is not None and not (conv_prev.is_contiguous() and conv_prev.dtype == qkv.dtype
-                                          and conv_prev.shape[-2:] == conv_out.shape[-2:]):
-            raise ValueError("conv_prev must be contiguous, [.., keep, C], in the dtype of qkv")
+                                          and conv_prev.ndim >= 3 and tuple(conv_prev.shape[-2:]) == (keep, C)
+                                          and leading(conv_prev) == slots and conv_prev.device == qkv.device):
+            raise ValueError("conv_prev must be contiguous, [slots.., keep, C], in the dtype of qkv, on its device")
         rc = lib.dflash_rollback_layer(
             tape.data_ptr(), k.data_ptr(), g.data_ptr(), state_in.data_ptr(), state_out.data_ptr(),
             None if conv_prev is None else conv_prev.data_ptr(), qkv.data_ptr(), conv_out.data_ptr(),

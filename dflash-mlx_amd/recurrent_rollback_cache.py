@@ -78,6 +78,10 @@ class RecurrentRollbackCache:
         self._snapshot = None
         self._arena: Optional["RollbackArena"] = None
         self._layer = -1
+        # batched generation (dflash_mlx/recurrent_rollback_cache.py:18-19): per-row lengths of a
+        # right-padded block, or per-row left padding, as `prepare` / a batching loop sets them
+        self.lengths: Optional[torch.Tensor] = None
+        self.left_padding: Optional[torch.Tensor] = None
 
     def __getitem__(self, idx: int):
         return self.cache[idx]
@@ -96,6 +100,76 @@ class RecurrentRollbackCache:
     @property
     def nbytes(self):
         return sum(c.numel() * c.element_size() for c in self.cache if c is not None)
+
+    # -- batch-cache protocol of the generation loops (recurrent_rollback_cache.py:46-94) ------
+    # Rows of a batch come and go between steps, never inside a verify step: what a rollback
+    # needs (snapshot, tapes) describes the batch as it was, so every change of the batch drops
+    # it, and a cache that was a view into a RollbackArena stands on tensors of its own afterwards.
+    def _leave_arena(self) -> None:
+        self.clear_transients()
+        self._arena, self._layer = None, -1
+
+    def filter(self, batch_indices) -> None:
+        """Keep the rows ``batch_indices`` (in that order)."""
+        self._leave_arena()
+        self.cache = [c[batch_indices] if c is not None else None for c in self.cache]
+        if self.lengths is not None:
+            self.lengths = self.lengths[batch_indices]
+        if self.left_padding is not None:
+            self.left_padding = self.left_padding[batch_indices]
+
+    def extend(self, other: "RecurrentRollbackCache") -> None:
+        """Append the rows of ``other``."""
+        if len(self.cache) != len(other.cache):
+            raise ValueError(f"caches of {len(self.cache)} and {len(other.cache)} entries cannot be joined")
+        self._leave_arena()
+
+        def joined(mine, theirs):
+            if mine is None:
+                return theirs
+            if theirs is None:
+                return mine
+            return torch.cat([mine, theirs], dim=0)
+
+        self.cache = [joined(a, b) for a, b in zip(self.cache, other.cache)]
+
+    def extract(self, idx: int) -> "RecurrentRollbackCache":
+        """A cache of its own holding row ``idx`` (batch dimension kept)."""
+        one = RecurrentRollbackCache(len(self.cache), conv_kernel_size=self.conv_kernel_size)
+        one.cache = [c[idx:idx + 1] if c is not None else None for c in self.cache]
+        return one
+
+    def prepare(self, lengths=None, **kwargs) -> None:
+        del kwargs
+        if lengths is None:
+            self.lengths = None
+            return
+        device = next((c.device for c in self.cache if c is not None), None)
+        self.lengths = torch.as_tensor(lengths, device=device)
+
+    def finalize(self) -> None:
+        self.lengths = None
+        self.left_padding = None
+        self.clear_transients()
+
+    def advance(self, n: int) -> None:
+        if self.lengths is not None:
+            self.lengths = self.lengths - n
+        if self.left_padding is not None:
+            self.left_padding = self.left_padding - n
+
+    def make_mask(self, n: int):
+        """[B, n] bool, true where a position of the next ``n`` holds a token; None without padding."""
+        ref = self.left_padding if self.left_padding is not None else self.lengths
+        if ref is None:
+            return None
+        pos = torch.arange(n, device=ref.device)
+        if self.left_padding is not None:
+            return pos >= self.left_padding[:, None]
+        return pos < self.lengths[:, None]
+
+    def empty(self) -> bool:
+        return self.cache[0] is None
 
     # -- rollback state machine (recurrent_rollback_cache.py:96-171)
     def checkpoint(self) -> None:

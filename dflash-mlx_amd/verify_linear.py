@@ -188,7 +188,7 @@ def silu_gate_up(parent: nn.Module, x: torch.Tensor, names: Tuple[str, str] = ("
         if group.names == tuple(names) and group.applies(parent, x) and group.silu_mul_ready(x):
             return group.silu_mul(x)
     gate, up = shared_input_outputs(parent, names, x)
-    return torch.nn.functional.silu(gate) * up
+    return (gate * torch.sigmoid(gate)) * up   # x * sigmoid(x): the operators the epilogue follows, one rounding each
 
 
 def shared_input_outputs(parent: nn.Module, names: Sequence[str], x: torch.Tensor) -> Tuple[torch.Tensor, ...]:

@@ -88,6 +88,30 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
     return ws
 
 
+def raise_on_device_errors(device: Optional[torch.device] = None) -> None:
+    """Call where the host synchronises with the device anyway (the read-back of the acceptance
+    length in a speculative cycle): a bounded wait inside a qmm kernel that gave up - a chained
+    projection waiting for its input, the streaming kernel's adding workgroup waiting for partial
+    tiles - leaves a word in the workspace and wrong outputs behind, and nothing else tells the
+    caller.  Reads that word of every workspace of ``device`` (all devices if None; each read waits
+    for the device); on a non-zero word the workspace is zero-filled again, as its contract asks,
+    and ``NativeLibraryError`` raised."""
+    for (index, stream), ws in list(_WORKSPACES.items()):
+        if device is not None and device.index is not None and device.index != index:
+            continue
+        word = int(ws[_native.QMM_ERROR_OFFSET:_native.QMM_ERROR_OFFSET + 4].view(torch.int32).item()) & 0xFFFFFFFF
+        if word == 0:
+            continue
+        ws.zero_()
+        if word & 0x80000000:
+            what = f"the streaming kernel gave up waiting for the partial tiles of row block {word & 0x3FFFFFFF}"
+        else:
+            what = f"projection {word - 1} of a chained launch gave up waiting for its input"
+        raise _native.NativeLibraryError(
+            f"qmm workspace of device {index}, stream {stream:#x}: {what}; the outputs of that launch and of "
+            "everything computed from them are undefined (is the device shared with a long-running kernel?)")
+
+
 def _require_operands(who: str, K: int, N: int, group_size: int, w: torch.Tensor, scales: torch.Tensor,
                       biases: torch.Tensor, device: torch.device, lead: Tuple[int, ...] = ()) -> None:
     """The kernels read what K, N and the group size say: weights of any other extent, word size
@@ -302,6 +326,12 @@ class QmmChain:
 
     def clear_error(self) -> None:
         self._ws[_native.QMM_CHAIN_ERROR_OFFSET:_native.QMM_CHAIN_ERROR_OFFSET + 4].zero_()
+
+    def check(self) -> None:
+        """Waits for the device and raises ``NativeLibraryError`` if a wait of the last launches
+        was given up (``raise_on_device_errors`` for this chain's device).  A chain with
+        projections that read one another should be checked before its outputs are trusted."""
+        raise_on_device_errors(self._device)
 
 
 class PackedWeights:

@@ -149,8 +149,9 @@ int dflash_qmm_m16_static(const void* x, const uint32_t* w_q, const void* scales
  *               problem j's output has been stored; its weights stream regardless.
  *   epilogue    DFLASH_QMM_EPILOGUE_NONE, or DFLASH_QMM_EPILOGUE_SILU_MUL: w_q, scales, biases hold
  *               N/2 gate rows followed by N/2 up rows and y is [16, N/2],
- *                   y = round(round(silu(round(gate))) * round(up))     (round: to act_dtype),
- *               what `silu(gate_proj(x)) * up_proj(x)` of an MLP gives operator by operator.
+ *                   g = round(gate), y = round(round(g * round(sigmoid(g))) * round(up))
+ *               (round: to act_dtype), what `silu(gate_proj(x)) * up_proj(x)` of an MLP gives
+ *               operator by operator with silu(x) = x * sigmoid(x).
  * Requirements: 1 <= count <= DFLASH_QMM_CHAIN_MAX; group_size 64; K % 1024 == 0; N % 16 == 0
  * (N % 128 == 0 with an epilogue); pointers 16-byte aligned; workspace of
  * dflash_qmm_m16_chain_workspace_bytes(...) bytes under the rules of dflash_qmm_m16 (zero-filled

@@ -65,6 +65,30 @@ def test_recurrence_wrappers(native_lib):
             tape[:, :, :2], k, gate, state, steps=2)                               # tape of two heads, rows read in place
     assert K.tape_replay_kernel(tape, k, gate, state).shape == state.shape
 
+    # replay with the conv windows riding along: the kernel writes slots * keep rows of C elements
+    B, T, C = int(tape.shape[0]), int(tape.shape[1]), 24
+    qkv = torch.randn((B, T, C), device=DEV).to(torch.bfloat16)
+    prev = torch.randn((B, 3, C), device=DEV).to(torch.bfloat16)
+    out = torch.empty((B, 3, C), dtype=torch.bfloat16, device=DEV)
+    s_in, s_out = state.contiguous(), torch.empty_like(state)
+
+    def launch(conv):
+        K.replay_launch(tape.contiguous(), k.contiguous(), gate.contiguous(), s_in, s_out, steps=2, T_alloc=T, slots=B, conv=conv)
+
+    launch((prev, qkv, out))
+    torch.cuda.synchronize()
+    assert torch.equal(out, torch.cat([prev, qkv], dim=1)[:, 2:5])
+    for bad in ((prev, qkv, out.float()),                                   # another element type
+                (prev, qkv, torch.empty((B, 3, C - 8), dtype=torch.bfloat16, device=DEV)),   # narrower rows
+                (prev, qkv, torch.empty((B + 1, 3, C), dtype=torch.bfloat16, device=DEV)),   # more slots than the launch
+                (prev, torch.cat([qkv, qkv]), out),                         # qkv of more slots
+                (prev, qkv, out.cpu()),                                     # host memory
+                (prev[:, :2].contiguous(), qkv, out),                       # conv_prev of another window
+                (torch.cat([prev, prev]), qkv, out),                        # conv_prev of more slots
+                (prev.cpu(), qkv, out)):
+        with pytest.raises(ValueError):
+            launch(bad)
+
 
 def test_attention_wrapper_declines(native_lib):
     q = torch.randn((1, 4, 16, 128), device=DEV).to(torch.bfloat16)

@@ -15,6 +15,8 @@ import numpy as np
 import pytest
 import torch
 
+from dflash_mlx_amd.gdn_layer import silu_ops
+
 import dflash_mlx_amd._native as nat
 from dflash_mlx_amd import verify_qmm as VQ
 from dflash_mlx_amd.workloads import make_qmm_case
@@ -145,7 +147,7 @@ def test_mlp_in_one_launch(native_lib, c_oracle, K, I):
         # the gate/up pair does, so g and u may differ in their last bit where sums cancel - equal
         # on nearly all elements, and everywhere within the bar on the exact product below
         g, u = _separate(x, gate), _separate(x, up)
-        want_h = torch.nn.functional.silu(g) * u
+        want_h = silu_ops(g) * u
         assert float((h != want_h).float().mean()) <= 2e-3
         ge, ue = (_exact(c_oracle, c, x).astype(np.float64) for c in (gate, up))
         exact = ge / (1.0 + np.exp(-ge)) * ue
@@ -174,7 +176,20 @@ def test_bounded_wait_gives_up_and_the_launch_still_ends(native_lib):
     assert word in (0, 2)
     y0 = _separate(cases[0].x, cases[0])
     assert torch.equal(hasty.outputs[0].view(torch.int16), y0.view(torch.int16))   # nothing waits for x0
-    hasty.clear_error()
+    if word:
+        with pytest.raises(nat.NativeLibraryError, match="projection 1 of a chained launch"):
+            hasty.check()                          # says so, and hands the workspace back zero-filled
+        assert hasty.error_word() == 0
+    else:
+        hasty.check()
+    # the same for a word as the streaming kernel leaves it (its waits cannot be made to expire
+    # from the host: written by hand)
+    ws = VQ._workspace(cases[0].x.device, nat.raw_stream(cases[0].x.device), 1)
+    ws[nat.QMM_ERROR_OFFSET:nat.QMM_ERROR_OFFSET + 4].view(torch.int32).fill_(-2147483648 + 7)
+    with pytest.raises(nat.NativeLibraryError, match="row block 7"):
+        VQ.raise_on_device_errors(cases[0].x.device)
+    VQ.raise_on_device_errors()                    # cleared: nothing to report
+    assert int((ws != 0).sum()) == 0
     patient = VQ.QmmChain([p0, p1])
     ys = patient()
     torch.cuda.synchronize()
@@ -241,7 +256,7 @@ def test_hidden_activation_of_a_gated_mlp_in_one_launch(native_lib, c_oracle, mo
         assert h.shape == (1, 16, I) and all(h.data_ptr() != o.data_ptr() for o in outs)
         outs.append(h)
         g, u = VL.shared_input_outputs(model.mlp, ("gate_proj", "up_proj"), x)
-        ops = torch.nn.functional.silu(g) * u
+        ops = silu_ops(g) * u
         assert float((h.reshape(16, I) != ops).float().mean()) <= 2e-3
         ge, ue = (_exact(c_oracle, c, x).astype(np.float64) for c in (gate, up))
         exact = ge / (1.0 + np.exp(-ge)) * ue
@@ -251,7 +266,7 @@ def test_hidden_activation_of_a_gated_mlp_in_one_launch(native_lib, c_oracle, mo
     # a block that is not a verify block: array operators on the members' own outputs
     x5 = torch.randn(5, K).to(torch.bfloat16).to(DEV)
     assert torch.equal(VL.silu_gate_up(model.mlp, x5),
-                       torch.nn.functional.silu(model.mlp.gate_proj(x5)) * model.mlp.up_proj(x5))
+                       silu_ops(model.mlp.gate_proj(x5)) * model.mlp.up_proj(x5))
     assert launches == [1, 1, 1]
     # rebinding is refused where it would break the chain, or where the tensor does not fit
     small = _cases([(1024, 64), (64, 32)], 881)[0]

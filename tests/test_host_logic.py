@@ -6,6 +6,8 @@ import itertools
 import numpy as np
 import pytest
 import torch
+
+from dflash_mlx_amd.gdn_layer import silu_ops
 import torch.nn as nn
 
 import dflash_mlx_amd._native as nat
@@ -308,6 +310,69 @@ def test_rollback_cache_state_machine_on_host():
         _tape_replay_ops(t(tape)[:, :, :3], t(k), t(g)[:, :, :3], t(S0)[:, :3])
 
 
+def test_rollback_cache_batch_protocol():
+    """filter / extend / extract / prepare / finalize / advance / make_mask / empty, as the batched
+    generation loops of mlx-lm use them on the reference class
+    (dflash_mlx/recurrent_rollback_cache.py:18-19, 46-94)."""
+    conv = torch.arange(4 * 3 * 5, dtype=torch.float32).reshape(4, 3, 5)
+    state = torch.arange(4 * 2 * 3 * 8, dtype=torch.float32).reshape(4, 2, 3, 8)
+    cache = RecurrentRollbackCache(size=2, conv_kernel_size=4)
+    assert cache.empty() and cache.lengths is None and cache.left_padding is None
+    assert cache.make_mask(5) is None
+    cache[0], cache[1] = conv.clone(), state.clone()
+    assert not cache.empty()
+
+    # lengths of a right-padded block: true where a row still has tokens
+    cache.prepare(lengths=[3, 5, 0, 2])
+    assert torch.equal(cache.make_mask(4), torch.tensor([[1, 1, 1, 0], [1, 1, 1, 1], [0, 0, 0, 0], [1, 1, 0, 0]]).bool())
+    cache.advance(2)
+    assert cache.lengths.tolist() == [1, 3, -2, 0]
+    assert torch.equal(cache.make_mask(2), torch.tensor([[1, 0], [1, 1], [0, 0], [0, 0]]).bool())
+    # left padding wins over lengths: true from the first real token on
+    cache.left_padding = torch.tensor([0, 2, 1, 4])
+    assert torch.equal(cache.make_mask(3), torch.tensor([[1, 1, 1], [0, 0, 1], [0, 1, 1], [0, 0, 0]]).bool())
+    cache.advance(1)
+    assert cache.left_padding.tolist() == [-1, 1, 0, 3] and cache.lengths.tolist() == [0, 2, -3, -1]
+
+    # a change of the batch drops what a rollback would need, and keeps rows in the order asked for
+    cache.arm_rollback()
+    cache.record_tape(tape=torch.zeros(4, 2, 2, 3), k=torch.zeros(4, 2, 1, 8), g=torch.ones(4, 2, 2), qkv=torch.zeros(4, 2, 5))
+    cache.filter(torch.tensor([2, 0]))
+    assert cache._snapshot is None and cache._tape is None and not cache._armed
+    assert torch.equal(cache[0], conv[[2, 0]]) and torch.equal(cache[1], state[[2, 0]])
+    assert cache.lengths.tolist() == [-3, 0] and cache.left_padding.tolist() == [0, -1]
+    cache.rollback(0)   # nothing armed any more: a no-op
+    assert torch.equal(cache[1], state[[2, 0]])
+
+    one = cache.extract(1)
+    assert isinstance(one, RecurrentRollbackCache) and one.conv_kernel_size == 4
+    assert torch.equal(one[0], conv[0:1]) and torch.equal(one[1], state[0:1]) and one.lengths is None
+
+    other = RecurrentRollbackCache(size=2, conv_kernel_size=4)
+    other[0], other[1] = conv[3:4].clone(), state[3:4].clone()
+    cache.extend(other)
+    assert torch.equal(cache[0], conv[[2, 0, 3]]) and torch.equal(cache[1], state[[2, 0, 3]])
+    fresh = RecurrentRollbackCache(size=2)
+    fresh.extend(other)   # an empty cache takes the other's rows
+    assert torch.equal(fresh[1], state[3:4])
+    with pytest.raises(ValueError):
+        cache.extend(RecurrentRollbackCache(size=3))
+
+    cache.arm_rollback()
+    cache.finalize()
+    assert cache.lengths is None and cache.left_padding is None and cache._snapshot is None and not cache._armed
+    cache.prepare(lengths=None)
+    assert cache.lengths is None
+
+    # a cache that is a view into an arena stands on its own tensors after the batch changed
+    from dflash_mlx_amd.recurrent_rollback_cache import RollbackArena
+    arena = RollbackArena(2, batch=3, max_steps=4, Hk=1, Hv=2, Dk=32, Dv=4, conv_dim=6, device="cpu")
+    view = arena.caches()[1]
+    assert view._arena is arena
+    view.filter(torch.tensor([1]))
+    assert view._arena is None and view[1].shape[0] == 1 and view[1].data_ptr() != arena.state[0, 1].data_ptr()
+
+
 @pytest.mark.parametrize("g_per_dk", [False, True])
 def test_array_op_forms_match_the_oracle(g_per_dk):
     """The torch array-op forms of forward-with-tape and replay (what host tensors and
@@ -429,7 +494,7 @@ def test_silu_gate_up_on_the_host_is_the_array_operators(monkeypatch):
     install_verify_linears(m)
     x = torch.randn(16, 512).to(torch.bfloat16)
     m.mlp.up_proj = VerifyQuantizedLinear.from_quantized(QuantizedLinear.from_linear(_mk_linear(512, 256), 64, 4))
-    want = torch.nn.functional.silu(m.mlp.gate_proj(x)) * m.mlp.up_proj(x)
+    want = silu_ops(m.mlp.gate_proj(x)) * m.mlp.up_proj(x)
     assert torch.equal(VL.silu_gate_up(m.mlp, x), want)
     assert fuse_shared_input_linears(m) >= 1
     group = m.mlp.gate_proj._shared_input[0]
