@@ -501,7 +501,7 @@ def test_silu_gate_up_on_the_host_is_the_array_operators(monkeypatch):
     assert group.bounds == [(0, 256), (256, 512)] and not group.silu_mul_ready(x)      # host tensor
     assert torch.equal(VL.silu_gate_up(m.mlp, x), want)
     assert torch.equal(VL.silu_gate_up(m.odd, torch.ones(3, 384).to(torch.bfloat16)),
-                       torch.nn.functional.silu(m.odd.gate_proj(torch.ones(3, 384).to(torch.bfloat16))) *
+                       silu_ops(m.odd.gate_proj(torch.ones(3, 384).to(torch.bfloat16))) *
                        m.odd.up_proj(torch.ones(3, 384).to(torch.bfloat16)))
 
 
