@@ -40,7 +40,7 @@ MEASURED_TRAFFIC_BYTES = {"27b": 44.32e6, "9b": None}
 TRAFFIC_SOURCE = "profiles/qmm_stream_kernel_27b_stack_pmc.txt"
 
 
-LEGS = ("other_stack", "gate_up", "packed", "chain", "mlp", "single", "moe", "replay", "forward", "sdpa", "glue")
+LEGS = ("other_stack", "dependent", "gate_up", "packed", "chain", "mlp", "single", "moe", "replay", "forward", "sdpa", "glue")
 
 
 def log(*a):
@@ -285,6 +285,90 @@ def bench_mlp_chain(stack: str, steps: int, warmup: int, device: str):
                          frac_hbm=nbytes / (ev_ms / steps * 1e-3) / HBM_PEAK)
         del graph
     del chains, mlps, ref, got
+    torch.cuda.empty_cache()
+    return res
+
+
+def bench_dependent_layers(stack: str, steps: int, warmup: int, device: str):
+    """The stack in the order a model runs it (dflash_mlx/runtime.py:779-821, the layer loop of the
+    verify forward): every launch consumes what the one before produced.  Per layer: the joined
+    q/k/v projection of the layer's input; a copy of the first `hidden` columns of its output
+    stands in for the attention between it and o_proj; o_proj; gate_proj and up_proj as one
+    launch with the silu * mul epilogue on o_proj's output; down_proj on the hidden activation;
+    its output is the next layer's input.  Four qmm launches and one small copy per layer, none
+    of which can start before the previous one has ended.  Scales and biases are shrunk so that
+    activations keep their magnitude from layer to layer; the bytes moved are the headline's minus
+    the second read of x by up_proj."""
+    import torch
+
+    from dflash_mlx_amd.verify_qmm import ChainProblem, QmmChain, verify_matmul
+    from dflash_mlx_amd.workloads import qmm_algorithmic_bytes, stack_linears
+
+    linears, layers, _ = stack_linears(stack)
+    dims = {name: (K, N) for name, K, N in linears}
+    H = dims["o_proj"][0]
+    calls = build_stack(stack, device, join_gate_up=True)   # qkv, o, gate/up joined, down per layer
+    per_layer = len(linears) - 1
+    total_bytes = sum(qmm_algorithmic_bytes(c.K, c.N)[1] for c in calls)
+    x0 = calls[0].x
+
+    def unit_gain(c, x, halves=False):
+        """Shrinks the scales and biases of c so that its output on x has unit rms (zero-mean
+        weights: the benchmark's bias of -8 scale leaves a mean that would add up over K)."""
+        c.biases.copy_(-7.5 * c.scales)
+        y = verify_matmul(x, c.w, c.scales, c.biases).float()
+        parts = (y[:, :c.N // 2], y[:, c.N // 2:]) if halves else (y,)
+        for i, part in enumerate(parts):
+            rows = slice(i * c.N // len(parts), (i + 1) * c.N // len(parts))
+            rms = float(part.pow(2).mean().sqrt())
+            c.scales[rows] /= rms
+            c.biases[rows] /= rms
+        return verify_matmul(x, c.w, c.scales, c.biases)
+
+    x = x0
+    for layer in range(layers):  # once, before anything is timed
+        qkv, o, gu, down = calls[layer * per_layer:(layer + 1) * per_layer]
+        a = unit_gain(qkv, x)[:, :H].contiguous()
+        both = unit_gain(gu, unit_gain(o, a), halves=True)
+        g, u = both[:, :gu.N // 2], both[:, gu.N // 2:]
+        x = unit_gain(down, (g * torch.sigmoid(g)) * u)
+    gate_up = []
+    for layer in range(layers):
+        c = calls[layer * per_layer + 2]
+        gate_up.append(QmmChain([ChainProblem(torch.empty((16, c.K), dtype=x0.dtype, device=device), c.w, c.scales,
+                                              c.biases, epilogue="silu_mul")]))
+
+    def one_pass():
+        x = x0
+        for layer in range(layers):
+            qkv, o, gu, down = calls[layer * per_layer:(layer + 1) * per_layer]
+            y = verify_matmul(x, qkv.w, qkv.scales, qkv.biases)
+            a = y[:, :H].contiguous()
+            o_out = verify_matmul(a, o.w, o.scales, o.biases)
+            h = torch.empty((16, gu.N // 2), dtype=x0.dtype, device=device)
+            chain = gate_up[layer]
+            chain.rebind(0, x=o_out, out=h)
+            chain()
+            x = verify_matmul(h, down.w, down.scales, down.biases)
+        return x
+
+    eager = one_pass()
+    torch.cuda.synchronize()
+    if not bool(torch.isfinite(eager.float()).all()):
+        raise RuntimeError("dependent layers: activations left the finite range")
+    graph, captured = capture(one_pass)
+    for r in range(2):
+        graph.replay()
+        torch.cuda.synchronize()
+        if not torch.equal(captured, eager):
+            raise RuntimeError(f"dependent layers: graph replay {r} differs from the eager result")
+    for _ in range(warmup):
+        graph.replay()
+    wall_ms, ev_ms = time_region(graph.replay, steps)
+    res = dict(launches_per_layer=per_layer, layers=layers, ms_per_step=wall_ms / steps,
+               us_per_layer=ev_ms / steps / layers * 1e3, total_bytes=total_bytes,
+               frac_hbm=total_bytes / (ev_ms / steps * 1e-3) / HBM_PEAK)
+    del graph, captured, eager, calls, gate_up
     torch.cuda.empty_cache()
     return res
 
@@ -808,6 +892,11 @@ def main() -> int:
         extra[f"stack_{other}"] = dict(ms_per_step=round(o["ms_per_step"], 4),
                                        weight_gbps=round(o["weight_gbps"], 1),
                                        frac_hbm=round(o["total_bytes"] / (o["event_ms_per_step"] * 1e-3) / HBM_PEAK, 4))
+    if "dependent" in legs:
+        dep = bench_dependent_layers(args.workload, args.steps, args.warmup, device)
+        log(f"[bench] {args.workload} stack, every launch waiting for the one before: {dep['ms_per_step']:.3f} ms/step, "
+            f"{dep['us_per_layer']:.2f} us/layer, {dep['frac_hbm']:.3f} of peak")
+        extra[f"stack_{args.workload}_dependent_layer"] = rnd(dep)
     stack_variants = []
     if "gate_up" in legs:
         stack_variants.append(("gate_up_in_one_launch", dict(join_gate_up=True)))
