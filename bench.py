@@ -31,13 +31,41 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
-# HBM bytes per launch of the qmm kernel on each stack (mean over its launches).  Not measured
-# by this file: counters need the profiler.  The figure is copied from the two rocprofv3 --pmc
-# runs (FETCH_SIZE, WRITE_SIZE) of this file summarised in TRAFFIC_SOURCE, scaled by the same
-# counters' reading for a 1 GiB copy (x2.000 / x1.000), and is reported under that label;
-# None where no such run exists for the current kernel.
-MEASURED_TRAFFIC_BYTES = {"27b": 44.32e6, "9b": None}
-TRAFFIC_SOURCE = "profiles/qmm_stream_kernel_27b_stack_pmc.txt"
+# HBM bytes per launch of the qmm kernel (mean over the launches of a stack) cannot be measured by
+# this file: counters need the profiler.  The figure is read from the text summary of the two
+# rocprofv3 --pmc runs of this file (FETCH_SIZE, WRITE_SIZE, scaled by the same counters' reading
+# for a 1 GiB copy) kept under profiles/, which also states the SHA-256 of the kernel's source
+# files as they were when the counters were taken.  If the sources have changed since, the figure
+# describes another kernel and is not reported.
+TRAFFIC_PROFILES = {"27b": "profiles/qmm_stream_kernel_27b_stack_pmc.txt"}
+KERNEL_SOURCES = ("dflash-mlx_amd/csrc/qmm_m16_stream.hip", "dflash-mlx_amd/csrc/qmm_stream_device.h")
+
+
+def kernel_sources_sha256() -> str:
+    import hashlib
+
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def measured_traffic(workload: str):
+    """(bytes per launch or None, where the figure comes from or why there is none)."""
+    import re
+
+    rel = TRAFFIC_PROFILES.get(workload)
+    if rel is None or not os.path.exists(os.path.join(ROOT, rel)):
+        return None, "no counter summary for this workload"
+    text = open(os.path.join(ROOT, rel)).read()
+    sha = re.search(r"^kernel_sources_sha256:\s*([0-9a-f]{64})", text, flags=re.M)
+    traffic = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", text, flags=re.M)
+    if not sha or not traffic:
+        return None, f"{rel} does not state the kernel sources it was taken with"
+    if sha.group(1) != kernel_sources_sha256():
+        return None, f"{rel} was taken with other kernel sources"
+    return float(traffic.group(1)), rel
 
 
 LEGS = ("other_stack", "dependent", "gate_up", "packed", "chain", "mlp", "single", "moe", "replay", "forward", "sdpa", "glue")
@@ -849,6 +877,8 @@ def main() -> int:
     ap.add_argument("--packed-weights", action="store_true",
                     help="headline stack through verify_matmul_packed (weights stored in the streaming "
                          "kernel's order); off by default: the headline uses the reference's operands")
+    ap.add_argument("--kernel-sources-sha256", action="store_true",
+                    help="print the hash a counter summary under profiles/ has to state, and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run three 1 GiB device-to-device copies (a kernel of known traffic, "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings) and exit")
@@ -857,6 +887,10 @@ def main() -> int:
         print("bench.py measures one GPU: the verify hot path is a single-device path and this "
               "build has no multi-GPU leg; run with --gpus 1", file=sys.stderr)
         return 2
+
+    if args.kernel_sources_sha256:
+        print(kernel_sources_sha256())
+        return 0
 
     import torch
 
@@ -922,6 +956,11 @@ def main() -> int:
             log(f"[bench] {args.workload} stack, {n_layers} layer(s) per chained launch, gate/up as one problem: "
                 f"{ch['ms_per_step']:.3f} ms/step, {ch['us_per_layer']:.2f} us/layer")
             extra[f"stack_{args.workload}_chained_{n_layers}_layer_per_launch_gate_up_as_one_problem"] = rnd(ch)
+        other = "9b" if args.workload == "27b" else "27b"
+        ch = bench_qmm_chain_stack(other, args.steps, args.warmup, device, layers_per_launch=3, join_gate_up=True)
+        log(f"[bench] {other} stack, 3 layers per chained launch, gate/up as one problem: {ch['ms_per_step']:.3f} ms/step, "
+            f"{ch['frac_hbm']:.3f} of peak")
+        extra[f"stack_{other}_chained_3_layer_per_launch_gate_up_as_one_problem"] = rnd(ch)
     if "mlp" in legs:
         mlp = bench_mlp_chain(args.workload, args.steps, args.warmup, device)
         extra[f"mlp_{args.workload}"] = {k: (rnd(v) if isinstance(v, dict) else round(v, 6)) for k, v in mlp.items()}
@@ -957,10 +996,11 @@ def main() -> int:
                                    for k, v in bench_gdn_glue(device, args.steps, args.warmup).items()}
 
     achieved = main_res["bytes_per_launch"] / (main_res["avg_launch_us"] * 1e-6) / 1e9
-    traffic = None if args.packed_weights else MEASURED_TRAFFIC_BYTES.get(args.workload)
+    traffic, traffic_source = (None, "packed weights: see the profile summary") if args.packed_weights \
+        else measured_traffic(args.workload)
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK / 1e9, unit="GB/s",
                     frac=round(achieved * 1e9 / HBM_PEAK, 4),
-                    traffic=traffic, traffic_source=TRAFFIC_SOURCE if traffic is not None else None,
+                    traffic=traffic, traffic_source=traffic_source,
                     kernel="qmm_stream_kernel", bytes_per_launch=round(main_res["bytes_per_launch"]),
                     avg_launch_us=round(main_res["avg_launch_us"], 3))
     cpu = None if args.skip_cpu else bench_cpu_baseline(args.workload)

@@ -198,6 +198,21 @@ def test_bf16_arrays_take_the_16_bit_matrix_cores_without_losing_a_bit(native_li
         got[dt] = (s, tape)
     assert _rel(_f64(got[torch.bfloat16][0]), _f64(got[torch.float16][0])) <= 5e-7
     assert _rel(_f64(got[torch.bfloat16][1]), _f64(got[torch.float16][1])) <= 5e-7
+    # Element by element: the two routes add the same exact products in another order, so a state
+    # entry may differ by the rounding of its partial sums, never by more.  Bar: one unit in the
+    # last place of fp32 per route, at the size of the entry's terms
+    #   S_T = c_T S_0 + sum_t (c_T / c_t) delta_t (x) k_t,   c_t = g_1 .. g_t
+    # (not at the size of the entry itself, which cancellation can make much smaller).
+    g64, k64, tape64, s064 = _f64(gate), _f64(k), ref[2], _f64(state)
+    B, T, Hv = g64.shape
+    rep = Hv // k64.shape[2]
+    c = np.cumprod(g64, axis=1)                                   # [B, T, Hv]
+    size = np.abs(c[:, -1][:, :, None, None] * s064)
+    for t in range(T):
+        w = (c[:, -1] / c[:, t])[:, :, None, None]
+        size += np.abs(w * tape64[:, t][:, :, :, None] * np.repeat(k64[:, t], rep, axis=1)[:, :, None, :])
+    diff = np.abs(_f64(got[torch.bfloat16][0]) - _f64(got[torch.float16][0]))
+    assert np.all(diff <= 2.0 ** -22 * size), float((diff / (2.0 ** -23 * size + 1e-300)).max())
 
 
 def test_errors_and_host_tensors(native_lib):
