@@ -199,10 +199,12 @@ def test_bf16_arrays_take_the_16_bit_matrix_cores_without_losing_a_bit(native_li
     assert _rel(_f64(got[torch.bfloat16][0]), _f64(got[torch.float16][0])) <= 5e-7
     assert _rel(_f64(got[torch.bfloat16][1]), _f64(got[torch.float16][1])) <= 5e-7
     # Element by element: the two routes add the same exact products in another order, so a state
-    # entry may differ by the rounding of its partial sums, never by more.  Bar: one unit in the
-    # last place of fp32 per route, at the size of the entry's terms
+    # entry may differ by the roundings of its partial sums, never by more.  An entry is a sum of
+    # T + 1 terms, each with a rounding of its own and the roundings of the delta it is made from:
     #   S_T = c_T S_0 + sum_t (c_T / c_t) delta_t (x) k_t,   c_t = g_1 .. g_t
-    # (not at the size of the entry itself, which cancellation can make much smaller).
+    # Bar: 8 units in the last place of fp32 at the size of the entry's terms (not at the size of
+    # the entry itself, which cancellation can make much smaller); 2.5 units are seen.  The third
+    # bf16 piece of a state entry left out would cost 2^-16 of a term, sixteen times the bar.
     g64, k64, tape64, s064 = _f64(gate), _f64(k), ref[2], _f64(state)
     B, T, Hv = g64.shape
     rep = Hv // k64.shape[2]
@@ -212,7 +214,7 @@ def test_bf16_arrays_take_the_16_bit_matrix_cores_without_losing_a_bit(native_li
         w = (c[:, -1] / c[:, t])[:, :, None, None]
         size += np.abs(w * tape64[:, t][:, :, :, None] * np.repeat(k64[:, t], rep, axis=1)[:, :, None, :])
     diff = np.abs(_f64(got[torch.bfloat16][0]) - _f64(got[torch.float16][0]))
-    assert np.all(diff <= 2.0 ** -22 * size), float((diff / (2.0 ** -23 * size + 1e-300)).max())
+    assert np.all(diff <= 2.0 ** -20 * size), float((diff / (2.0 ** -23 * size + 1e-300)).max())
 
 
 def test_errors_and_host_tensors(native_lib):
