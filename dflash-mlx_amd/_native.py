@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
@@ -22,7 +22,7 @@ QMM_CHAIN_MAX = 16                       # DFLASH_QMM_CHAIN_MAX
 QMM_ERROR_OFFSET = (16384 - 64 + 1) * 4        # DFLASH_QMM_ERROR_OFFSET
 QMM_CHAIN_ERROR_OFFSET = QMM_ERROR_OFFSET      # DFLASH_QMM_CHAIN_ERROR_OFFSET
 QMM_EPILOGUE_NONE, QMM_EPILOGUE_SILU_MUL = 0, 1
-OPT_GDN_STEP_BY_STEP, OPT_SDPA_SPLITS, OPT_SDPA_STAGED = 0, 1, 2  # DFLASH_OPT_*
+OPT_GDN_STEP_BY_STEP, OPT_SDPA_SPLITS, OPT_SDPA_STAGED, OPT_QMM_SPIN_LIMIT = 0, 1, 2, 3  # DFLASH_OPT_*
 
 
 class QmmProblem(ctypes.Structure):

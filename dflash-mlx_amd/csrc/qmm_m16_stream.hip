@@ -770,6 +770,8 @@ int launch_stream(stream::Params& p, bool gather, int grid, int act_dtype, int s
   using namespace stream;
   const bool a16 = act_dtype == DFLASH_FP16, s16 = sb_dtype == DFLASH_FP16;
   const bool chunk4 = p.K % (kUnitK * 4) == 0;
+  // (tests shorten the wait of the workgroups that add partial tiles to see them give up)
+  p.spin_limit = option(DFLASH_OPT_QMM_SPIN_LIMIT) > 0 ? option(DFLASH_OPT_QMM_SPIN_LIMIT) : kSpinLimit;
   const void* fn = gather ? stream_kernel_for<true>(a16, s16, chunk4) : stream_kernel_for<false>(a16, s16, chunk4);
   const int lds_bytes = gather ? kLdsBytesGather : kLdsBytes;
   // the attribute belongs to the device's copy of the kernel: once per device and kernel
@@ -811,7 +813,6 @@ int qmm_stream_launch(const void* x, const uint32_t* w, const void* scales, cons
                  workspace ? workspace_bytes : (size_t)0);
   p.status = (uint32_t*)workspace;
   p.partials = (float*)((char*)workspace + 64 * 1024);
-  p.spin_limit = kSpinLimit;
   return launch_stream(p, false, grid, act_dtype, sb_dtype, stream);
 }
 
@@ -859,7 +860,6 @@ int qmm_stream_packed_launch(const void* x, const void* w_img, const void* s_img
                  workspace ? workspace_bytes : (size_t)0);
   p.status = (uint32_t*)workspace;
   p.partials = (float*)((char*)workspace + 64 * 1024);
-  p.spin_limit = kSpinLimit;
   return launch_stream(p, false, grid, act_dtype, sb_dtype, stream);
 }
 
@@ -889,7 +889,6 @@ int qmm_stream_gather_launch(const void* x, const int32_t* expert_ids, const uin
                  workspace ? workspace_bytes : (size_t)0);
   p.status = (uint32_t*)workspace;
   p.partials = (float*)((char*)workspace + 64 * 1024);
-  p.spin_limit = kSpinLimit;
   return launch_stream(p, true, grid, act_dtype, sb_dtype, stream);
 }
 

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 13
+#define DFLASH_ABI_VERSION 14
 
 enum {
   DFLASH_OK = 0,
@@ -63,10 +63,19 @@ const char* dflash_last_error(void);
  *                                n ranges (fewer if a range would fall below one tile)
  *   DFLASH_OPT_SDPA_STAGED       1: dflash_sdpa_q16 without a mask keeps the kernel that stages its
  *                                tiles through registers (the one a mask always takes)
+ *   DFLASH_OPT_QMM_SPIN_LIMIT    n > 0: the streaming qmm kernel's workgroups that add partial tiles
+ *                                give up after n polls instead of 2^18 (tests of that path: the
+ *                                launch ends, the error word is set, results are unspecified)
  * dflash_set_option returns 0, or DFLASH_ERR_ARG for an unknown option or a negative value;
  * dflash_get_option returns the value, or DFLASH_ERR_ARG.
  */
-enum { DFLASH_OPT_GDN_STEP_BY_STEP = 0, DFLASH_OPT_SDPA_SPLITS = 1, DFLASH_OPT_SDPA_STAGED = 2, DFLASH_OPT_COUNT = 3 };
+enum {
+  DFLASH_OPT_GDN_STEP_BY_STEP = 0,
+  DFLASH_OPT_SDPA_SPLITS = 1,
+  DFLASH_OPT_SDPA_STAGED = 2,
+  DFLASH_OPT_QMM_SPIN_LIMIT = 3,
+  DFLASH_OPT_COUNT = 4
+};
 int dflash_set_option(int option, int value);
 int dflash_get_option(int option);
 

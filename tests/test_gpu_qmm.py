@@ -249,6 +249,34 @@ def test_every_kernel_hands_the_shared_workspace_back_zero_filled(verify_env, na
     _check_north_star(_f32(yc).astype(np.float64), _oracle_exact(c_oracle, c.to("cpu")))
 
 
+def test_adding_workgroup_that_gives_up_says_so_and_the_launch_ends(verify_env, native_lib):
+    """The wait of the streaming kernel's adding workgroups cut to two polls from the host (an
+    option of the library): the launch ends like any other, the workgroups that found a tile
+    missing leave the error word behind, `raise_on_device_errors` turns it into an exception and
+    zero-fills the workspace - late tiles may sit in it - and the next launch, with the wait at its
+    default, is right again.  5120 x 17408: 136 row blocks, each shared by two or three workgroups
+    that finish microseconds apart, so some of the 136 waits are cut short in any run."""
+    verify_env.setenv("DFLASH_QMM_KERNEL", "auto")
+    case = make_qmm_case(5120, 17408, 41).to(DEV)
+    good = VQ.verify_matmul(case.x, case.w, case.scales, case.biases)
+    torch.cuda.synchronize()
+    VQ.raise_on_device_errors(torch.device(DEV))                       # nothing to report
+    assert native_lib.dflash_set_option(nat.OPT_QMM_SPIN_LIMIT, 1) == 0
+    try:
+        VQ.verify_matmul(case.x, case.w, case.scales, case.biases)
+        torch.cuda.synchronize()                                       # the launch ends
+    finally:
+        assert native_lib.dflash_set_option(nat.OPT_QMM_SPIN_LIMIT, 0) == 0
+    with pytest.raises(nat.NativeLibraryError, match="partial tiles of row block"):
+        VQ.raise_on_device_errors(torch.device(DEV))
+    ws = VQ._workspace(torch.device(DEV), nat.raw_stream(torch.device(DEV)), 1)
+    assert int((ws != 0).sum()) == 0
+    again = VQ.verify_matmul(case.x, case.w, case.scales, case.biases)
+    torch.cuda.synchronize()
+    VQ.raise_on_device_errors(torch.device(DEV))
+    assert torch.equal(again, good)
+
+
 def test_n_tiles_are_independent_full_size(verify_env, native_lib, kernel_mode):
     """Size-independent property at a full 27B shape: any N-slice of W gives the matching
     slice of the full product - the same bits with the tile kernel (fixed K split), and to
