@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
@@ -22,6 +22,7 @@ QMM_CHAIN_MAX = 16                       # DFLASH_QMM_CHAIN_MAX
 QMM_ERROR_OFFSET = (16384 - 64 + 1) * 4        # DFLASH_QMM_ERROR_OFFSET
 QMM_CHAIN_ERROR_OFFSET = QMM_ERROR_OFFSET      # DFLASH_QMM_CHAIN_ERROR_OFFSET
 QMM_EPILOGUE_NONE, QMM_EPILOGUE_SILU_MUL = 0, 1
+QMM_CHAIN_JOINT_SPLIT = 1                # DFLASH_QMM_CHAIN_JOINT_SPLIT
 OPT_GDN_STEP_BY_STEP, OPT_SDPA_SPLITS, OPT_SDPA_STAGED, OPT_QMM_SPIN_LIMIT = 0, 1, 2, 3  # DFLASH_OPT_*
 
 
@@ -88,9 +89,9 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.dflash_qmm_m16_static.restype = c.c_int
     lib.dflash_qmm_m16_static.argtypes = [c.c_void_p] * 5 + [c.c_int] * 8 + [c.c_void_p]
     lib.dflash_qmm_m16_chain_workspace_bytes.restype = c.c_size_t
-    lib.dflash_qmm_m16_chain_workspace_bytes.argtypes = [c.POINTER(QmmProblem), c.c_int, c.c_int]
+    lib.dflash_qmm_m16_chain_workspace_bytes.argtypes = [c.POINTER(QmmProblem), c.c_int, c.c_int, c.c_int]
     lib.dflash_qmm_m16_chain.restype = c.c_int
-    lib.dflash_qmm_m16_chain.argtypes = [c.POINTER(QmmProblem), c.c_int, c.c_void_p, c.c_size_t] + [c.c_int] * 4 + [c.c_void_p]
+    lib.dflash_qmm_m16_chain.argtypes = [c.POINTER(QmmProblem), c.c_int, c.c_void_p, c.c_size_t] + [c.c_int] * 5 + [c.c_void_p]
     lib.dflash_qmm_m16_packed_bytes.restype = c.c_int
     lib.dflash_qmm_m16_packed_bytes.argtypes = [c.c_int] * 3 + [c.POINTER(c.c_size_t)] * 2
     lib.dflash_qmm_m16_pack.restype = c.c_int

@@ -43,8 +43,8 @@ constexpr int kChainAhead = DFLASH_CHAIN_AHEAD;  // units issued beyond the one 
 // 1 KiB) for each of the two row blocks a workgroup can be last at, the table of ranges.
 constexpr int kChainFlags = kLdsBytes;
 constexpr int kChainExchange = kChainFlags + 64;
-constexpr int kChainTable = kChainExchange + 2 * 4096;  // 32 bytes per problem: its Range
-constexpr int kLdsBytesChain = kChainTable + 32 * kMaxChain;  // 152.6 KiB
+constexpr int kChainTable = kChainExchange + 2 * 4096;  // 48 bytes per problem: its Range
+constexpr int kLdsBytesChain = kChainTable + 48 * kMaxChain;  // 152.8 KiB
 // The last words of the 64 KiB counter block: launch bookkeeping of chains.
 constexpr int kChainStatusWord = 16384 - 64;  // [0] exit counter, [1] error word
 constexpr int kChainDoneWord = kChainStatusWord + 8;  // [kMaxChain] row blocks stored, per problem
@@ -71,6 +71,7 @@ struct ChainParams {
   uint32_t* counters;
   int has_deps;
   int spin_limit;
+  int joint;  // the problems' units laid end to end and divided as ONE range (independent problems only)
 };
 
 // The kernel reads its argument block in place, through the constant address space: a
@@ -80,15 +81,54 @@ typedef const __attribute__((address_space(4))) ChainProblem CProblem;
 typedef const __attribute__((address_space(4))) ChainParams CParams;
 
 // How one problem is divided: this workgroup's range of units, or wg < 0 if it has none.
+// `off` and `total` place the problem's units on the line that `grid` workgroups divide: the
+// problem's own units (off 0, total = units) or, in the joint form, the units of all problems
+// end to end (off = units of the problems before it, total = all of them).
 struct Range {
   int stages, RB, units, grid, wg;
   int u0, u1, rb0, st0;
+  int off, total;
 };
-__device__ __forceinline__ Range problem_range(CProblem& q, int block, int nblocks) {
+__device__ __forceinline__ Range problem_range(CParams& p, int i, int block, int nblocks) {
+  CProblem& q = p.prob[i];
   Range r;
   r.stages = q.K / kUnitK;
   r.RB = (q.N + kRows - 1) / kRows;
   r.units = r.RB * r.stages;
+  r.off = 0;
+  r.total = r.units;
+  r.u0 = r.u1 = r.rb0 = r.st0 = 0;
+  if (p.joint) {
+    // One range per workgroup over all problems: nearly every row block is computed by one
+    // workgroup from end to end, only the row blocks at the ends of a range are shared.
+    int off = 0, total = 0;
+    for (int j = 0; j < p.count; ++j) {
+      const int u = ((p.prob[j].N + kRows - 1) / kRows) * (p.prob[j].K / kUnitK);
+      off += j < i ? u : 0;
+      total += u;
+    }
+    r.off = off;
+    r.total = total;
+    // (no more workgroups than units: every workgroup between two contributors of a row block
+    // must be a contributor itself)
+    const int grid = nblocks < total ? nblocks : total;
+    r.grid = grid;
+    const int wg = grid == nblocks && nblocks % 8 == 0 ? (block % 8) * (nblocks / 8) + block / 8 : block;  // XCD-major, as below
+    int a = 0, b = 0;
+    if (wg < grid) {
+      a = range_begin(total, wg, grid) - off, b = range_begin(total, wg + 1, grid) - off;
+      a = a < 0 ? 0 : (a > r.units ? r.units : a);
+      b = b < 0 ? 0 : (b > r.units ? r.units : b);
+    }
+    r.wg = a < b ? wg : -1;
+    if (r.wg >= 0) {
+      r.u0 = a;
+      r.u1 = b;
+      r.rb0 = a / r.stages;
+      r.st0 = a - r.rb0 * r.stages;
+    }
+    return r;
+  }
   r.grid = q.grid;
   // Workgroups are dealt to the eight XCDs in turn (block % 8); unit ranges follow the XCD-major
   // order, so that the neighbours that share a row block sit behind one L2 (as a launch of its
@@ -99,7 +139,6 @@ __device__ __forceinline__ Range problem_range(CProblem& q, int block, int nbloc
   } else {
     r.wg = block < r.grid ? block : -1;
   }
-  r.u0 = r.u1 = r.rb0 = r.st0 = 0;
   if (r.wg >= 0) {
     r.u0 = range_begin(r.units, r.wg, r.grid);
     r.u1 = range_begin(r.units, r.wg + 1, r.grid);
@@ -113,9 +152,10 @@ __device__ __forceinline__ Range problem_range(CProblem& q, int block, int nbloc
 // qmm_m16_stream.hip).  All values are the same in every lane.
 __device__ __forceinline__ Range read_range(uint32_t lds0, int i) {
   u32x4_t a, b;
-  const uint32_t addr = lds0 + kChainTable + i * 32;
-  asm volatile("ds_read_b128 %0, %2\n ds_read_b128 %1, %2 offset:16\n s_waitcnt lgkmcnt(0)"
-               : "=&v"(a), "=&v"(b)
+  u32x2_t c;
+  const uint32_t addr = lds0 + kChainTable + i * 48;
+  asm volatile("ds_read_b128 %0, %3\n ds_read_b128 %1, %3 offset:16\n ds_read_b64 %2, %3 offset:32\n s_waitcnt lgkmcnt(0)"
+               : "=&v"(a), "=&v"(b), "=&v"(c)
                : "v"(addr)
                : "memory");
   Range r;
@@ -127,6 +167,8 @@ __device__ __forceinline__ Range read_range(uint32_t lds0, int i) {
   r.stages = __builtin_amdgcn_readfirstlane((int)b.y);
   r.units = __builtin_amdgcn_readfirstlane((int)b.z);
   r.grid = __builtin_amdgcn_readfirstlane((int)b.w);
+  r.off = __builtin_amdgcn_readfirstlane((int)c.x);
+  r.total = __builtin_amdgcn_readfirstlane((int)c.y);
   r.RB = r.units / r.stages;
   return r;
 }
@@ -241,9 +283,10 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
   // How every problem is divided (this workgroup's range): computed once, lane i of wave 0 for
   // problem i, and kept in LDS; the waves look a problem up when they reach it.
   if (wave == 0 && lane < p.count) {
-    const Range r = problem_range(p.prob[lane], block, nblocks);
-    int* t = reinterpret_cast<int*>(lds + kChainTable + lane * 32);
+    const Range r = problem_range(p, lane, block, nblocks);
+    int* t = reinterpret_cast<int*>(lds + kChainTable + lane * 48);
     t[0] = r.wg, t[1] = r.u0, t[2] = r.u1, t[3] = r.rb0, t[4] = r.st0, t[5] = r.stages, t[6] = r.units, t[7] = r.grid;
+    t[8] = r.off, t[9] = r.total;
   }
   __syncthreads();
 
@@ -542,11 +585,12 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
   }
 
   // Contributors of row block rb of a problem divided as `rx`: the workgroups whose ranges
-  // intersect [lo, lo + stages); owner(v) = ceil((v+1)*grid/units) - 1 holds unit v.
+  // intersect [lo, lo + stages) of the divided line; owner(v) = ceil((v+1)*grid/total) - 1 holds
+  // unit v of it.
   auto contributors = [&](const Range& rx, int rb, int& lo_wg, int& hi_wg) __attribute__((always_inline)) {
-    const int lo = rb * rx.stages;
-    lo_wg = (int)((((unsigned)lo + 1u) * (unsigned)rx.grid + rx.units - 1) / (unsigned)rx.units) - 1;
-    hi_wg = (int)((((unsigned)(lo + rx.stages)) * (unsigned)rx.grid + rx.units - 1) / (unsigned)rx.units) - 1;
+    const int lo = rx.off + rb * rx.stages;
+    lo_wg = (int)((((unsigned)lo + 1u) * (unsigned)rx.grid + rx.total - 1) / (unsigned)rx.total) - 1;
+    hi_wg = (int)((((unsigned)(lo + rx.stages)) * (unsigned)rx.grid + rx.total - 1) / (unsigned)rx.total) - 1;
   };
 
   // ================================== worker waves ====================================
@@ -677,7 +721,10 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
       contributors(rx, srb[i], lo_wg, hi_wg);
       // Only the first contributor can have started before the row block (then the block is the
       // one its range ends in, slot 1); every later one starts inside it (slot 0).
-      const int which_first = range_begin(rx.units, lo_wg, rx.grid) < srb[i] * rx.stages ? 1 : 0;
+      // (in the joint form its range may begin in an earlier problem: here it then begins with
+      // row block 0)
+      const int first_begin = range_begin(rx.total, lo_wg, rx.grid) - rx.off;
+      const int which_first = (first_begin > 0 ? first_begin : 0) < srb[i] * rx.stages ? 1 : 0;
       for (int wg0 = lo_wg; wg0 <= hi_wg; wg0 += 8) {
         const float* src[8];
 #pragma unroll
@@ -909,23 +956,26 @@ bool chain_problem_ok(const dflash_qmm_problem& q, int group_size) {
 int chain_row_blocks(const dflash_qmm_problem& q) { return (q.N + stream::kRows - 1) / stream::kRows; }
 }  // namespace
 
-size_t qmm_chain_workspace_bytes(const dflash_qmm_problem* problems, int count, int group_size) {
+size_t qmm_chain_workspace_bytes(const dflash_qmm_problem* problems, int count, int group_size, int flags) {
   if (!problems || count <= 0 || count > stream::kMaxChain) return 0;
   const int cus = qmm_stream_grid();
+  const bool joint = (flags & DFLASH_QMM_CHAIN_JOINT_SPLIT) != 0;
   size_t tiles = 0;
   for (int i = 0; i < count; ++i) {
     if (!chain_problem_ok(problems[i], group_size)) return 0;
     const int rbs = chain_row_blocks(problems[i]);
-    tiles += 2 * (size_t)qmm_stream_pick_grid(rbs * (problems[i].K / stream::kUnitK), rbs, cus);
+    tiles += 2 * (size_t)(joint ? cus : qmm_stream_pick_grid(rbs * (problems[i].K / stream::kUnitK), rbs, cus));
   }
   return (size_t)64 * 1024 + tiles * stream::kPartialFloats * sizeof(float);
 }
 
 int qmm_chain_launch(const dflash_qmm_problem* problems, int count, void* workspace,
                      size_t workspace_bytes, int group_size, int act_dtype, int sb_dtype,
-                     int spin_limit, hipStream_t stream) {
+                     int spin_limit, int flags, hipStream_t stream) {
   using namespace stream;
   DFLASH_REQUIRE(problems && count > 0, DFLASH_ERR_ARG, "dflash_qmm_m16_chain: no problems");
+  DFLASH_REQUIRE((flags & ~DFLASH_QMM_CHAIN_JOINT_SPLIT) == 0, DFLASH_ERR_ARG, "dflash_qmm_m16_chain: flags %d", flags);
+  const bool joint = (flags & DFLASH_QMM_CHAIN_JOINT_SPLIT) != 0;
   DFLASH_REQUIRE(count <= kMaxChain, DFLASH_ERR_SHAPE, "dflash_qmm_m16_chain: at most %d problems per launch, got %d",
                  kMaxChain, count);
   ChainParams p{};
@@ -946,6 +996,9 @@ int qmm_chain_launch(const dflash_qmm_problem* problems, int count, void* worksp
     DFLASH_REQUIRE(q.wait_for >= -1 && q.wait_for < i, DFLASH_ERR_ARG,
                    "dflash_qmm_m16_chain: problem %d can only wait for an earlier problem (wait_for=%d)", i,
                    q.wait_for);
+    DFLASH_REQUIRE(!(joint && q.wait_for >= 0), DFLASH_ERR_ARG,
+                   "dflash_qmm_m16_chain: the joint split is for independent problems (problem %d waits for %d): "
+                   "a workgroup whose range lies in a later problem would sit waiting from the start", i, q.wait_for);
     if (q.wait_for >= 0) {
       const dflash_qmm_problem& src = problems[q.wait_for];
       const int src_cols = src.epilogue == DFLASH_QMM_EPILOGUE_SILU_MUL ? src.N / 2 : src.N;
@@ -964,7 +1017,7 @@ int qmm_chain_launch(const dflash_qmm_problem* problems, int count, void* worksp
     d.K = q.K;
     d.N = q.N;
     const int rbs = chain_row_blocks(q);
-    d.grid = qmm_stream_pick_grid(rbs * (q.K / kUnitK), rbs, cus);
+    d.grid = joint ? cus : qmm_stream_pick_grid(rbs * (q.K / kUnitK), rbs, cus);
     d.counter_base = counters;
     d.partial_base = tiles;
     d.wait_for = q.wait_for;
@@ -982,6 +1035,7 @@ int qmm_chain_launch(const dflash_qmm_problem* problems, int count, void* worksp
   p.counters = (uint32_t*)workspace;
   p.partials = (float*)((char*)workspace + 64 * 1024);
   p.spin_limit = spin_limit > 0 ? spin_limit : (1 << 22);
+  p.joint = joint ? 1 : 0;
 
   const bool a16 = act_dtype == DFLASH_FP16, s16 = sb_dtype == DFLASH_FP16;
   const void* fn = a16 ? (s16 ? (const void*)qmm_chain_kernel<true, true> : (const void*)qmm_chain_kernel<true, false>)
@@ -1009,18 +1063,18 @@ extern "C" int dflash_debug_read_stamps(unsigned long long* out_host) {
 #endif
 
 extern "C" size_t dflash_qmm_m16_chain_workspace_bytes(const dflash_qmm_problem* problems, int count,
-                                                       int group_size) {
-  return dflash::qmm_chain_workspace_bytes(problems, count, group_size);
+                                                       int group_size, int flags) {
+  return dflash::qmm_chain_workspace_bytes(problems, count, group_size, flags);
 }
 
 extern "C" int dflash_qmm_m16_chain(const dflash_qmm_problem* problems, int count, void* workspace,
                                     size_t workspace_bytes, int group_size, int act_dtype, int sb_dtype,
-                                    int spin_limit, void* stream) {
+                                    int spin_limit, int flags, void* stream) {
   using namespace dflash;
   DFLASH_REQUIRE(act_dtype == DFLASH_BF16 || act_dtype == DFLASH_FP16, DFLASH_ERR_ARG,
                  "dflash_qmm_m16_chain: act_dtype %d is not bf16/fp16", act_dtype);
   DFLASH_REQUIRE(sb_dtype == DFLASH_BF16 || sb_dtype == DFLASH_FP16, DFLASH_ERR_ARG,
                  "dflash_qmm_m16_chain: sb_dtype %d is not bf16/fp16", sb_dtype);
   return qmm_chain_launch(problems, count, workspace, workspace_bytes, group_size, act_dtype, sb_dtype,
-                          spin_limit, (hipStream_t)stream);
+                          spin_limit, flags, (hipStream_t)stream);
 }

@@ -226,9 +226,16 @@ class QmmChain:
     of times: ``chain()`` enqueues the launch on the current stream and returns the outputs, which
     are the same tensors every time.  Inputs are read from where they were when the chain was
     built (``x`` tensors are not copied).  Needs 4-bit codes, group 64, K a multiple of 1024,
-    N of 32, bf16/fp16 activations on the GPU; at most 16 projections."""
+    N of 32, bf16/fp16 activations on the GPU; at most 16 projections.
 
-    def __init__(self, problems, *, group_size: int = 64, bits: int = 4, spin_limit: int = 0):
+    ``joint_split=True`` (independent projections only): the units of all projections are divided
+    among the workgroups as ONE range, so that nearly every row block is computed by a single
+    workgroup over all of K and hardly any partial sums cross workgroups.  Outputs then equal
+    ``verify_matmul``'s to within one rounding of the output type (a row block's sum is cut in
+    other places), and are the same from run to run."""
+
+    def __init__(self, problems, *, group_size: int = 64, bits: int = 4, spin_limit: int = 0,
+                 joint_split: bool = False):
         problems = list(problems)
         if bits != 4 or group_size != 64:
             raise ValueError("QmmChain: 4-bit codes in groups of 64 only")
@@ -279,7 +286,10 @@ class QmmChain:
         self._count, self._group = len(problems), group_size
         self._act, self._sb, self._device = _DTYPE_CODE[act], _DTYPE_CODE[sb], device
         self._spin = int(spin_limit)
-        self._need = int(lib.dflash_qmm_m16_chain_workspace_bytes(self._table, self._count, group_size))
+        self._flags = _native.QMM_CHAIN_JOINT_SPLIT if joint_split else 0
+        if joint_split and any(self._table[i].wait_for >= 0 for i in range(len(problems))):
+            raise ValueError("QmmChain: joint_split is for projections that do not read each other")
+        self._need = int(lib.dflash_qmm_m16_chain_workspace_bytes(self._table, self._count, group_size, self._flags))
         if self._need == 0:
             raise ValueError("QmmChain: a projection has a shape the chained kernel does not cover "
                              "(group 64, K % 1024 == 0, N % 32 == 0; N % 128 == 0 with an epilogue)")
@@ -289,7 +299,7 @@ class QmmChain:
         ws = _workspace(self._device, stream, self._need)
         self._ws = ws
         rc = _native.lib().dflash_qmm_m16_chain(self._table, self._count, ws.data_ptr(), ws.numel(), self._group,
-                                                self._act, self._sb, self._spin, stream)
+                                                self._act, self._sb, self._spin, self._flags, stream)
         _native.check(rc, "dflash_qmm_m16_chain")
         return self.outputs
 

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 14
+#define DFLASH_ABI_VERSION 15
 
 enum {
   DFLASH_OK = 0,
@@ -171,10 +171,18 @@ int dflash_qmm_m16_static(const void* x, const uint32_t* w_q, const void* scales
  * goes on with whatever x holds, and the launch ends normally: the outputs of problem i and of
  * what depends on it are then undefined.  The grid is one workgroup per compute unit, all of
  * which must be resident at once: the device must not be shared with other long-running kernels.
+ * flags: 0, or DFLASH_QMM_CHAIN_JOINT_SPLIT for independent problems (every wait_for -1): the units
+ * of all problems are laid end to end and divided among the workgroups as ONE range, so that
+ * nearly every row block is computed by a single workgroup over all of K and only the row blocks
+ * at the two ends of a workgroup's range go through partial tiles.  A row block's sum is then no
+ * longer cut where a launch of its own would cut it: results equal dflash_qmm_m16's to within one
+ * rounding of the output type instead of bit for bit, and are the same from run to run.  The
+ * workspace size depends on the flag.
  */
 #define DFLASH_QMM_CHAIN_MAX 16
 #define DFLASH_QMM_CHAIN_ERROR_OFFSET DFLASH_QMM_ERROR_OFFSET
 enum { DFLASH_QMM_EPILOGUE_NONE = 0, DFLASH_QMM_EPILOGUE_SILU_MUL = 1 };
+enum { DFLASH_QMM_CHAIN_JOINT_SPLIT = 1 };
 
 typedef struct dflash_qmm_problem {
   const void* x;
@@ -187,11 +195,12 @@ typedef struct dflash_qmm_problem {
   int epilogue;
 } dflash_qmm_problem;
 
-size_t dflash_qmm_m16_chain_workspace_bytes(const dflash_qmm_problem* problems, int count, int group_size);
+size_t dflash_qmm_m16_chain_workspace_bytes(const dflash_qmm_problem* problems, int count, int group_size,
+                                            int flags);
 
 int dflash_qmm_m16_chain(const dflash_qmm_problem* problems, int count, void* workspace,
                          size_t workspace_bytes, int group_size, int act_dtype, int sb_dtype,
-                         int spin_limit, void* stream);
+                         int spin_limit, int flags, void* stream);
 
 /*
  * The same product on weights stored in the order the streaming kernel consumes them.  No

@@ -71,6 +71,66 @@ def test_independent_projections_equal_separate_launches(native_lib, shapes):
     assert chain.error_word() == 0
 
 
+@pytest.mark.parametrize("shapes", [LAYER_27B, LAYER_9B, [(1024, 64), (2048, 32), (1024, 4096), (3072, 96)],
+                                    [(5120, 5120)], [(1024, 32)] * 16, LAYER_27B * 3],
+                         ids=["27b-layer", "9b-layer", "small-and-ragged", "single", "sixteen-tiny", "three-27b-layers"])
+def test_joint_split_of_independent_projections(native_lib, c_oracle, shapes):
+    """All units of all projections divided as one range: most row blocks are summed by one
+    workgroup over all of K, so a sum is cut in other places than in a launch of its own.  Bars:
+    the same bits from run to run; against the exact product the bar of the single launches
+    (max-abs <= 2e-2 * row-inf, rel-L2 <= 5e-3, checked on the projections the oracle finishes
+    quickly); against separate launches at most one step of the output type apart, and equal on at
+    least 99 % of the elements; the workspace handed back zero-filled."""
+    cases = _cases(shapes, 760)
+    chain = VQ.QmmChain([VQ.ChainProblem(c.x, c.w, c.scales, c.biases) for c in cases], joint_split=True)
+    runs = []
+    for rep in range(3):
+        for y in chain.outputs:
+            y.fill_(float("nan"))
+        ys = chain()
+        torch.cuda.synchronize()
+        runs.append([y.clone() for y in ys])
+    assert chain.error_word() == 0
+    assert int((chain._ws != 0).sum()) == 0
+    for i, c in enumerate(cases):
+        assert torch.equal(runs[0][i].view(torch.int16), runs[1][i].view(torch.int16)), (i, shapes[i])
+        assert torch.equal(runs[0][i].view(torch.int16), runs[2][i].view(torch.int16)), (i, shapes[i])
+        got = runs[0][i].float()
+        want = _separate(c.x, c).float()
+        assert torch.isfinite(got).all()
+        # one bf16 step at that size; sums that cancel to next to nothing may differ by the fp32 rounding of their terms
+        step = 2.0 ** -7 * torch.maximum(got.abs(), want.abs()) + 1e-5 * want.abs().max()
+        assert bool(((got - want).abs() <= step).all()), (i, shapes[i])
+        assert float((got == want).float().mean()) >= 0.99, (i, shapes[i])
+    for i, c in enumerate(cases[:5]):
+        if c.K * c.N > 5120 * 7168:
+            continue
+        exact = _exact(c_oracle, c).astype(np.float64)
+        got = runs[0][i].float().cpu().numpy().astype(np.float64)
+        assert np.all(np.abs(got - exact) <= 2e-2 * np.abs(exact).max(axis=1, keepdims=True)), (i, shapes[i])
+        assert np.linalg.norm(got - exact) / np.linalg.norm(exact) <= 5e-3, (i, shapes[i])
+
+
+def test_joint_split_with_the_activation_epilogue(native_lib):
+    """Gate/up matrices with the silu-mul epilogue next to plain projections in a joint split:
+    the hidden activation equals the per-projection split's on nearly every element."""
+    K, I = 2048, 4096
+    gate, up = make_qmm_case(K, I, 771).to(DEV), make_qmm_case(K, I, 772).to(DEV)
+    other = make_qmm_case(2048, 1024, 773).to(DEV)
+    w = torch.cat([gate.w, up.w]); sc = torch.cat([gate.scales, up.scales]); bi = torch.cat([gate.biases, up.biases])
+    probs = lambda: [VQ.ChainProblem(other.x, other.w, other.scales, other.biases),
+                     VQ.ChainProblem(gate.x, w, sc, bi, epilogue="silu_mul"),
+                     VQ.ChainProblem(other.x, other.w, other.scales, other.biases)]
+    joint = [y.clone() for y in VQ.QmmChain(probs(), joint_split=True)()]
+    plain = [y.clone() for y in VQ.QmmChain(probs())()]
+    torch.cuda.synchronize()
+    for a, b in zip(joint, plain):
+        assert torch.isfinite(a.float()).all()
+        assert float((a == b).float().mean()) >= 0.99
+        assert bool(((a.float() - b.float()).abs() <= 2.0 ** -6 * torch.maximum(a.float().abs(), b.float().abs())
+                     + 1e-4 * b.float().abs().max()).all())
+
+
 def test_chain_against_the_oracle(native_lib, c_oracle):
     cases = _cases([(1024, 512), (2048, 256), (1024, 1024)], 720)
     ys = VQ.QmmChain([VQ.ChainProblem(c.x, c.w, c.scales, c.biases) for c in cases])()
@@ -205,23 +265,30 @@ def test_argument_errors(native_lib):
         t.x = t.w_q = t.scales = t.biases = t.y = one
         t.K, t.N, t.wait_for, t.epilogue = 1024, 64, -1, 0
     ws = ctypes.c_void_p(one)
-    assert L.dflash_qmm_m16_chain(tab, 0, ws, 1 << 30, 64, 0, 0, 0, None) == -1
-    assert L.dflash_qmm_m16_chain(tab, 17, ws, 1 << 30, 64, 0, 0, 0, None) == -2
+    assert L.dflash_qmm_m16_chain(tab, 0, ws, 1 << 30, 64, 0, 0, 0, 0, None) == -1
+    assert L.dflash_qmm_m16_chain(tab, 17, ws, 1 << 30, 64, 0, 0, 0, 0, None) == -2
     tab[1].K = 512
-    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, None) == -2      # K % 1024
+    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, 0, None) == -2      # K % 1024
     tab[1].K = 1024
     tab[1].wait_for = 1
-    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, None) == -1      # waits for itself
+    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, 0, None) == -1      # waits for itself
     tab[1].wait_for = 0
-    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, None) == -1      # x is not problem 0's y / K != N0
+    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, 0, None) == -1      # x is not problem 0's y / K != N0
     assert b"waits for" in L.dflash_last_error()
     tab[1].wait_for = -1
     tab[0].epilogue = 1
-    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, None) == -2      # N % 128 with an epilogue
+    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, 0, None) == -2      # N % 128 with an epilogue
     tab[0].epilogue = 0
-    assert L.dflash_qmm_m16_chain(tab, 2, None, 0, 64, 0, 0, 0, None) == -3
-    assert L.dflash_qmm_m16_chain_workspace_bytes(tab, 2, 64) >= 64 * 1024 + 2 * 2 * 8192
-    assert L.dflash_qmm_m16_chain_workspace_bytes(tab, 2, 32) == 0
+    assert L.dflash_qmm_m16_chain(tab, 2, None, 0, 64, 0, 0, 0, 0, None) == -3
+    assert L.dflash_qmm_m16_chain_workspace_bytes(tab, 2, 64, 0) >= 64 * 1024 + 2 * 2 * 8192
+    assert L.dflash_qmm_m16_chain_workspace_bytes(tab, 2, 32, 0) == 0
+    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, 2, None) == -1      # unknown flag
+    tab[1].wait_for = 0
+    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, nat.QMM_CHAIN_JOINT_SPLIT, None) == -1
+    assert b"independent" in L.dflash_last_error()
+    tab[1].wait_for = -1
+    assert (L.dflash_qmm_m16_chain_workspace_bytes(tab, 2, 64, nat.QMM_CHAIN_JOINT_SPLIT)
+            >= L.dflash_qmm_m16_chain_workspace_bytes(tab, 2, 64, 0))
 
 
 def test_hidden_activation_of_a_gated_mlp_in_one_launch(native_lib, c_oracle, monkeypatch):
