@@ -190,7 +190,7 @@ def bench_qmm_stack(stack: str, steps: int, warmup: int, device: str, join_gate_
 
 
 def bench_qmm_chain_stack(stack: str, steps: int, warmup: int, device: str, layers_per_launch: int = 1,
-                          join_gate_up: bool = False, joint_split: bool = False):
+                          join_gate_up: bool = False, joint_split: bool = False, packed: bool = False):
     """The same stack with the projections of ``layers_per_launch`` layers handed over as one list
     per launch (``QmmChain``, dflash_qmm_m16_chain): one persistent grid runs them back to back,
     each divided among the workgroups as a launch of its own would be.  Every projection has an
@@ -199,7 +199,8 @@ def bench_qmm_chain_stack(stack: str, steps: int, warmup: int, device: str, laye
     up_proj as one problem of both matrices' rows (see ``build_stack``).  ``joint_split``: the units
     of a launch's problems divided among the workgroups as one range (hardly any row block then
     crosses workgroups); outputs must be within one step of the output type of the separate
-    launches and equal on at least 99 % of the elements."""
+    launches and equal on at least 99 % of the elements.  ``packed``: every problem's weights as the
+    packed images of ``pack_weights`` (a second copy of the weights; same bits out)."""
     import torch
 
     from dflash_mlx_amd._native import QMM_CHAIN_MAX
@@ -215,9 +216,14 @@ def bench_qmm_chain_stack(stack: str, steps: int, warmup: int, device: str, laye
         from dflash_mlx_amd.workloads import qmm_algorithmic_bytes
 
         total_bytes = sum(qmm_algorithmic_bytes(c.K, c.N)[1] for c in calls)
-    chains = [QmmChain([ChainProblem(c.x, c.w, c.scales, c.biases) for c in calls[i:i + per_chain]],
-                       joint_split=joint_split)
-              for i in range(0, len(calls), per_chain)]
+    if packed:
+        from dflash_mlx_amd.verify_qmm import pack_weights
+
+        images = [pack_weights(c.w, c.scales, c.biases) for c in calls]
+        problems = [ChainProblem(c.x, im) for c, im in zip(calls, images)]
+    else:
+        problems = [ChainProblem(c.x, c.w, c.scales, c.biases) for c in calls]
+    chains = [QmmChain(problems[i:i + per_chain], joint_split=joint_split) for i in range(0, len(calls), per_chain)]
 
     def one_pass():
         return [chain() for chain in chains]
@@ -241,7 +247,9 @@ def bench_qmm_chain_stack(stack: str, steps: int, warmup: int, device: str, laye
                ms_per_step=wall_ms / steps, us_per_layer=ev_ms / steps / (len(calls) / per_layer) * 1e3,
                avg_launch_us=ev_ms / steps / len(chains) * 1e3, bytes_per_launch=total_bytes / len(chains),
                frac_hbm=total_bytes / (ev_ms / steps * 1e-3) / HBM_PEAK)
-    del graph, chains, calls, got, separate
+    del graph, chains, calls, got, separate, problems
+    if packed:
+        del images
     torch.cuda.empty_cache()
     return res
 
@@ -972,6 +980,11 @@ def main() -> int:
             log(f"[bench] {name}, units of a launch divided as one range: {ch['ms_per_step']:.3f} ms/step, "
                 f"{ch['us_per_layer']:.2f} us/layer, {ch['frac_hbm']:.3f} of peak")
             extra[name + "_joint_split"] = rnd(ch)
+        ch = bench_qmm_chain_stack(args.workload, args.steps, args.warmup, device, layers_per_launch=4, join_gate_up=True,
+                                   joint_split=True, packed=True)
+        log(f"[bench] {args.workload} stack, 4 layers per chained launch, gate/up as one problem, joint split, packed "
+            f"weights: {ch['ms_per_step']:.3f} ms/step, {ch['us_per_layer']:.2f} us/layer, {ch['frac_hbm']:.3f} of peak")
+        extra[f"stack_{args.workload}_chained_4_layer_per_launch_gate_up_as_one_problem_joint_split_packed_weights"] = rnd(ch)
         other = "9b" if args.workload == "27b" else "27b"
         ch = bench_qmm_chain_stack(other, args.steps, args.warmup, device, layers_per_launch=3, join_gate_up=True)
         log(f"[bench] {other} stack, 3 layers per chained launch, gate/up as one problem: {ch['ms_per_step']:.3f} ms/step, "

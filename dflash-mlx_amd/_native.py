@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
@@ -23,6 +23,7 @@ QMM_ERROR_OFFSET = (16384 - 64 + 1) * 4        # DFLASH_QMM_ERROR_OFFSET
 QMM_CHAIN_ERROR_OFFSET = QMM_ERROR_OFFSET      # DFLASH_QMM_CHAIN_ERROR_OFFSET
 QMM_EPILOGUE_NONE, QMM_EPILOGUE_SILU_MUL = 0, 1
 QMM_CHAIN_JOINT_SPLIT = 1                # DFLASH_QMM_CHAIN_JOINT_SPLIT
+QMM_LAYOUT_ROWS, QMM_LAYOUT_PACKED = 0, 1  # DFLASH_QMM_LAYOUT_*
 OPT_GDN_STEP_BY_STEP, OPT_SDPA_SPLITS, OPT_SDPA_STAGED, OPT_QMM_SPIN_LIMIT = 0, 1, 2, 3  # DFLASH_OPT_*
 
 
@@ -30,7 +31,7 @@ class QmmProblem(ctypes.Structure):
     """dflash_qmm_problem of include/dflash_mi355.h."""
     _fields_ = [("x", ctypes.c_void_p), ("w_q", ctypes.c_void_p), ("scales", ctypes.c_void_p),
                 ("biases", ctypes.c_void_p), ("y", ctypes.c_void_p), ("K", ctypes.c_int), ("N", ctypes.c_int),
-                ("wait_for", ctypes.c_int), ("epilogue", ctypes.c_int)]
+                ("wait_for", ctypes.c_int), ("epilogue", ctypes.c_int), ("layout", ctypes.c_int)]
 
 # every symbol include/dflash_mi355.h declares
 EXPORTED_SYMBOLS = (

@@ -263,7 +263,9 @@ __device__ __forceinline__ float silu_mul(float g, float u) {
   return s * u;
 }
 
-template <bool ACT_FP16, bool SB_FP16>
+// PACKED: w, scales, biases of every problem are the packed images of dflash_qmm_m16_pack (a
+// property of the launch, so that the loaders carry no per-problem strides in registers).
+template <bool ACT_FP16, bool SB_FP16, bool PACKED>
 __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_value) {
   using A = Act<ACT_FP16>;
   (void)by_value;  // the first (and only) argument: offset 0 of the argument block
@@ -327,6 +329,9 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
     // byte offsets of this lane's pieces from the problem's x, w and scales (= biases) arrays
     // (named one by one: an array indexed inside these loops would be placed in memory)
     uint32_t xo0 = 0u, xo1 = 0u, wo0 = 0u, wo1 = 0u, wo2 = 0u, wo3 = 0u, so = 0u;
+    // bytes from unit to unit / chunk to chunk of a row block
+    constexpr uint32_t w_step = PACKED ? kPackedUnitBytes : kUnitK / 2;
+    constexpr uint32_t sb_step = PACKED ? kPackedChunkBytes : CHUNK * kGroups * 2;
     int slot_i = 0, sb_slot_i = 0;
     int n_issued = 0, n_cons = 0;  // units issued / units whose barrier has passed
     int tot = 0;                   // loads this wave has issued
@@ -335,6 +340,13 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
 
     auto set_row_block = [&](int rb) __attribute__((always_inline)) {
       CProblem& q = p.prob[ip];
+      if constexpr (PACKED) {
+        // every instruction of a wave moves 1 KiB of consecutive memory (see qmm_pack_kernel)
+        const uint32_t unit0 = (uint32_t)rb * (uint32_t)(q.K / kUnitK) * kPackedUnitBytes + lane * 16;
+        wo0 = unit0 + (ld + 0) * 1024, wo1 = unit0 + (ld + 4) * 1024, wo2 = unit0 + (ld + 8) * 1024, wo3 = unit0 + (ld + 12) * 1024;
+        so = (uint32_t)rb * (uint32_t)(q.K / (kUnitK * 4)) * kPackedChunkBytes + ld * 1024 + lane * 16;
+        return;
+      }
       const uint32_t row_bytes = (uint32_t)q.K >> 1;
       wo0 = (uint32_t)weight_row(q, rb, 8 * (ld + 0) + w_r) * row_bytes + w_c * 16;
       wo1 = (uint32_t)weight_row(q, rb, 8 * (ld + 4) + w_r) * row_bytes + w_c * 16;
@@ -393,7 +405,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
         char* slot = lds + slot_i * kSlotBytes;
         if ((ist & (CHUNK - 1)) == 0 || i_first) {
           char* sb = lds + kSbOffset + sb_slot_i * kSbSlotBytes;
-          const uint32_t off = so + (uint32_t)(ist / CHUNK) * (CHUNK * kGroups * 2);
+          const uint32_t off = so + (uint32_t)(ist / CHUNK) * sb_step;
           load16_to_lds(bs + off, sb + ld * 1024);
           load16_to_lds(bb + off, sb + kSbArrayBytes + ld * 1024);
           tot += 2;
@@ -407,7 +419,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
           ++def_n;
         }
         {
-          const uint32_t step = (uint32_t)ist * (kUnitK / 2);
+          const uint32_t step = (uint32_t)ist * w_step;
           char* dst = slot + ld * 1024;
           load16_to_lds_stream(bw + (wo0 + step), dst);
           load16_to_lds_stream(bw + (wo1 + step), dst + 4096);
@@ -499,7 +511,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
             int sb_issued = 0;
             uint32_t slot_off = (uint32_t)slot_i * kSlotBytes + ld * 1024;
             uint32_t sb_off = kSbOffset + (uint32_t)sb_slot_i * kSbSlotBytes + ld * 1024;
-            uint32_t w_step = (uint32_t)ist * (kUnitK / 2), x_step = (uint32_t)ist * (kUnitK * 2);
+            uint32_t w_off = (uint32_t)ist * w_step, x_step = (uint32_t)ist * (kUnitK * 2);
             int st = ist;
 #pragma unroll 1
             for (int k = 0; k < n; ++k) {
@@ -509,7 +521,7 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
               asm volatile("s_barrier" ::: "memory");
               newest_had_sb = (st & (CHUNK - 1)) == 0;
               if (newest_had_sb) {
-                const uint32_t off = so + (uint32_t)(st / CHUNK) * (CHUNK * kGroups * 2);
+                const uint32_t off = so + (uint32_t)(st / CHUNK) * sb_step;
                 load16_to_lds(bs + off, lds + sb_off);
                 load16_to_lds(bb + off, lds + sb_off + kSbArrayBytes);
                 ++sb_issued;
@@ -524,12 +536,12 @@ __global__ __launch_bounds__(kThreads, 1) void qmm_chain_kernel(ChainParams by_v
                 load16_to_lds(bx + (xo0 + x_step), dst + kXOffset);
                 load16_to_lds(bx + (xo1 + x_step), dst + kXOffset + 4096);
               }
-              load16_to_lds_stream(bw + (wo0 + w_step), dst);
-              load16_to_lds_stream(bw + (wo1 + w_step), dst + 4096);
-              load16_to_lds_stream(bw + (wo2 + w_step), dst + 8192);
-              load16_to_lds_stream(bw + (wo3 + w_step), dst + 12288);
+              load16_to_lds_stream(bw + (wo0 + w_off), dst);
+              load16_to_lds_stream(bw + (wo1 + w_off), dst + 4096);
+              load16_to_lds_stream(bw + (wo2 + w_off), dst + 8192);
+              load16_to_lds_stream(bw + (wo3 + w_off), dst + 12288);
               ++st;
-              w_step += kUnitK / 2;
+              w_off += w_step;
               x_step += kUnitK * 2;
               slot_off += kSlotBytes;
               if (slot_off >= kDepth * kSlotBytes) slot_off -= kDepth * kSlotBytes;
@@ -950,6 +962,8 @@ namespace {
 bool chain_problem_ok(const dflash_qmm_problem& q, int group_size) {
   if (!qmm_stream_eligible(q.K, q.N, group_size) || q.K % (stream::kUnitK * 4) != 0) return false;
   if ((long long)q.N * q.K / 2 >= (1ll << 32)) return false;  // 32-bit byte offsets inside a matrix
+  if (q.layout != DFLASH_QMM_LAYOUT_ROWS && q.layout != DFLASH_QMM_LAYOUT_PACKED) return false;
+  if (q.layout == DFLASH_QMM_LAYOUT_PACKED && q.epilogue != DFLASH_QMM_EPILOGUE_NONE) return false;
   if (q.epilogue == DFLASH_QMM_EPILOGUE_SILU_MUL) return q.N % 128 == 0;  // 64 rows of each half per row block
   return q.epilogue == DFLASH_QMM_EPILOGUE_NONE;
 }
@@ -987,9 +1001,9 @@ int qmm_chain_launch(const dflash_qmm_problem* problems, int count, void* worksp
                    "dflash_qmm_m16_chain: null operand in problem %d", i);
     DFLASH_REQUIRE(chain_problem_ok(q, group_size), DFLASH_ERR_SHAPE,
                    "dflash_qmm_m16_chain: problem %d needs group_size 64, K %% 1024 == 0, N %% 16 == 0 "
-                   "(N %% 128 == 0 with an epilogue), less than 4 GiB of codes and a known epilogue "
-                   "(K=%d N=%d gs=%d epilogue=%d)",
-                   i, q.K, q.N, group_size, q.epilogue);
+                   "(N %% 128 == 0 with an epilogue), less than 4 GiB of codes, a known epilogue and layout, "
+                   "no epilogue on packed weights (K=%d N=%d gs=%d epilogue=%d layout=%d)",
+                   i, q.K, q.N, group_size, q.epilogue, q.layout);
     DFLASH_REQUIRE(((uintptr_t)q.x % 16) == 0 && ((uintptr_t)q.w_q % 16) == 0 && ((uintptr_t)q.scales % 16) == 0 &&
                        ((uintptr_t)q.biases % 16) == 0,
                    DFLASH_ERR_ARG, "dflash_qmm_m16_chain: operands of problem %d must be 16-byte aligned", i);
@@ -1022,6 +1036,8 @@ int qmm_chain_launch(const dflash_qmm_problem* problems, int count, void* worksp
     d.partial_base = tiles;
     d.wait_for = q.wait_for;
     d.epilogue = q.epilogue;
+    DFLASH_REQUIRE(q.layout == problems[0].layout, DFLASH_ERR_ARG,
+                   "dflash_qmm_m16_chain: all problems of a launch share one weight layout (problem %d)", i);
     counters += rbs;
     tiles += 2 * d.grid;
   }
@@ -1038,10 +1054,15 @@ int qmm_chain_launch(const dflash_qmm_problem* problems, int count, void* worksp
   p.joint = joint ? 1 : 0;
 
   const bool a16 = act_dtype == DFLASH_FP16, s16 = sb_dtype == DFLASH_FP16;
-  const void* fn = a16 ? (s16 ? (const void*)qmm_chain_kernel<true, true> : (const void*)qmm_chain_kernel<true, false>)
-                       : (s16 ? (const void*)qmm_chain_kernel<false, true> : (const void*)qmm_chain_kernel<false, false>);
-  static bool attr_set[kMaxDevices][4] = {};
-  const int idx = (a16 ? 2 : 0) + (s16 ? 1 : 0);
+  const bool packed = problems[0].layout == DFLASH_QMM_LAYOUT_PACKED;
+  const void* const table[2][2][2] = {
+      {{(const void*)qmm_chain_kernel<false, false, false>, (const void*)qmm_chain_kernel<false, false, true>},
+       {(const void*)qmm_chain_kernel<false, true, false>, (const void*)qmm_chain_kernel<false, true, true>}},
+      {{(const void*)qmm_chain_kernel<true, false, false>, (const void*)qmm_chain_kernel<true, false, true>},
+       {(const void*)qmm_chain_kernel<true, true, false>, (const void*)qmm_chain_kernel<true, true, true>}}};
+  const void* fn = table[a16][s16][packed];
+  static bool attr_set[kMaxDevices][8] = {};
+  const int idx = (a16 ? 4 : 0) + (s16 ? 2 : 0) + (packed ? 1 : 0);
   const int slot = current_device_slot();
   if (!attr_set[slot][idx] || slot == kMaxDevices - 1) {
     DFLASH_HIP_OK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytesChain));

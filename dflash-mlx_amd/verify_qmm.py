@@ -205,12 +205,21 @@ class ChainProblem:
     ``x`` is a device tensor of 16 rows of K values, or the ``ChainProblem`` whose output this
     projection reads (its weights then stream while that output is still being computed).
     ``epilogue="silu_mul"``: ``w``/``scales``/``biases`` hold the gate rows followed by the up rows
-    of an MLP and the output is ``silu(gate) * up`` of ``[16, N/2]``."""
+    of an MLP and the output is ``silu(gate) * up`` of ``[16, N/2]``.
+    ``w`` may be a ``PackedWeights`` (``pack_weights``; ``scales`` and ``biases`` are then left out):
+    same bits out, the loads read consecutive memory; not with an epilogue."""
 
-    def __init__(self, x, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, *,
+    def __init__(self, x, w, scales: Optional[torch.Tensor] = None, biases: Optional[torch.Tensor] = None, *,
                  epilogue: Optional[str] = None, out: Optional[torch.Tensor] = None):
         if epilogue not in (None, "silu_mul"):
             raise ValueError(f"unknown epilogue {epilogue!r}")
+        self.packed = None
+        if isinstance(w, PackedWeights):
+            if epilogue is not None or scales is not None or biases is not None:
+                raise ValueError("ChainProblem: packed weights come alone, and without an epilogue")
+            self.packed, w, scales, biases = w, w.codes, w.scales, w.biases
+        elif scales is None or biases is None:
+            raise ValueError("ChainProblem: scales and biases are missing")
         self.x, self.w, self.scales, self.biases = x, w, scales, biases
         self.epilogue, self.out = epilogue, out
 
@@ -263,10 +272,16 @@ class QmmChain:
                 if not x2.is_contiguous():
                     raise ValueError(f"QmmChain: x of projection {i} must be contiguous (it is read in place)")
             w, s, b = pr.w.contiguous(), pr.scales.contiguous(), pr.biases.contiguous()
-            K, N = int(w.shape[1]) * 8, int(w.shape[0])
+            if pr.packed is not None:
+                K, N = pr.packed.K, pr.packed.N
+                if pr.packed.group_size != group_size or w.device != x2.device:
+                    raise ValueError(f"QmmChain: packed weights of projection {i} do not fit this chain")
+            else:
+                K, N = int(w.shape[1]) * 8, int(w.shape[0])
             if int(x2.shape[1]) != K or s.dtype not in _DTYPE_CODE or b.dtype != s.dtype or N % 32 != 0:
                 raise ValueError(f"QmmChain: operands of projection {i} do not fit together (K={K}, N={N})")
-            _require_operands(f"QmmChain, projection {i}", K, N, group_size, w, s, b, x2.device)
+            if pr.packed is None:
+                _require_operands(f"QmmChain, projection {i}", K, N, group_size, w, s, b, x2.device)
             act = x2.dtype if act is None else act
             sb = s.dtype if sb is None else sb
             device = x2.device if device is None else device
@@ -280,9 +295,12 @@ class QmmChain:
             t.x, t.w_q, t.scales, t.biases, t.y = x2.data_ptr(), w.data_ptr(), s.data_ptr(), b.data_ptr(), y.data_ptr()
             t.K, t.N, t.wait_for = K, N, wait_for
             t.epilogue = _native.QMM_EPILOGUE_SILU_MUL if pr.epilogue == "silu_mul" else _native.QMM_EPILOGUE_NONE
+            t.layout = _native.QMM_LAYOUT_PACKED if pr.packed is not None else _native.QMM_LAYOUT_ROWS
             self._keep.append((x2, w, s, b))
             self.outputs.append(y)
             index[id(pr)] = i
+        if len({pr.packed is not None for pr in problems}) > 1:
+            raise ValueError("QmmChain: packed weights for all projections of a chain or for none")
         self._count, self._group = len(problems), group_size
         self._act, self._sb, self._device = _DTYPE_CODE[act], _DTYPE_CODE[sb], device
         self._spin = int(spin_limit)

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 15
+#define DFLASH_ABI_VERSION 16
 
 enum {
   DFLASH_OK = 0,
@@ -152,7 +152,10 @@ int dflash_qmm_m16_static(const void* x, const uint32_t* w_q, const void* scales
  * for bit the same, the weights of the next problem already streaming while the current one
  * ends.
  *
- *   problems[i]: x [16, K], w_q [N, K/8], scales/biases [N, K/64], y [16, N] as for dflash_qmm_m16.
+ *   problems[i]: x [16, K], w_q [N, K/8], scales/biases [N, K/64], y [16, N] as for dflash_qmm_m16
+ *               (layout DFLASH_QMM_LAYOUT_ROWS), or the packed images of dflash_qmm_m16_pack
+ *               (DFLASH_QMM_LAYOUT_PACKED; same bits out, the loads of a wave then read consecutive memory).
+ *               All problems of a launch share one layout.
  *   wait_for    -1, or the index j < i of the problem whose y is this problem's x (x == problems[j].y,
  *               K == its number of output columns): the x loads of problem i are held back until
  *               problem j's output has been stored; its weights stream regardless.
@@ -183,6 +186,7 @@ int dflash_qmm_m16_static(const void* x, const uint32_t* w_q, const void* scales
 #define DFLASH_QMM_CHAIN_ERROR_OFFSET DFLASH_QMM_ERROR_OFFSET
 enum { DFLASH_QMM_EPILOGUE_NONE = 0, DFLASH_QMM_EPILOGUE_SILU_MUL = 1 };
 enum { DFLASH_QMM_CHAIN_JOINT_SPLIT = 1 };
+enum { DFLASH_QMM_LAYOUT_ROWS = 0, DFLASH_QMM_LAYOUT_PACKED = 1 };
 
 typedef struct dflash_qmm_problem {
   const void* x;
@@ -193,6 +197,8 @@ typedef struct dflash_qmm_problem {
   int K, N;
   int wait_for;
   int epilogue;
+  int layout; /* DFLASH_QMM_LAYOUT_ROWS, or DFLASH_QMM_LAYOUT_PACKED: w_q, scales, biases are the images
+                 dflash_qmm_m16_pack wrote for this K and N (no epilogue on packed weights) */
 } dflash_qmm_problem;
 
 size_t dflash_qmm_m16_chain_workspace_bytes(const dflash_qmm_problem* problems, int count, int group_size,

@@ -131,6 +131,32 @@ def test_joint_split_with_the_activation_epilogue(native_lib):
                      + 1e-4 * b.float().abs().max()).all())
 
 
+@pytest.mark.parametrize("joint", [False, True], ids=["per-problem", "joint-split"])
+def test_packed_weights_in_a_chain(native_lib, joint):
+    """A chain whose problems' weights are the packed images of `pack_weights`: bit for bit the
+    chain on the row-major triples, in either split, and the packed single launches."""
+    shapes = [(5120, 7168), (1024, 96), (5120, 5120), (2048, 4096), (17408, 5120)]
+    cases = _cases(shapes, 790)
+    packed = [VQ.pack_weights(c.w, c.scales, c.biases) for c in cases]
+    rows = VQ.QmmChain([VQ.ChainProblem(c.x, c.w, c.scales, c.biases) for c in cases], joint_split=joint)
+    want = [y.clone() for y in rows()]
+    with pytest.raises(ValueError, match="for all projections"):
+        VQ.QmmChain([VQ.ChainProblem(cases[0].x, packed[0]),
+                     VQ.ChainProblem(cases[1].x, cases[1].w, cases[1].scales, cases[1].biases)])
+    mixed = VQ.QmmChain([VQ.ChainProblem(c.x, pk) for c, pk in zip(cases, packed)], joint_split=joint)
+    for rep in range(2):
+        got = mixed()
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16)), (rep, i, shapes[i])
+    assert mixed.error_word() == 0 and int((mixed._ws != 0).sum()) == 0
+    if not joint:
+        for c, pk, y in zip(cases, packed, want):
+            assert torch.equal(VQ.verify_matmul_packed(c.x, pk).view(torch.int16), y.view(torch.int16))
+    with pytest.raises(ValueError, match="without an epilogue"):
+        VQ.ChainProblem(cases[0].x, packed[0], epilogue="silu_mul")
+
+
 def test_chain_against_the_oracle(native_lib, c_oracle):
     cases = _cases([(1024, 512), (2048, 256), (1024, 1024)], 720)
     ys = VQ.QmmChain([VQ.ChainProblem(c.x, c.w, c.scales, c.biases) for c in cases])()
@@ -283,6 +309,11 @@ def test_argument_errors(native_lib):
     assert L.dflash_qmm_m16_chain_workspace_bytes(tab, 2, 64, 0) >= 64 * 1024 + 2 * 2 * 8192
     assert L.dflash_qmm_m16_chain_workspace_bytes(tab, 2, 32, 0) == 0
     assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, 2, None) == -1      # unknown flag
+    tab[0].layout = 2
+    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, 0, None) == -2      # unknown layout
+    tab[0].layout, tab[0].epilogue, tab[0].N = nat.QMM_LAYOUT_PACKED, 1, 128
+    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, 0, None) == -2      # epilogue on packed weights
+    tab[0].layout, tab[0].epilogue, tab[0].N = 0, 0, 64
     tab[1].wait_for = 0
     assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, nat.QMM_CHAIN_JOINT_SPLIT, None) == -1
     assert b"independent" in L.dflash_last_error()
