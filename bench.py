@@ -334,7 +334,7 @@ def bench_mlp_chain(stack: str, steps: int, warmup: int, device: str):
     return res
 
 
-def bench_dependent_layers(stack: str, steps: int, warmup: int, device: str):
+def bench_dependent_layers(stack: str, steps: int, warmup: int, device: str, packed: bool = False):
     """The stack in the order a model runs it (dflash_mlx/runtime.py:779-821, the layer loop of the
     verify forward): every launch consumes what the one before produced.  Per layer: the joined
     q/k/v projection of the layer's input; a copy of the first `hidden` columns of its output
@@ -343,10 +343,11 @@ def bench_dependent_layers(stack: str, steps: int, warmup: int, device: str):
     its output is the next layer's input.  Four qmm launches and one small copy per layer, none
     of which can start before the previous one has ended.  Scales and biases are shrunk so that
     activations keep their magnitude from layer to layer; the bytes moved are the headline's minus
-    the second read of x by up_proj."""
+    the second read of x by up_proj.  ``packed``: every launch on the packed copy of its weights
+    (what ``pack_verify_linears`` gives a model; the result must be the row-major one bit for bit)."""
     import torch
 
-    from dflash_mlx_amd.verify_qmm import ChainProblem, QmmChain, verify_matmul
+    from dflash_mlx_amd.verify_qmm import ChainProblem, QmmChain, pack_weights, verify_matmul, verify_matmul_packed
     from dflash_mlx_amd.workloads import qmm_algorithmic_bytes, stack_linears
 
     linears, layers, _ = stack_linears(stack)
@@ -377,30 +378,51 @@ def bench_dependent_layers(stack: str, steps: int, warmup: int, device: str):
         both = unit_gain(gu, unit_gain(o, a), halves=True)
         g, u = both[:, :gu.N // 2], both[:, gu.N // 2:]
         x = unit_gain(down, (g * torch.sigmoid(g)) * u)
-    gate_up = []
-    for layer in range(layers):
-        c = calls[layer * per_layer + 2]
-        gate_up.append(QmmChain([ChainProblem(torch.empty((16, c.K), dtype=x0.dtype, device=device), c.w, c.scales,
-                                              c.biases, epilogue="silu_mul")]))
-
-    def one_pass():
-        x = x0
+    def plan(use_packed):
+        gate_up, images = [], []
         for layer in range(layers):
-            qkv, o, gu, down = calls[layer * per_layer:(layer + 1) * per_layer]
-            y = verify_matmul(x, qkv.w, qkv.scales, qkv.biases)
-            a = y[:, :H].contiguous()
-            o_out = verify_matmul(a, o.w, o.scales, o.biases)
-            h = torch.empty((16, gu.N // 2), dtype=x0.dtype, device=device)
-            chain = gate_up[layer]
-            chain.rebind(0, x=o_out, out=h)
-            chain()
-            x = verify_matmul(h, down.w, down.scales, down.biases)
-        return x
+            c = calls[layer * per_layer + 2]
+            x_slot = torch.empty((16, c.K), dtype=x0.dtype, device=device)
+            if use_packed:
+                problem = ChainProblem(x_slot, pack_weights(c.w, c.scales, c.biases, gate_up=True), epilogue="silu_mul")
+                images.append([pack_weights(d.w, d.scales, d.biases) if i != 2 else None
+                               for i, d in enumerate(calls[layer * per_layer:(layer + 1) * per_layer])])
+            else:
+                problem = ChainProblem(x_slot, c.w, c.scales, c.biases, epilogue="silu_mul")
+            gate_up.append(QmmChain([problem]))
 
+        def product(x, layer, i):
+            if use_packed:
+                return verify_matmul_packed(x, images[layer][i])
+            c = calls[layer * per_layer + i]
+            return verify_matmul(x, c.w, c.scales, c.biases)
+
+        def one_pass():
+            x = x0
+            for layer in range(layers):
+                gu = calls[layer * per_layer + 2]
+                a = product(x, layer, 0)[:, :H].contiguous()
+                o_out = product(a, layer, 1)
+                h = torch.empty((16, gu.N // 2), dtype=x0.dtype, device=device)
+                chain = gate_up[layer]
+                chain.rebind(0, x=o_out, out=h)
+                chain()
+                x = product(h, layer, 3)
+            return x
+
+        return one_pass, gate_up, images
+
+    one_pass, gate_up, images = plan(False)
     eager = one_pass()
     torch.cuda.synchronize()
     if not bool(torch.isfinite(eager.float()).all()):
         raise RuntimeError("dependent layers: activations left the finite range")
+    if packed:
+        one_pass, gate_up, images = plan(True)
+        again = one_pass()
+        torch.cuda.synchronize()
+        if not torch.equal(again, eager):
+            raise RuntimeError("dependent layers: packed weights give other bits than the row-major triples")
     graph, captured = capture(one_pass)
     for r in range(2):
         graph.replay()
@@ -413,7 +435,7 @@ def bench_dependent_layers(stack: str, steps: int, warmup: int, device: str):
     res = dict(launches_per_layer=per_layer, layers=layers, ms_per_step=wall_ms / steps,
                us_per_layer=ev_ms / steps / layers * 1e3, total_bytes=total_bytes,
                frac_hbm=total_bytes / (ev_ms / steps * 1e-3) / HBM_PEAK)
-    del graph, captured, eager, calls, gate_up
+    del graph, captured, eager, calls, gate_up, images, one_pass
     torch.cuda.empty_cache()
     return res
 
@@ -948,6 +970,10 @@ def main() -> int:
         log(f"[bench] {args.workload} stack, every launch waiting for the one before: {dep['ms_per_step']:.3f} ms/step, "
             f"{dep['us_per_layer']:.2f} us/layer, {dep['frac_hbm']:.3f} of peak")
         extra[f"stack_{args.workload}_dependent_layer"] = rnd(dep)
+        dep = bench_dependent_layers(args.workload, args.steps, args.warmup, device, packed=True)
+        log(f"[bench] {args.workload} stack, every launch waiting for the one before, packed weights: "
+            f"{dep['ms_per_step']:.3f} ms/step, {dep['us_per_layer']:.2f} us/layer, {dep['frac_hbm']:.3f} of peak")
+        extra[f"stack_{args.workload}_dependent_layer_packed_weights"] = rnd(dep)
     stack_variants = []
     if "gate_up" in legs:
         stack_variants.append(("gate_up_in_one_launch", dict(join_gate_up=True)))

@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
@@ -43,6 +43,7 @@ EXPORTED_SYMBOLS = (
     "dflash_qmm_m16",
     "dflash_qmm_error",
     "dflash_qmm_m16_static",
+    "dflash_qmm_m16_pack_gate_up",
     "dflash_qmm_m16_chain_workspace_bytes",
     "dflash_qmm_m16_chain",
     "dflash_qmm_m16_packed_bytes",
@@ -97,6 +98,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.dflash_qmm_m16_packed_bytes.argtypes = [c.c_int] * 3 + [c.POINTER(c.c_size_t)] * 2
     lib.dflash_qmm_m16_pack.restype = c.c_int
     lib.dflash_qmm_m16_pack.argtypes = [c.c_void_p] * 6 + [c.c_int] * 3 + [c.c_void_p]
+    lib.dflash_qmm_m16_pack_gate_up.restype = c.c_int
+    lib.dflash_qmm_m16_pack_gate_up.argtypes = [c.c_void_p] * 6 + [c.c_int] * 3 + [c.c_void_p]
     lib.dflash_qmm_m16_packed.restype = c.c_int
     lib.dflash_qmm_m16_packed.argtypes = [c.c_void_p] * 6 + [c.c_size_t] + [c.c_int] * 5 + [c.c_void_p]
     lib.dflash_qmm_m16_gather_workspace_bytes.restype = c.c_size_t

@@ -263,6 +263,46 @@ __device__ __forceinline__ float silu_mul(float g, float u) {
   return s * u;
 }
 
+// Packed images (see qmm_pack_kernel in qmm_m16_stream.hip) of a gate/up matrix for the silu-mul
+// epilogue: row block rb holds gate rows 64 rb .. 64 rb + 63 followed by the up rows of the same
+// output columns - weight_row() below as a layout.  One thread per 16 bytes of output.
+__global__ __launch_bounds__(256) void qmm_pack_gate_up_kernel(const uint32_t* __restrict__ w,
+                                                               const uint16_t* __restrict__ scales,
+                                                               const uint16_t* __restrict__ biases,
+                                                               uint4* __restrict__ w_out, uint4* __restrict__ s_out,
+                                                               uint4* __restrict__ b_out, int K, int N) {
+  const int stages = K / kUnitK, chunks = stages / 4;
+  const int half_rows = N >> 1;
+  const int RB = (half_rows + 63) / 64;
+  const size_t code_granules = (size_t)RB * stages * (kPackedUnitBytes / 16);
+  const size_t sb_granules = (size_t)RB * chunks * (kPackedChunkBytes / 16);
+  const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  auto source_row = [&](int rb, int v) {
+    int r = 64 * rb + (v & 63);
+    r = r < half_rows ? r : half_rows - 1;
+    return v < 64 ? r : half_rows + r;
+  };
+  if (t < code_granules) {
+    const int lane = (int)(t & 63), q = (int)((t >> 6) & 15);
+    const size_t unit = t >> 10;
+    const int st = (int)(unit % stages), rb = (int)(unit / stages);
+    const int r8 = lane >> 3;
+    const int row = source_row(rb, 8 * q + r8);
+    const int g = (lane & 7) ^ (((r8 >> 1) & 3) << 1);
+    w_out[t] = *reinterpret_cast<const uint4*>((const char*)w + (size_t)row * (K >> 1) + st * (kUnitK / 2) + g * 16);
+  } else if (t < code_granules + 2 * sb_granules) {
+    size_t u = t - code_granules;
+    const bool is_bias = u >= sb_granules;
+    if (is_bias) u -= sb_granules;
+    const int lane = (int)(u & 63), part = (int)((u >> 6) & 3);
+    const size_t chunk = u >> 8;
+    const int c = (int)(chunk % chunks), rb = (int)(chunk / chunks);
+    const int row = source_row(rb, 32 * part + (lane >> 1));
+    const char* src = (const char*)(is_bias ? biases : scales) + ((size_t)row * (K / kGS) + c * 16) * 2 + (lane & 1) * 16;
+    (is_bias ? b_out : s_out)[u] = *reinterpret_cast<const uint4*>(src);
+  }
+}
+
 // PACKED: w, scales, biases of every problem are the packed images of dflash_qmm_m16_pack (a
 // property of the launch, so that the loaders carry no per-problem strides in registers).
 template <bool ACT_FP16, bool SB_FP16, bool PACKED>
@@ -963,7 +1003,6 @@ bool chain_problem_ok(const dflash_qmm_problem& q, int group_size) {
   if (!qmm_stream_eligible(q.K, q.N, group_size) || q.K % (stream::kUnitK * 4) != 0) return false;
   if ((long long)q.N * q.K / 2 >= (1ll << 32)) return false;  // 32-bit byte offsets inside a matrix
   if (q.layout != DFLASH_QMM_LAYOUT_ROWS && q.layout != DFLASH_QMM_LAYOUT_PACKED) return false;
-  if (q.layout == DFLASH_QMM_LAYOUT_PACKED && q.epilogue != DFLASH_QMM_EPILOGUE_NONE) return false;
   if (q.epilogue == DFLASH_QMM_EPILOGUE_SILU_MUL) return q.N % 128 == 0;  // 64 rows of each half per row block
   return q.epilogue == DFLASH_QMM_EPILOGUE_NONE;
 }
@@ -1001,8 +1040,8 @@ int qmm_chain_launch(const dflash_qmm_problem* problems, int count, void* worksp
                    "dflash_qmm_m16_chain: null operand in problem %d", i);
     DFLASH_REQUIRE(chain_problem_ok(q, group_size), DFLASH_ERR_SHAPE,
                    "dflash_qmm_m16_chain: problem %d needs group_size 64, K %% 1024 == 0, N %% 16 == 0 "
-                   "(N %% 128 == 0 with an epilogue), less than 4 GiB of codes, a known epilogue and layout, "
-                   "no epilogue on packed weights (K=%d N=%d gs=%d epilogue=%d layout=%d)",
+                   "(N %% 128 == 0 with an epilogue), less than 4 GiB of codes, a known epilogue and layout "
+                   "(K=%d N=%d gs=%d epilogue=%d layout=%d)",
                    i, q.K, q.N, group_size, q.epilogue, q.layout);
     DFLASH_REQUIRE(((uintptr_t)q.x % 16) == 0 && ((uintptr_t)q.w_q % 16) == 0 && ((uintptr_t)q.scales % 16) == 0 &&
                        ((uintptr_t)q.biases % 16) == 0,
@@ -1082,6 +1121,29 @@ extern "C" int dflash_debug_read_stamps(unsigned long long* out_host) {
                                   sizeof(dflash::stream::g_stamps));
 }
 #endif
+
+extern "C" int dflash_qmm_m16_pack_gate_up(const uint32_t* w_q, const void* scales, const void* biases,
+                                           void* codes_out, void* scales_out, void* biases_out, int K, int N,
+                                           int group_size, void* stream) {
+  using namespace dflash;
+  using namespace dflash::stream;
+  DFLASH_REQUIRE(w_q && scales && biases && codes_out && scales_out && biases_out, DFLASH_ERR_ARG,
+                 "dflash_qmm_m16_pack_gate_up: null operand");
+  DFLASH_REQUIRE(group_size == 64 && K > 0 && K % (kUnitK * 4) == 0 && N > 0 && N % 128 == 0, DFLASH_ERR_SHAPE,
+                 "dflash_qmm_m16_pack_gate_up: group_size 64, K %% 1024 == 0 and N %% 128 == 0 (gate rows then up rows) "
+                 "(K=%d N=%d gs=%d)", K, N, group_size);
+  DFLASH_REQUIRE(((uintptr_t)w_q % 16) == 0 && ((uintptr_t)scales % 16) == 0 && ((uintptr_t)biases % 16) == 0 &&
+                     ((uintptr_t)codes_out % 16) == 0 && ((uintptr_t)scales_out % 16) == 0 &&
+                     ((uintptr_t)biases_out % 16) == 0,
+                 DFLASH_ERR_ARG, "dflash_qmm_m16_pack_gate_up: operands must be 16-byte aligned");
+  const size_t RB = (size_t)(N / 2 + 63) / 64, stages = (size_t)K / kUnitK;
+  const size_t threads = (RB * stages * kPackedUnitBytes + 2 * RB * (stages / 4) * kPackedChunkBytes) / 16;
+  hipLaunchKernelGGL(qmm_pack_gate_up_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, w_q, (const uint16_t*)scales, (const uint16_t*)biases, (uint4*)codes_out,
+                     (uint4*)scales_out, (uint4*)biases_out, K, N);
+  DFLASH_HIP_OK(hipGetLastError());
+  return DFLASH_OK;
+}
 
 extern "C" size_t dflash_qmm_m16_chain_workspace_bytes(const dflash_qmm_problem* problems, int count,
                                                        int group_size, int flags) {

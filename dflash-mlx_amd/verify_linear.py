@@ -118,6 +118,7 @@ class FusedProjections:
             self.bounds.append((row, row + n))
             row += n
         self._packed = None  # the joint matrix in the streaming kernel's order (pack_verify_linears)
+        self._packed_silu = None  # ... and in the order of the silu-mul epilogue, for silu_mul()
         self._silu_chain = None  # the planned launch of silu_mul(), made on first use
 
     def applies(self, parent: nn.Module, x: torch.Tensor) -> bool:
@@ -154,8 +155,12 @@ class FusedProjections:
         out = torch.empty((*x.shape[:-1], rows), dtype=x.dtype, device=x.device)
         chain = self._silu_chain
         if chain is None:
-            chain = QmmChain([ChainProblem(x.reshape(16, -1), self.weight, self.scales, self.biases,
-                                           epilogue="silu_mul", out=out.view(16, rows))])
+            if self._packed_silu is not None:
+                problem = ChainProblem(x.reshape(16, -1), self._packed_silu, epilogue="silu_mul", out=out.view(16, rows))
+            else:
+                problem = ChainProblem(x.reshape(16, -1), self.weight, self.scales, self.biases,
+                                       epilogue="silu_mul", out=out.view(16, rows))
+            chain = QmmChain([problem])
             self._silu_chain = chain
         else:
             chain.rebind(0, x=x.reshape(16, -1), out=out.view(16, rows))
@@ -297,6 +302,11 @@ def pack_verify_linears(model: nn.Module) -> int:
         if shared is not None and shared[0]._packed is None and shared[0].bits == 4 \
                 and packable(shared[0].weight, shared[0].scales, shared[0].biases, shared[0].group_size, 4):
             shared[0]._packed = pack_weights(shared[0].weight, shared[0].scales, shared[0].biases)
+            group = shared[0]
+            # a gate/up pair also in the order its one-launch activation reads (silu_gate_up)
+            if (len(group.bounds) == 2 and group.bounds[1] == (group.bounds[0][1], 2 * group.bounds[0][1])
+                    and group.bounds[0][1] % 64 == 0 and group._silu_chain is None):
+                group._packed_silu = pack_weights(group.weight, group.scales, group.biases, gate_up=True)
             count += 1
         if (isinstance(m, VerifyQuantizedLinear) and getattr(m, "_shared_input", None) is None
                 and getattr(m, "_packed", None) is None and m.biases is not None and m.mode == "affine"

@@ -207,7 +207,8 @@ class ChainProblem:
     ``epilogue="silu_mul"``: ``w``/``scales``/``biases`` hold the gate rows followed by the up rows
     of an MLP and the output is ``silu(gate) * up`` of ``[16, N/2]``.
     ``w`` may be a ``PackedWeights`` (``pack_weights``; ``scales`` and ``biases`` are then left out):
-    same bits out, the loads read consecutive memory; not with an epilogue."""
+    same bits out, the loads read consecutive memory; with ``epilogue="silu_mul"`` the images
+    must come from ``pack_weights(..., gate_up=True)``."""
 
     def __init__(self, x, w, scales: Optional[torch.Tensor] = None, biases: Optional[torch.Tensor] = None, *,
                  epilogue: Optional[str] = None, out: Optional[torch.Tensor] = None):
@@ -215,8 +216,11 @@ class ChainProblem:
             raise ValueError(f"unknown epilogue {epilogue!r}")
         self.packed = None
         if isinstance(w, PackedWeights):
-            if epilogue is not None or scales is not None or biases is not None:
-                raise ValueError("ChainProblem: packed weights come alone, and without an epilogue")
+            if scales is not None or biases is not None:
+                raise ValueError("ChainProblem: packed weights come alone")
+            if (epilogue == "silu_mul") != bool(w.gate_up):
+                raise ValueError("ChainProblem: the silu-mul epilogue reads images of pack_weights(..., gate_up=True), "
+                                 "every other problem those of pack_weights(...)")
             self.packed, w, scales, biases = w, w.codes, w.scales, w.biases
         elif scales is None or biases is None:
             raise ValueError("ChainProblem: scales and biases are missing")
@@ -367,11 +371,12 @@ class PackedWeights:
     (``pack_weights``).  A second copy of the weights, made once when the model is loaded; the
     row-major MLX triple it was made from is not referenced."""
 
-    __slots__ = ("codes", "scales", "biases", "K", "N", "group_size")
+    __slots__ = ("codes", "scales", "biases", "K", "N", "group_size", "gate_up")
 
-    def __init__(self, codes, scales, biases, K, N, group_size):
+    def __init__(self, codes, scales, biases, K, N, group_size, gate_up=False):
         self.codes, self.scales, self.biases = codes, scales, biases
         self.K, self.N, self.group_size = K, N, group_size
+        self.gate_up = gate_up  # rows ordered for the chained kernel's silu-mul epilogue: that use only
 
 
 def packable(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, group_size: int = 64,
@@ -386,12 +391,17 @@ def packable(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, group_
 
 
 def pack_weights(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, *, group_size: int = 64,
-                 bits: int = 4) -> PackedWeights:
+                 bits: int = 4, gate_up: bool = False) -> PackedWeights:
     """Rewrites an MLX affine triple (``w [N, K/8]`` words, ``scales``/``biases [N, K/64]``) into the
     packed images ``verify_matmul_packed`` reads: per 128 rows and 256 k the 16 KiB of codes in
     the order of the kernel's LDS slot, per 128 rows and 1024 k the 4 KiB of scales and of
     biases.  No counterpart in the reference, whose kernel gathers 4-byte words from the
-    row-major arrays (``verify_qmm.py:68-72``)."""
+    row-major arrays (``verify_qmm.py:68-72``).  ``gate_up=True``: ``w`` holds the gate rows of an
+    MLP followed by its up rows, and the images are those a ``ChainProblem`` with the silu-mul
+    epilogue reads (64 gate rows and the 64 up rows of the same columns per row block; N a
+    multiple of 128) - not ``verify_matmul_packed``."""
+    if gate_up and int(w.shape[0]) % 128 != 0:
+        raise ValueError("pack_weights: gate_up needs a number of rows that is a multiple of 128")
     if not packable(w, scales, biases, group_size, bits):
         raise ValueError("pack_weights: needs 4-bit codes, group 64, K % 1024 == 0, N % 32 == 0, "
                          "bf16/fp16 scales and biases of shape [N, K/64], on the GPU")
@@ -404,17 +414,19 @@ def pack_weights(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, *,
     codes = torch.empty(cb.value, dtype=torch.uint8, device=w.device)
     s_img = torch.empty(sb.value // 2, dtype=scales.dtype, device=w.device)
     b_img = torch.empty(sb.value // 2, dtype=scales.dtype, device=w.device)
-    rc = lib.dflash_qmm_m16_pack(w.data_ptr(), scales.data_ptr(), biases.data_ptr(), codes.data_ptr(),
-                                 s_img.data_ptr(), b_img.data_ptr(), K, N, group_size,
-                                 _native.raw_stream(w.device))
-    _native.check(rc, "dflash_qmm_m16_pack")
-    return PackedWeights(codes, s_img, b_img, K, N, group_size)
+    pack = lib.dflash_qmm_m16_pack_gate_up if gate_up else lib.dflash_qmm_m16_pack
+    rc = pack(w.data_ptr(), scales.data_ptr(), biases.data_ptr(), codes.data_ptr(),
+              s_img.data_ptr(), b_img.data_ptr(), K, N, group_size, _native.raw_stream(w.device))
+    _native.check(rc, "dflash_qmm_m16_pack_gate_up" if gate_up else "dflash_qmm_m16_pack")
+    return PackedWeights(codes, s_img, b_img, K, N, group_size, gate_up)
 
 
 def verify_matmul_packed(x: torch.Tensor, packed: PackedWeights) -> torch.Tensor:
     """``verify_matmul`` on packed weights: 16 rows of bf16/fp16 device activations; the result is
     bit for bit that of the streaming kernel on the triple the weights were packed from."""
     K, N = packed.K, packed.N
+    if packed.gate_up:
+        raise ValueError("verify_matmul_packed: these images are ordered for the silu-mul epilogue of a chain")
     m = 1
     for d in x.shape[:-1]:
         m *= int(d)

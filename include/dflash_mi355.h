@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 16
+#define DFLASH_ABI_VERSION 17
 
 enum {
   DFLASH_OK = 0,
@@ -198,11 +198,23 @@ typedef struct dflash_qmm_problem {
   int wait_for;
   int epilogue;
   int layout; /* DFLASH_QMM_LAYOUT_ROWS, or DFLASH_QMM_LAYOUT_PACKED: w_q, scales, biases are the images
-                 dflash_qmm_m16_pack wrote for this K and N (no epilogue on packed weights) */
+                 dflash_qmm_m16_pack wrote for this K and N - with the silu-mul epilogue those of
+                 dflash_qmm_m16_pack_gate_up */
 } dflash_qmm_problem;
 
 size_t dflash_qmm_m16_chain_workspace_bytes(const dflash_qmm_problem* problems, int count, int group_size,
                                             int flags);
+
+/*
+ * Packed images of a gate/up matrix (N/2 gate rows followed by N/2 up rows) for a chained problem
+ * with the silu-mul epilogue and DFLASH_QMM_LAYOUT_PACKED: row block rb holds the gate rows
+ * 64 rb .. 64 rb + 63 and the up rows of the same output columns.  Sizes as
+ * dflash_qmm_m16_packed_bytes(K, N, ...) gives them; group_size 64, K % 1024 == 0, N % 128 == 0.
+ * dflash_qmm_m16_packed does not read these images.
+ */
+int dflash_qmm_m16_pack_gate_up(const uint32_t* w_q, const void* scales, const void* biases,
+                                void* codes_out, void* scales_out, void* biases_out, int K, int N,
+                                int group_size, void* stream);
 
 int dflash_qmm_m16_chain(const dflash_qmm_problem* problems, int count, void* workspace,
                          size_t workspace_bytes, int group_size, int act_dtype, int sb_dtype,

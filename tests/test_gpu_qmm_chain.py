@@ -153,8 +153,31 @@ def test_packed_weights_in_a_chain(native_lib, joint):
     if not joint:
         for c, pk, y in zip(cases, packed, want):
             assert torch.equal(VQ.verify_matmul_packed(c.x, pk).view(torch.int16), y.view(torch.int16))
-    with pytest.raises(ValueError, match="without an epilogue"):
+    with pytest.raises(ValueError, match="gate_up=True"):
         VQ.ChainProblem(cases[0].x, packed[0], epilogue="silu_mul")
+
+
+@pytest.mark.parametrize("K,I", [(2048, 4096), (5120, 17408)])
+def test_packed_gate_up_with_the_activation_epilogue(native_lib, K, I):
+    """The gate/up matrix packed in the order of the epilogue's row blocks (64 gate rows, then the
+    64 up rows of the same columns): the hidden activation bit for bit that of the row-major
+    matrix, alone and next to another packed problem."""
+    gate, up = make_qmm_case(K, I, 801).to(DEV), make_qmm_case(K, I, 802).to(DEV)
+    other = make_qmm_case(1024, 2048, 803).to(DEV)
+    w = torch.cat([gate.w, up.w]); sc = torch.cat([gate.scales, up.scales]); bi = torch.cat([gate.biases, up.biases])
+    want = VQ.QmmChain([VQ.ChainProblem(gate.x, w, sc, bi, epilogue="silu_mul")])()[0].clone()
+    images = VQ.pack_weights(w, sc, bi, gate_up=True)
+    got = VQ.QmmChain([VQ.ChainProblem(gate.x, images, epilogue="silu_mul")])()[0].clone()
+    both = VQ.QmmChain([VQ.ChainProblem(other.x, VQ.pack_weights(other.w, other.scales, other.biases)),
+                        VQ.ChainProblem(gate.x, images, epilogue="silu_mul")])()
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(both[1].view(torch.int16), want.view(torch.int16))
+    assert torch.equal(both[0].view(torch.int16), _separate(other.x, other).view(torch.int16))
+    with pytest.raises(ValueError, match="ordered for the silu-mul epilogue"):
+        VQ.verify_matmul_packed(gate.x, images)
+    with pytest.raises(ValueError, match="gate_up=True"):
+        VQ.ChainProblem(gate.x, images)
 
 
 def test_chain_against_the_oracle(native_lib, c_oracle):
@@ -311,9 +334,12 @@ def test_argument_errors(native_lib):
     assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, 2, None) == -1      # unknown flag
     tab[0].layout = 2
     assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, 0, None) == -2      # unknown layout
-    tab[0].layout, tab[0].epilogue, tab[0].N = nat.QMM_LAYOUT_PACKED, 1, 128
-    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, 0, None) == -2      # epilogue on packed weights
-    tab[0].layout, tab[0].epilogue, tab[0].N = 0, 0, 64
+    tab[0].layout = nat.QMM_LAYOUT_PACKED
+    assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, 0, None) == -1      # two layouts in one launch
+    assert b"one weight layout" in L.dflash_last_error()
+    tab[0].layout = 0
+    assert L.dflash_qmm_m16_pack_gate_up(one, one, one, one, one, one, 1024, 64, 64, None) == -2   # N % 128
+    assert L.dflash_qmm_m16_pack_gate_up(one, one, one, None, one, one, 1024, 128, 64, None) == -1
     tab[1].wait_for = 0
     assert L.dflash_qmm_m16_chain(tab, 2, ws, 1 << 30, 64, 0, 0, 0, nat.QMM_CHAIN_JOINT_SPLIT, None) == -1
     assert b"independent" in L.dflash_last_error()
@@ -388,3 +414,39 @@ def test_hidden_activation_of_a_gated_mlp_in_one_launch(native_lib, c_oracle, mo
     ys = chain()
     torch.cuda.synchronize()
     assert ys[1] is fresh and torch.equal(fresh, _separate(_separate(two[0].x, two[0]), two[1]))
+
+
+def test_gated_mlp_activation_on_packed_weights(native_lib, monkeypatch):
+    """pack_verify_linears gives a joined gate/up pair a copy in the order of the epilogue's row
+    blocks as well: silu_gate_up then reads that copy and returns the bits it returned before."""
+    import dflash_mlx_amd.verify_linear as VL
+    from dflash_mlx_amd.quantized import QuantizedLinear
+
+    monkeypatch.setenv("DFLASH_VERIFY_QMM", "1")
+    K, I = 2048, 1536
+
+    def build():
+        gate, up = _cases([(K, I), (K, I)], 890)
+        mlp = torch.nn.Module()
+        mlp.gate_proj = QuantizedLinear(gate.w.clone(), gate.scales.clone(), gate.biases.clone(), group_size=64, bits=4)
+        mlp.up_proj = QuantizedLinear(up.w.clone(), up.scales.clone(), up.biases.clone(), group_size=64, bits=4)
+        model = torch.nn.Module()
+        model.mlp = mlp
+        assert VL.install_verify_linears(model) == 2 and VL.fuse_shared_input_linears(model) == 1
+        return model
+
+    x = (torch.randn(1, 16, K, generator=torch.Generator().manual_seed(9)) * 0.5).to(torch.bfloat16).to(DEV)
+    plain = build()
+    before = VL.silu_gate_up(plain.mlp, x).clone()
+    packed = build()
+    assert VL.pack_verify_linears(packed) == 1
+    group = packed.mlp.gate_proj._shared_input[0]
+    assert group._packed_silu is not None and group._packed_silu.gate_up and not group._packed.gate_up
+    after = VL.silu_gate_up(packed.mlp, x)
+    torch.cuda.synchronize()
+    assert group._silu_chain._table[0].layout == nat.QMM_LAYOUT_PACKED
+    assert torch.equal(after.view(torch.int16), before.view(torch.int16))
+    g, u = VL.shared_input_outputs(packed.mlp, ("gate_proj", "up_proj"), x)          # the plain packed copy
+    g0, u0 = VL.shared_input_outputs(plain.mlp, ("gate_proj", "up_proj"), x)
+    assert torch.equal(g, g0) and torch.equal(u, u0)
+
