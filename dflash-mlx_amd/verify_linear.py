@@ -291,7 +291,9 @@ def pack_verify_linears(model: nn.Module) -> int:
     """Gives every swapped linear that stands alone, and every shared-input group (its joint
     matrix, counted once), whose shape the packed form covers (group 64, K a multiple of 1024, on the GPU) a second copy
     of its weights in the order the streaming kernel reads them; its 16-row calls then go through
-    ``verify_matmul_packed`` and return the same bits as before, 3-8 % sooner.  The row-major
+    ``verify_matmul_packed`` and return the same bits as before, 3-8 % sooner.  A joined gate/up
+    pair of equal heights gets one more copy, in the order of the chained kernel's silu-mul
+    epilogue, which ``silu_gate_up`` then reads (same bits, about 10 % sooner).  The row-major
     buffers stay for every other call shape.  Call it after ``install_verify_linears`` (and
     after ``fuse_shared_input_linears``, if used) with the model on its device; moving a module
     afterwards drops its packed copy.  Returns the number of linears packed.  No counterpart in
