@@ -157,6 +157,27 @@ def test_packed_weights_in_a_chain(native_lib, joint):
         VQ.ChainProblem(cases[0].x, packed[0], epilogue="silu_mul")
 
 
+def test_joint_split_on_packed_weights_with_fp16_activations(native_lib):
+    """The remaining corner of the table: fp16 activations and scales, packed weights, joint split,
+    outputs rebound between launches."""
+    shapes = [(2048, 1024), (1024, 4096), (4096, 2048)]
+    cases = _cases(shapes, 810, torch.float16)
+    chain = VQ.QmmChain([VQ.ChainProblem(c.x, VQ.pack_weights(c.w, c.scales, c.biases)) for c in cases], joint_split=True)
+    first = [y.clone() for y in chain()]
+    elsewhere = torch.empty_like(first[1])
+    chain.rebind(1, out=elsewhere)
+    second = chain()
+    torch.cuda.synchronize()
+    assert chain.error_word() == 0
+    assert torch.equal(elsewhere, first[1]) and torch.equal(second[0], first[0]) and torch.equal(second[2], first[2])
+    for c, y in zip(cases, first):
+        want = _separate(c.x, c).float()
+        got = y.float()
+        assert bool(((got - want).abs() <= 2.0 ** -10 * torch.maximum(got.abs(), want.abs()) + 1e-5 * want.abs().max()).all())
+        # (fp16 keeps three more bits of the fp32 sum than bf16: another order of additions shows eight times as often)
+        assert float((got == want).float().mean()) >= 0.95
+
+
 @pytest.mark.parametrize("K,I", [(2048, 4096), (5120, 17408)])
 def test_packed_gate_up_with_the_activation_epilogue(native_lib, K, I):
     """The gate/up matrix packed in the order of the epilogue's row blocks (64 gate rows, then the
