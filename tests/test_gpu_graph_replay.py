@@ -54,6 +54,33 @@ def test_qmm_chain_replays(verify_env, native_lib):
     _replays_match(graph, captured, run, refill)
 
 
+def test_chained_launches_replay(verify_env, native_lib):
+    """Chained launches in a graph: the per-problem split, the joint split on packed weights and a
+    gate/up problem with the activation epilogue, one after the other on one workspace; every
+    replay with new inputs gives what the same launches give eagerly."""
+    verify_env.setenv("DFLASH_QMM_KERNEL", "stream")
+    cases = [make_qmm_case(2048, 1536, seed_for(0, 91)).to(DEV), make_qmm_case(1024, 4096, seed_for(0, 92)).to(DEV),
+             make_qmm_case(3072, 512, seed_for(0, 93)).to(DEV)]
+    gate, up = make_qmm_case(2048, 1024, seed_for(0, 94)).to(DEV), make_qmm_case(2048, 1024, seed_for(0, 95)).to(DEV)
+    gu = (torch.cat([gate.w, up.w]), torch.cat([gate.scales, up.scales]), torch.cat([gate.biases, up.biases]))
+    plain = VQ.QmmChain([VQ.ChainProblem(c.x, c.w, c.scales, c.biases) for c in cases])
+    joint = VQ.QmmChain([VQ.ChainProblem(c.x, VQ.pack_weights(c.w, c.scales, c.biases)) for c in cases], joint_split=True)
+    hidden = VQ.QmmChain([VQ.ChainProblem(gate.x, VQ.pack_weights(*gu, gate_up=True), epilogue="silu_mul")])
+
+    def run():
+        return [y.clone() for chain in (plain, joint, hidden) for y in chain()]
+
+    graph, captured = _capture(run)
+    gen = torch.Generator(device=DEV).manual_seed(6)
+
+    def refill(r):
+        for c in cases + [gate]:
+            c.x.copy_(torch.randn(c.x.shape, generator=gen, device=DEV).to(c.x.dtype))
+
+    _replays_match(graph, captured, run, refill)
+    VQ.raise_on_device_errors(torch.device(DEV))
+
+
 def test_rollback_replays_with_device_step_counts(native_lib):
     """Tape replay with the accepted length in device memory: one recorded launch serves every
     acceptance length."""
