@@ -248,8 +248,9 @@ __device__ __forceinline__ f32x4_t reduce_groups_read(uint32_t base, const f32x4
 // (DFLASH_QMM_ERROR_OFFSET / 4 of the C interface).
 constexpr int kErrorWord = 16384 - 64 + 1;
 // Polls of a row block's partial tiles (about a microsecond each) before the adding workgroup
-// gives up.
-constexpr int kSpinLimit = 1 << 18;
+// gives up: seconds, so that other work that keeps a contributor off the device for a while
+// (another stream's long kernel on a shared GPU) does not turn into an error.
+constexpr int kSpinLimit = 1 << 22;
 
 // A partial tile on its way through memory doubles as its own "ready" flag: +0.0 travels as
 // -0.0 (the sum starts from +0.0, and +0.0 + -0.0 = +0.0, x + -0.0 = x: nothing changes), so

@@ -64,7 +64,7 @@ const char* dflash_last_error(void);
  *   DFLASH_OPT_SDPA_STAGED       1: dflash_sdpa_q16 without a mask keeps the kernel that stages its
  *                                tiles through registers (the one a mask always takes)
  *   DFLASH_OPT_QMM_SPIN_LIMIT    n > 0: the streaming qmm kernel's workgroups that add partial tiles
- *                                give up after n polls instead of 2^18 (tests of that path: the
+ *                                give up after n polls instead of 2^22 (tests of that path: the
  *                                launch ends, the error word is set, results are unspecified)
  * dflash_set_option returns 0, or DFLASH_ERR_ARG for an unknown option or a negative value;
  * dflash_get_option returns the value, or DFLASH_ERR_ARG.
