@@ -104,8 +104,8 @@ int dflash_get_option(int option);
  * The streaming kernel hands partial sums of row blocks that several workgroups share to one
  * of them through the workspace; that workgroup waits for the others' partial tiles (they
  * were dispatched before it, so they are running or done).  The wait is bounded: a workgroup
- * that gives up - which takes a device that stops running resident workgroups for about a
- * second - stores 0x80000000 | row block into the 32-bit word at byte offset
+ * that gives up - which takes a device that keeps a workgroup of the launch from running for
+ * several seconds - stores 0x80000000 | row block into the 32-bit word at byte offset
  * DFLASH_QMM_ERROR_OFFSET of the workspace, the launch ends normally, and y is then
  * undefined.  The word stays set until the caller zero-fills the workspace again, which it
  * must do before the next call; dflash_qmm_error() reads it.
