@@ -813,17 +813,18 @@ def bench_gdn_glue(device: str, steps: int, warmup: int):
     return out
 
 
-def bench_sdpa(device: str, steps: int, warmup: int):
-    """Attention of the 16-token verify block over the KV caches of config[2]'s 16 full-attention
-    layers: 8 key/value heads of 256 over 4096 + 16 positions (bf16, read in place from buffers of
-    capacity 4352), 32 query heads.  Algorithmic bytes per layer: K and V once, q and out once."""
+def bench_sdpa(device: str, steps: int, warmup: int, N: int = 4112, L: int = 16, with_torch: bool = True):
+    """Attention of the 16-token verify block over the KV caches of config[2]'s full-attention
+    layers: 8 key/value heads of 256 over N = 4096 + 16 positions (bf16, read in place from buffers
+    of capacity N + 240), 32 query heads, L layers with caches of their own (16 in the model).
+    Algorithmic bytes per layer: K and V once, q and out once."""
     import torch
 
     from dflash_mlx_amd import _native
     from dflash_mlx_amd.kernels import _DTYPE_CODE
 
     lib = _native.lib()
-    L, B, Hq, Hk, N, D, cap = 16, 1, 32, 8, 4112, 256, 4352
+    B, Hq, Hk, D, cap = 1, 32, 8, 256, N + 240
     bf = torch.bfloat16
     gen = torch.Generator(device=device).manual_seed(0xDF1A + 2700)
     caches = [(torch.randn((B, Hk, cap, D), generator=gen, device=device).to(bf),
@@ -851,7 +852,7 @@ def bench_sdpa(device: str, steps: int, warmup: int):
                                                              scale=scale, enable_gqa=True)
 
     res = {}
-    for name, fn in (("kernel", kernel_pass), ("torch_sdpa", torch_pass)):
+    for name, fn in (("kernel", kernel_pass), ("torch_sdpa", torch_pass))[:2 if with_torch else 1]:
         for _ in range(max(warmup, 2)):
             fn()
         n = max(steps, 5)
@@ -1051,6 +1052,7 @@ def main() -> int:
         extra["gdn_forward_with_tape"] = rnd(fw)
     if "sdpa" in legs:
         extra["sdpa_q16_kv4112"] = rnd(bench_sdpa(device, args.steps, args.warmup))
+        extra["sdpa_q16_kv32784"] = rnd(bench_sdpa(device, args.steps, args.warmup, N=32784, with_torch=False))
     if "glue" in legs:
         extra["gdn_layer_glue"] = {k: (round(v, 3) if isinstance(v, float) else v)
                                    for k, v in bench_gdn_glue(device, args.steps, args.warmup).items()}

@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdflash_mi355.so")
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 BF16, FP16, FP32 = 0, 1, 2
 QMM_MMA2BIG, QMM_MMA2BIG_PIPE = 0, 1
@@ -24,7 +24,7 @@ QMM_CHAIN_ERROR_OFFSET = QMM_ERROR_OFFSET      # DFLASH_QMM_CHAIN_ERROR_OFFSET
 QMM_EPILOGUE_NONE, QMM_EPILOGUE_SILU_MUL = 0, 1
 QMM_CHAIN_JOINT_SPLIT = 1                # DFLASH_QMM_CHAIN_JOINT_SPLIT
 QMM_LAYOUT_ROWS, QMM_LAYOUT_PACKED = 0, 1  # DFLASH_QMM_LAYOUT_*
-OPT_GDN_STEP_BY_STEP, OPT_SDPA_SPLITS, OPT_SDPA_STAGED, OPT_QMM_SPIN_LIMIT = 0, 1, 2, 3  # DFLASH_OPT_*
+OPT_GDN_STEP_BY_STEP, OPT_SDPA_SPLITS, OPT_QMM_SPIN_LIMIT = 0, 1, 2  # DFLASH_OPT_*
 
 
 class QmmProblem(ctypes.Structure):

@@ -275,337 +275,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   }
 }
 
-// ---------------------------------------------------------------------------------------------
-// The same first pass with the whole key range of the workgroup resident in LDS (no mask).
-//
-// The staged kernel above moves every tile global -> registers -> LDS and keeps two tiles in
-// flight; with five tiles per workgroup most of its time is the latency of that chain.  Here a
-// workgroup's range is at most 144 keys of 256 (288 of 128): K and V of the whole range fit
-// 144 KiB of LDS, so every wave asks for its share of ALL rows at once with direct-to-LDS loads
-// (16 bytes per lane, no registers, no LDS writes by the waves), and the tiles are worked on in
-// the order they land: one wait on the wave's own load counter and one barrier per tile.
-// Rows keep their 2 D bytes without padding (a load instruction fills 1 KiB of consecutive
-// LDS); bank conflicts are avoided by storing the 16-byte piece p of row r at position
-// p ^ ((r mod 16) << 1) - the load fetches the piece that belongs at its lane's position.
-// The K fragments and the transposed V reads are written out by hand: the compiler would put a
-// wait for every load in flight in front of any LDS read it can see.
-// What bounds a workgroup is not the stream but the chain LDS reads -> K Q^T -> softmax -> LDS
-// reads -> V^T P^T of a tile, which a wave runs through tile after tile (switching single
-// parts off changes little, all of it 6 us of 17).  So where a key/value head has fewer than
-// eight query heads, the CS waves of a query head do not split the output columns (and repeat
-// K Q^T) as in the staged kernel: they take every CS-th TILE each, all columns, and their
-// (max, sum, output) states are merged through LDS when the range is done - half (a quarter)
-// as many tiles in a row per wave, and half (a quarter) of the K reads.
-typedef __attribute__((address_space(1))) const void sdpa_global_cvoid_t;
-typedef __attribute__((address_space(3))) void sdpa_lds_void_t;
-
-template <int N>
-__device__ __forceinline__ void wait_loads_in_flight() {
-  static_assert(N >= 0 && N < 64, "vmcnt is six bits");
-  // (the builtin, not inline asm: the compiler then knows that older loads - the queries - have
-  // landed as well, and puts no wait of its own in front of their first use)
-  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);  // vmcnt(N), the other counters untouched
-}
-
-#ifdef DFLASH_SDPA_STAMPS
-// Experiment builds only: wall-clock stamps of waves 0 and 4 of every workgroup. [block][wave 0|4][event]
-__device__ unsigned long long g_sdpa_stamps[512][2][16];
-#define SDPA_STAMP(idx)                                                                          \
-  do {                                                                                           \
-    if (lane == 0 && (wave == 0 || wave == 4) && blockIdx.x < 512)                               \
-      g_sdpa_stamps[blockIdx.x][wave >> 2][idx] = wall_clock64();                                \
-  } while (0)
-#else
-#define SDPA_STAMP(idx) do {} while (0)
-#endif
-
-template <int D, bool FP16, int CS, int H>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_q16_resident_kernel(SdpaArgs a) {
-  constexpr int kCols = D / 16;                // 16-column chunks of the output: every wave holds all of them
-  constexpr int kRows = 16 * H;                // rows of K (and of V) held in LDS
-  constexpr int kRowBytes = D * 2;
-  constexpr int kSwz = D == 256 ? 15 : 7;      // rows that differ in these bits sit in different banks
-  constexpr int kLoadsPerHalf = D == 256 ? 2 : 1;  // load instructions per wave and 16 rows (K and V together)
-  constexpr int kTiles = (H + 1) / 2;
-  extern __shared__ __align__(16) uint16_t lds[];  // [K rows | V rows]
-  char* const lds_k = reinterpret_cast<char*>(lds);
-  char* const lds_v = lds_k + kRows * kRowBytes;
-  const uint32_t k_addr = (uint32_t)(uintptr_t)lds_k, v_addr = k_addr + kRows * kRowBytes;
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int split = blockIdx.x % a.splits;
-  const int bh = blockIdx.x / a.splits;
-  const int b = bh / a.Hk, hk = bh % a.Hk;
-  const int n_begin = split * a.keys_per_split;
-  const int n_end = n_begin + a.keys_per_split < a.N ? n_begin + a.keys_per_split : a.N;
-  const int j = lane & 15, kb = lane >> 4;
-  const bool computes = wave < a.G * CS;  // the other waves only move rows
-  const int part = computes ? wave / a.G : 0;  // this wave's tiles: t = part, part + CS, ...
-  const int hq = hk * a.G + (computes ? wave % a.G : 0);
-  const size_t qrow = ((size_t)b * a.Hq + hq) * 16 + j;  // this lane's query
-
-  const uint16_t* kbase = a.k + (size_t)b * a.k_batch_stride + (size_t)hk * a.k_head_stride;
-  const uint16_t* vbase = a.v + (size_t)b * a.v_batch_stride + (size_t)hk * a.v_head_stride;
-
-  SDPA_STAMP(0);
-  // this wave's queries, as the B operand of K Q^T (asked for first: loads return in order)
-  // (by every wave, also those that only move rows: behind a condition the compiler could not
-  // count the loads in flight and would wait for all of them at the first use)
-  uint4 qreg[D / 32];
-#pragma unroll
-  for (int s = 0; s < D / 32; ++s) qreg[s] = *reinterpret_cast<const uint4*>(a.q + qrow * D + 32 * s + 8 * kb);
-
-  // ---- the rows of the range, 16 at a time; rows past the end repeat the last key (masked).
-  // They are asked for a group of CS tiles ahead of the arithmetic: a compute unit keeps about
-  // 64 KiB of loads in flight, and a wave that asks for more sits in its issue stage until the
-  // first ones have landed - asked for all at once, no wave would reach the first barrier before
-  // nearly everything is there.
-  auto ask_for_rows = [&](int h) __attribute__((always_inline)) {
-    if constexpr (D == 256) {  // a load instruction moves two rows; wave w: rows 2w, 2w+1 of K, then of V
-      const int r0 = 16 * h + 2 * wave;
-      const int r = r0 + (lane >> 5);
-      const int piece = (lane & 31) ^ ((r & kSwz) << 1);
-      const int n = n_begin + r < n_end ? n_begin + r : n_end - 1;
-      __builtin_amdgcn_global_load_lds((sdpa_global_cvoid_t*)(kbase + (size_t)n * a.k_seq_stride + 8 * piece),
-                                       (sdpa_lds_void_t*)(lds_k + r0 * kRowBytes), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((sdpa_global_cvoid_t*)(vbase + (size_t)n * a.v_seq_stride + 8 * piece),
-                                       (sdpa_lds_void_t*)(lds_v + r0 * kRowBytes), 16, 0, 0);
-    } else {  // four rows per instruction; waves 0-3: rows 4w..4w+3 of K, waves 4-7 the same of V
-      const bool is_v = wave >= 4;
-      const int r0 = 16 * h + 4 * (wave & 3);
-      const int r = r0 + (lane >> 4);
-      const int piece = (lane & 15) ^ ((r & kSwz) << 1);
-      const int n = n_begin + r < n_end ? n_begin + r : n_end - 1;
-      const uint16_t* src = is_v ? vbase + (size_t)n * a.v_seq_stride : kbase + (size_t)n * a.k_seq_stride;
-      __builtin_amdgcn_global_load_lds((sdpa_global_cvoid_t*)(src + 8 * piece),
-                                       (sdpa_lds_void_t*)((is_v ? lds_v : lds_k) + r0 * kRowBytes), 16, 0, 0);
-    }
-  };
-  constexpr int kGroupHalves = 2 * CS;  // 16-row halves per group of CS tiles
-#pragma unroll
-  for (int h = 0; h < (kGroupHalves < H ? kGroupHalves : H); ++h) ask_for_rows(h);  // the first group
-
-  SDPA_STAMP(1);
-  f32x4_t O[kCols];
-#pragma unroll
-  for (int c = 0; c < kCols; ++c) O[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  float m_run = kMasked, l_run = 0.f;  // l_run: this lane's keys only, merged at the end
-
-  const int src = lane & 15;  // V: source lane inside the group of 16: key 4 kb + src / 4, columns 4 (src % 4) ..+3
-
-#pragma unroll
-  for (int t = 0; t < kTiles; ++t) {
-    // CS tiles at a time (one for each of a head's waves, which then work side by side): their
-    // rows have landed for this wave's loads, and after the barrier for everyone's
-    if (t % CS == 0) {
-      // the next group's rows are asked for, then this group's awaited: what may still be in
-      // flight afterwards are the loads just issued
-      constexpr int kNone = 0;
-      const int first = 2 * t + kGroupHalves, last = first + kGroupHalves < H ? first + kGroupHalves : H;
-      int asked = kNone;
-#pragma unroll
-      for (int h = 0; h < kGroupHalves; ++h) {
-        if (first + h < last) {
-          ask_for_rows(first + h);
-          ++asked;
-        }
-      }
-      // (t is a constant after unrolling; the switch picks the immediate)
-      switch (kLoadsPerHalf * asked) {
-        case 0: wait_loads_in_flight<0>(); break;
-        case 1: wait_loads_in_flight<1>(); break;
-        case 2: wait_loads_in_flight<2>(); break;
-        case 3: wait_loads_in_flight<3>(); break;
-        case 4: wait_loads_in_flight<4>(); break;
-        case 5: wait_loads_in_flight<5>(); break;
-        case 6: wait_loads_in_flight<6>(); break;
-        case 7: wait_loads_in_flight<7>(); break;
-        case 8: wait_loads_in_flight<8>(); break;
-        case 9: wait_loads_in_flight<9>(); break;
-        case 10: wait_loads_in_flight<10>(); break;
-        case 11: wait_loads_in_flight<11>(); break;
-        case 12: wait_loads_in_flight<12>(); break;
-        case 13: wait_loads_in_flight<13>(); break;
-        case 14: wait_loads_in_flight<14>(); break;
-        case 15: wait_loads_in_flight<15>(); break;
-        default: wait_loads_in_flight<16>(); break;
-      }
-      asm volatile("s_barrier" ::: "memory");
-    }
-    SDPA_STAMP(2 + t);
-    const int n0 = n_begin + 32 * t;
-    if (!computes || n0 >= n_end || t % CS != part) continue;
-
-    // S^T = K Q^T for the two 16-key halves of the tile: all fragments asked for, then one wait
-    typedef __attribute__((ext_vector_type(4))) unsigned int frag_t;  // (a native vector: asm operands)
-    frag_t kf[2][D / 32];
-#pragma unroll
-    for (int hh = 0; hh < 2; ++hh) {
-      int r = 32 * t + 16 * hh + j;
-      r = r < kRows ? r : kRows - 1;  // (an odd last half: its keys are past the end anyway)
-      const uint32_t row_addr = k_addr + r * kRowBytes;
-      const int x = (r & kSwz) << 1;
-#pragma unroll
-      for (int s = 0; s < D / 32; ++s) {
-        const uint32_t addr = row_addr + (((4 * s + kb) ^ x) << 4);
-        asm volatile("ds_read_b128 %0, %1" : "=v"(kf[hh][s]) : "v"(addr) : "memory");
-      }
-    }
-    // one wait, naming every fragment so that nothing that uses one can be placed before it
-    if constexpr (D == 256) {
-      asm volatile("s_waitcnt lgkmcnt(0)"
-                   : "+v"(kf[0][0]), "+v"(kf[0][1]), "+v"(kf[0][2]), "+v"(kf[0][3]), "+v"(kf[0][D / 32 - 4]),
-                     "+v"(kf[0][D / 32 - 3]), "+v"(kf[0][D / 32 - 2]), "+v"(kf[0][D / 32 - 1])
-                   :
-                   : "memory");
-      asm volatile(""
-                   : "+v"(kf[1][0]), "+v"(kf[1][1]), "+v"(kf[1][2]), "+v"(kf[1][3]), "+v"(kf[1][D / 32 - 4]),
-                     "+v"(kf[1][D / 32 - 3]), "+v"(kf[1][D / 32 - 2]), "+v"(kf[1][D / 32 - 1])
-                   :
-                   : "memory");
-    } else {
-      asm volatile("s_waitcnt lgkmcnt(0)"
-                   : "+v"(kf[0][0]), "+v"(kf[0][1]), "+v"(kf[0][2]), "+v"(kf[0][3]), "+v"(kf[1][0]), "+v"(kf[1][1]),
-                     "+v"(kf[1][2]), "+v"(kf[1][3])
-                   :
-                   : "memory");
-    }
-    f32x4_t st[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
-#pragma unroll
-    for (int s = 0; s < D / 32; ++s)
-#pragma unroll
-      for (int hh = 0; hh < 2; ++hh) st[hh] = mfma32<FP16>(__builtin_bit_cast(uint4, kf[hh][s]), qreg[s], st[hh]);
-
-    // V fragments of the tile, asked for before the softmax arithmetic, waited for after it
-    s16x4_t lo[kCols], hi[kCols];
-    {
-      int r_lo = 32 * t + 4 * kb + (src >> 2), r_hi = r_lo + 16;
-      r_hi = r_hi < kRows ? r_hi : kRows - 1;
-      const uint32_t lo_addr = v_addr + r_lo * kRowBytes + 8 * (src & 1);
-      const uint32_t hi_addr = v_addr + r_hi * kRowBytes + 8 * (src & 1);
-      const int x_lo = (r_lo & kSwz) << 1, x_hi = (r_hi & kSwz) << 1;
-#pragma unroll
-      for (int c = 0; c < kCols; ++c) {
-        const int piece = 2 * c + ((src & 3) >> 1);
-        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo[c]) : "v"(lo_addr + ((piece ^ x_lo) << 4)) : "memory");
-        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(hi[c]) : "v"(hi_addr + ((piece ^ x_hi) << 4)) : "memory");
-      }
-    }
-
-    // scores of query j for keys n0 + 16 hh + 4 kb + r
-    float x[8];
-    bool use[8];
-    float m_tile = kMasked;
-#pragma unroll
-    for (int hh = 0; hh < 2; ++hh) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int n = n0 + 16 * hh + 4 * kb + r;
-        const bool ok = n < n_end && n <= a.N - 16 + j;
-        use[4 * hh + r] = ok;
-        x[4 * hh + r] = ok ? st[hh][r] * a.scale : kMasked;
-        m_tile = fmaxf(m_tile, x[4 * hh + r]);
-      }
-    }
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
-    const float m_new = fmaxf(m_run, m_tile);
-    const float factor = __expf(m_run - m_new);  // 1 while nothing has been seen (both masked)
-    float pe[8], sum = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      pe[e] = use[e] ? __expf(x[e] - m_new) : 0.f;
-      sum += pe[e];
-    }
-    l_run = l_run * factor + sum;
-    m_run = m_new;
-    if (__any(factor != 1.f)) {
-#pragma unroll
-      for (int c = 0; c < kCols; ++c) O[c] *= factor;
-    }
-    const uint4 pb = {pack2<FP16>(pe[0], pe[1]), pack2<FP16>(pe[2], pe[3]), pack2<FP16>(pe[4], pe[5]),
-                      pack2<FP16>(pe[6], pe[7])};
-    // O^T += V^T P^T, 16 columns of V at a time
-    static_assert(kCols == 2 || kCols == 4 || kCols == 8 || kCols == 16, "column chunks per wave");
-#pragma unroll
-    for (int c0 = 0; c0 < kCols; c0 += 2) {
-      if (c0 == 0)
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[c0]), "+v"(hi[c0]), "+v"(lo[c0 + 1]), "+v"(hi[c0 + 1]) : : "memory");
-      else
-        asm volatile("" : "+v"(lo[c0]), "+v"(hi[c0]), "+v"(lo[c0 + 1]), "+v"(hi[c0 + 1]) : : "memory");
-    }
-#pragma unroll
-    for (int c = 0; c < kCols; ++c) {
-      const uint2 lo2 = __builtin_bit_cast(uint2, lo[c]), hi2 = __builtin_bit_cast(uint2, hi[c]);
-      O[c] = mfma32<FP16>(uint4{lo2.x, lo2.y, hi2.x, hi2.y}, pb, O[c]);
-    }
-  }
-  wait_loads_in_flight<0>();  // (a range shorter than the rows asked for: nothing may be left in flight)
-  SDPA_STAMP(12);
-
-  // ---- the CS waves of a query head merge their states: the later parts hand theirs to part 0
-  // through LDS (the rows of K and V are done with after the barrier), value index major so that
-  // the 64 lanes of a wave touch 64 consecutive words ------------------------------------------
-  if constexpr (CS > 1) {
-    constexpr int kStateFloats = 4 * kCols + 2;  // O, max, sum per lane
-    // at most six waves hand over a state (G (CS - 1) with G CS <= 8); the launch sizes LDS for them
-    float* const state = reinterpret_cast<float*>(lds);
-    asm volatile("s_barrier" ::: "memory");
-    if (computes && part > 0) {
-      float* mine = state + (size_t)(wave - a.G) * kStateFloats * 64 + lane;
-#pragma unroll
-      for (int c = 0; c < kCols; ++c)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) mine[(4 * c + r) * 64] = O[c][r];
-      mine[(4 * kCols) * 64] = m_run;
-      mine[(4 * kCols + 1) * 64] = l_run;
-    }
-    __syncthreads();
-    if (computes && part == 0) {
-      for (int other = 1; other < CS; ++other) {
-        const float* theirs = state + (size_t)((other - 1) * a.G + wave) * kStateFloats * 64 + lane;
-        const float m_other = theirs[(4 * kCols) * 64], l_other = theirs[(4 * kCols + 1) * 64];
-        const float m_new = fmaxf(m_run, m_other);
-        const float f_mine = __expf(m_run - m_new), f_other = __expf(m_other - m_new);  // 0 for a part without keys
-        l_run = l_run * f_mine + l_other * f_other;
-        m_run = m_new;
-#pragma unroll
-        for (int c = 0; c < kCols; ++c)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) O[c][r] = O[c][r] * f_mine + theirs[(4 * c + r) * 64] * f_other;
-      }
-    }
-    if (part > 0) return;
-  }
-
-  SDPA_STAMP(13);
-  if (!computes) return;
-  l_run += __shfl_xor(l_run, 16, 64);
-  l_run += __shfl_xor(l_run, 32, 64);
-  // accumulator r of chunk c is column 16 c + 4 kb + r of query j
-  const int col0 = 4 * kb;
-  if (a.splits == 1) {
-    const float inv = l_run > 0.f ? 1.f / l_run : 1.f;
-#pragma unroll
-    for (int c = 0; c < kCols; ++c) {
-      const uint2 o = {pack2<FP16>(O[c][0] * inv, O[c][1] * inv), pack2<FP16>(O[c][2] * inv, O[c][3] * inv)};
-      *reinterpret_cast<uint2*>(a.out + qrow * D + col0 + 16 * c) = o;
-    }
-  } else {
-    const size_t prow = (size_t)split * a.B * a.Hq * 16 + qrow;
-#pragma unroll
-    for (int c = 0; c < kCols; ++c)
-      *reinterpret_cast<uint2*>(a.part_o + prow * D + col0 + 16 * c) =
-          uint2{pack2<FP16>(O[c][0], O[c][1]), pack2<FP16>(O[c][2], O[c][3])};
-    if (kb == 0) *reinterpret_cast<f32x2_t*>(a.part_ml + prow * 2) = f32x2_t{m_run, l_run};
-  }
-#ifdef DFLASH_SDPA_STAMPS
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  SDPA_STAMP(14);
-#endif
-}
-
 // Second pass: one workgroup of 256 threads per query row.  Thread (g, c) adds the partial
 // outputs of the splits s = g, g + 4, ... for 4 output columns; the weights exp(m_s - m) and the
 // total sum are worked out once, by the first wave.
@@ -700,41 +369,14 @@ int pick_splits(int B, int Hk, int N, int* keys_per_split) {
   return (N + per - 1) / per;  // no empty split
 }
 
-
-// The resident kernel: about one workgroup per compute unit, ranges a multiple of 16 keys and
-// at most what 144 KiB of LDS hold of K and V (144 keys of 256, 288 of 128).
-constexpr int resident_max_keys(int D) { return D == 256 ? 144 : 288; }
-int pick_resident_splits(int B, int Hk, int N, int D, int* keys_per_split) {
-  const int forced = option(DFLASH_OPT_SDPA_SPLITS);
-  int want = forced > 0 ? forced : (256 + B * Hk - 1) / (B * Hk);
-  if (want < 1) want = 1;
-  int per = ((N + want - 1) / want + 15) / 16 * 16;
-  if (per > resident_max_keys(D)) per = resident_max_keys(D);
-  *keys_per_split = per;
-  return (N + per - 1) / per;  // no empty split
-}
-bool resident_applies(const void* mask, int splits) {
-  return mask == nullptr && option(DFLASH_OPT_SDPA_STAGED) == 0 && splits <= kMaxSplits;
-}
 }  // namespace
 }  // namespace dflash
-
-#ifdef DFLASH_SDPA_STAMPS
-extern "C" int dflash_debug_read_sdpa_stamps(unsigned long long* out_host) {
-  return (int)hipMemcpyFromSymbol(out_host, HIP_SYMBOL(dflash::g_sdpa_stamps), sizeof(dflash::g_sdpa_stamps));
-}
-#endif
 
 extern "C" size_t dflash_sdpa_q16_workspace_bytes(int B, int Hq, int Hk, int N, int D) {
   using namespace dflash;
   if (B <= 0 || Hq <= 0 || Hk <= 0 || N <= 0 || D <= 0) return 0;
-  // enough for either kernel: which one runs depends on the mask and on the options of the moment
   int per = 0;
-  int splits = pick_splits(B, Hk, N, &per);
-  if (D == 128 || D == 256) {
-    const int resident = pick_resident_splits(B, Hk, N, D, &per);
-    if (resident <= kMaxSplits && resident > splits) splits = resident;
-  }
+  const int splits = pick_splits(B, Hk, N, &per);
   if (splits == 1) return 0;
   return (size_t)splits * B * Hq * 16 * (D * sizeof(uint16_t) + 2 * sizeof(float));
 }
@@ -768,16 +410,6 @@ extern "C" int dflash_sdpa_q16(const void* q, const void* k, const void* v, cons
   a.v_batch_stride = v_batch_stride; a.v_head_stride = v_head_stride; a.v_seq_stride = v_seq_stride;
   a.B = B; a.Hq = Hq; a.Hk = Hk; a.N = N; a.G = Hq / Hk;
   a.splits = pick_splits(B, Hk, N, &a.keys_per_split);
-  bool resident = false;
-  {
-    int per = 0;
-    const int splits = pick_resident_splits(B, Hk, N, D, &per);
-    if (resident_applies(mask, splits)) {
-      resident = true;
-      a.splits = splits;
-      a.keys_per_split = per;
-    }
-  }
   a.scale = scale;
   a.lowest = dtype == DFLASH_FP16 ? -65504.0f : -3.3895313892515355e38f;
   a.part_o = nullptr;
@@ -809,31 +441,7 @@ extern "C" int dflash_sdpa_q16(const void* q, const void* k, const void* v, cons
   const int ics = cs == 1 ? 0 : cs == 2 ? 1 : 2;
   void* args[] = {&a};
   const int slot = current_device_slot();
-  if (resident) {
-    // rows held in LDS: the smaller instantiation where the range fits it
-    const int small_h = D == 256 ? 5 : 9, large_h = D == 256 ? 9 : 18;
-    const bool small = a.keys_per_split <= 16 * small_h;
-    const size_t rows = (size_t)16 * (small ? small_h : large_h);
-    const size_t state_bytes = (size_t)6 * (4 * (D / 16) + 2) * 64 * sizeof(float);  // merge of a head's waves
-    const size_t rows_bytes = 2 * rows * D * sizeof(uint16_t);
-    const size_t resident_lds = rows_bytes > state_bytes ? rows_bytes : state_bytes;
-#define DFLASH_SDPA_RES(D_, F_, H_)                                                                 \
-  {(const void*)sdpa_q16_resident_kernel<D_, F_, 1, H_>, (const void*)sdpa_q16_resident_kernel<D_, F_, 2, H_>, \
-   (const void*)sdpa_q16_resident_kernel<D_, F_, 4, H_>}
-    const void* rtable[2][2][2][3] = {{{DFLASH_SDPA_RES(128, false, 9), DFLASH_SDPA_RES(128, false, 18)},
-                                       {DFLASH_SDPA_RES(128, true, 9), DFLASH_SDPA_RES(128, true, 18)}},
-                                      {{DFLASH_SDPA_RES(256, false, 5), DFLASH_SDPA_RES(256, false, 9)},
-                                       {DFLASH_SDPA_RES(256, true, 5), DFLASH_SDPA_RES(256, true, 9)}}};
-#undef DFLASH_SDPA_RES
-    const void* rfn = rtable[D == 256][f16][small ? 0 : 1][ics];
-    static bool rattr_set[kMaxDevices][24] = {};
-    const int ridx = (((D == 256) * 2 + f16) * 2 + (small ? 0 : 1)) * 3 + ics;
-    if (!rattr_set[slot][ridx] || slot == kMaxDevices - 1) {
-      DFLASH_HIP_OK(hipFuncSetAttribute(rfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)resident_lds));
-      rattr_set[slot][ridx] = true;
-    }
-    DFLASH_HIP_OK(hipLaunchKernel(rfn, dim3((unsigned)(B * Hk * a.splits)), dim3(kThreads), args, resident_lds, s));
-  } else {
+  {
     const void* fn = table[D == 256][f16][masked][ics];
     // the attribute belongs to the device's copy of the kernel: once per device and kernel
     static bool attr_set[kMaxDevices][24] = {};

@@ -31,8 +31,6 @@ CSRC = os.path.join(HERE, "csrc")
 KERNELS = (
     ("qmm_m16_stream.hip", "_ZN6dflash6stream17qmm_stream_kernel", 16, 40),  # activation x scale dtype x chunk x dense|gathered
     ("qmm_m16_chain.hip", "_ZN6dflash6stream16qmm_chain_kernel", 8, 40),     # activation x scale dtype x weight layout
-    # head dim x dtype x column split x rows held: hand-written K and transposed V reads
-    ("sdpa_q16.hip", "_ZN6dflash12_GLOBAL__N_124sdpa_q16_resident_kernel", 24, 60),
 )
 # source, number of counter bumps (arrival counters; the chained kernel's per-problem and exit counters too)
 ARRIVALS = (("qmm_m16.hip", 24), ("qmm_m16_stream.hip", 0), ("qmm_m16_chain.hip", 64))

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define DFLASH_ABI_VERSION 17
+#define DFLASH_ABI_VERSION 18
 
 enum {
   DFLASH_OK = 0,
@@ -61,8 +61,6 @@ const char* dflash_last_error(void);
  *                                where the block kernel would apply
  *   DFLASH_OPT_SDPA_SPLITS       n > 0: dflash_sdpa_q16 (and its workspace size) cut the keys into
  *                                n ranges (fewer if a range would fall below one tile)
- *   DFLASH_OPT_SDPA_STAGED       1: dflash_sdpa_q16 without a mask keeps the kernel that stages its
- *                                tiles through registers (the one a mask always takes)
  *   DFLASH_OPT_QMM_SPIN_LIMIT    n > 0: the streaming qmm kernel's workgroups that add partial tiles
  *                                give up after n polls instead of 2^22 (tests of that path: the
  *                                launch ends, the error word is set, results are unspecified)
@@ -72,9 +70,8 @@ const char* dflash_last_error(void);
 enum {
   DFLASH_OPT_GDN_STEP_BY_STEP = 0,
   DFLASH_OPT_SDPA_SPLITS = 1,
-  DFLASH_OPT_SDPA_STAGED = 2,
-  DFLASH_OPT_QMM_SPIN_LIMIT = 3,
-  DFLASH_OPT_COUNT = 4
+  DFLASH_OPT_QMM_SPIN_LIMIT = 2,
+  DFLASH_OPT_COUNT = 3
 };
 int dflash_set_option(int option, int value);
 int dflash_get_option(int option);

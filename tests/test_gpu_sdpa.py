@@ -36,21 +36,12 @@ def _dev(t, name):
     return torch.from_numpy(t).to(TORCH[name]).to(DEV)
 
 
-@pytest.fixture(params=["resident", "staged"])
-def kernel(request, native_lib):
-    """Without a mask two kernels serve the call: the one that keeps its whole key range in LDS
-    (default) and the one that stages tiles through registers (which a mask always takes)."""
-    assert native_lib.dflash_set_option(nat.OPT_SDPA_STAGED, 1 if request.param == "staged" else 0) == 0
-    yield request.param
-    native_lib.dflash_set_option(nat.OPT_SDPA_STAGED, 0)
-
-
 @pytest.mark.parametrize("name", ["bf16", "fp16"])
 @pytest.mark.parametrize("B,Hq,Hk,N,D", [(1, 4, 1, 300, 128), (2, 8, 2, 1000, 256), (1, 2, 2, 16, 128),
                                          (1, 6, 1, 17, 256), (1, 8, 1, 33, 128), (1, 16, 4, 1025, 256),
                                          (1, 3, 1, 4000, 128), (1, 32, 8, 4112, 256), (1, 5, 1, 289, 128),
                                          (1, 8, 8, 145, 256), (3, 7, 7, 81, 256)])
-def test_against_the_oracle(native_lib, kernel, name, B, Hq, Hk, N, D):
+def test_against_the_oracle(native_lib, name, B, Hq, Hk, N, D):
     q, k, v = _case(B, Hq, Hk, N, D, N + D, name)
     out = batched_sdpa_2pass_exact(_dev(q, name), _dev(k, name), _dev(v, name), D ** -0.5)
     torch.cuda.synchronize()
@@ -60,7 +51,7 @@ def test_against_the_oracle(native_lib, kernel, name, B, Hq, Hk, N, D):
 
 @pytest.mark.parametrize("D,N", [(128, 700), (256, 500)])
 @pytest.mark.parametrize("splits", [1, 2, 5, 64])
-def test_any_number_of_key_ranges_gives_the_same_attention(native_lib, kernel, splits, D, N):
+def test_any_number_of_key_ranges_gives_the_same_attention(native_lib, splits, D, N):
     q, k, v = _case(1, 4, 2, N, D, 77, "bf16")
     assert native_lib.dflash_set_option(nat.OPT_SDPA_SPLITS, splits) == 0
     try:
