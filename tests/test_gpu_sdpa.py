@@ -40,7 +40,8 @@ def _dev(t, name):
 @pytest.mark.parametrize("B,Hq,Hk,N,D", [(1, 4, 1, 300, 128), (2, 8, 2, 1000, 256), (1, 2, 2, 16, 128),
                                          (1, 6, 1, 17, 256), (1, 8, 1, 33, 128), (1, 16, 4, 1025, 256),
                                          (1, 3, 1, 4000, 128), (1, 32, 8, 4112, 256), (1, 5, 1, 289, 128),
-                                         (1, 8, 8, 145, 256), (3, 7, 7, 81, 256)])
+                                         (1, 8, 8, 145, 256), (3, 7, 7, 81, 256),
+                                         (1, 8, 2, 33000, 128), (1, 4, 1, 70001, 256)])  # long caches: dozens of tiles per key range
 def test_against_the_oracle(native_lib, name, B, Hq, Hk, N, D):
     q, k, v = _case(B, Hq, Hk, N, D, N + D, name)
     out = batched_sdpa_2pass_exact(_dev(q, name), _dev(k, name), _dev(v, name), D ** -0.5)
