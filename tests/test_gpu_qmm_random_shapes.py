@@ -84,3 +84,71 @@ def test_joint_split_on_random_lists_of_problems(verify_env, native_lib, c_oracl
         for c, a, b in zip(cases, first, second):
             assert torch.equal(a, b), shapes
             _close(a, _exact(c_oracle, c))
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_packed_weights_on_random_shapes(verify_env, native_lib, seed):
+    """The packed copy of a triple gives the bits of the row-major route, alone and in a chain
+    with the joint split (K a multiple of 1024: whole scale/bias chunks; N of 32)."""
+    verify_env.setenv("DFLASH_QMM_KERNEL", "stream")
+    rng = np.random.default_rng(seed)
+    cases, images = [], []
+    for i in range(12):
+        K = 1024 * int(rng.integers(1, 18))
+        N = 32 * int(rng.integers(1, 350))
+        case = make_qmm_case(K, N, 1000 * seed + i).to(DEV)
+        image = VQ.pack_weights(case.w, case.scales, case.biases)
+        want = VQ.verify_matmul(case.x, case.w, case.scales, case.biases, group_size=64, bits=4)
+        assert torch.equal(VQ.verify_matmul_packed(case.x, image), want), (K, N)
+        cases.append(case)
+        images.append(image)
+    separate = [VQ.verify_matmul(c.x, c.w, c.scales, c.biases, group_size=64, bits=4) for c in cases]
+    chain = VQ.QmmChain([VQ.ChainProblem(c.x, im) for c, im in zip(cases, images)])
+    for y, want in zip(chain(), separate):  # per-problem split: bit for bit the separate launches
+        assert torch.equal(y, want)
+    joint = VQ.QmmChain([VQ.ChainProblem(c.x, im) for c, im in zip(cases, images)], joint_split=True)
+    first = [y.clone() for y in joint()]
+    second = [y.clone() for y in joint()]
+    torch.cuda.synchronize()
+    for a, b, want in zip(first, second, separate):  # another split: within an output rounding, repeatable
+        assert torch.equal(a, b)
+        assert float((a == want).float().mean()) >= 0.97
+        assert float((a.float() - want.float()).abs().max()) <= 2 ** -7 * float(want.float().abs().max())
+    assert joint.error_word() == 0 and int((joint._ws != 0).sum()) == 0
+    _workspace_is_clean(torch.device(DEV))
+
+
+@pytest.mark.parametrize("seed", [41, 42, 43])
+def test_gathered_experts_on_random_routings(native_lib, monkeypatch, seed):
+    """Expert counts, rows per expert (none, one, more than sixteen) and shapes at random: every row
+    is the product with its own expert whatever else shares the launch, twice the same bits."""
+    from dflash_mlx_amd.verify_qmm import gather_qmm
+    from dflash_mlx_amd.workloads import make_moe_case
+    from oracle import dflash_oracle as O
+
+    monkeypatch.setenv("DFLASH_QMM_KERNEL", "auto")
+    rng = np.random.default_rng(seed)
+    for i in range(6):
+        K = 512 * int(rng.integers(1, 9))
+        N = 16 * int(rng.integers(1, 80))
+        E = int(rng.integers(1, 40))
+        P = int(rng.integers(1, 257))
+        case = make_moe_case(K, N, 100 * seed + i, experts=E, tokens=P, top_k=1)
+        # a skewed routing: most rows on a few experts, some experts without rows
+        weights = rng.random(E) ** 4
+        ids = rng.choice(E, size=P, p=weights / weights.sum()).astype(np.int32)
+        case.expert_ids = torch.from_numpy(ids)
+        d = case.to(DEV)
+        y = gather_qmm(d.x, d.w, d.scales, d.biases, d.expert_ids, group_size=64)
+        assert torch.equal(y, gather_qmm(d.x, d.w, d.scales, d.biases, d.expert_ids, group_size=64)), (K, N, E, P)
+        exact = O.qmm_gather_exact(case.x.float().numpy(), ids, case.w.numpy().view(np.uint32),
+                                   case.scales.float().numpy(), case.biases.float().numpy(), 64)
+        _close(y, exact)
+        j = int(rng.integers(0, P))
+        # (alone in a call the row's K range is cut at other places - the cut follows the number
+        # of units of the whole launch - so its fp32 sums associate differently: the same value
+        # to within an output rounding, not always the same bits)
+        one = gather_qmm(d.x[j:j + 1], d.w, d.scales, d.biases, d.expert_ids[j:j + 1], group_size=64)
+        assert float((one[0] == y[j]).float().mean()) >= 0.97, (K, N, E, P, j)
+        assert float((one[0].float() - y[j].float()).abs().max()) <= 2 ** -7 * float(y[j].float().abs().max())
+    VQ.raise_on_device_errors(torch.device(DEV))
