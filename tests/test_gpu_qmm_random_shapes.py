@@ -1,12 +1,16 @@
-"""Shapes drawn at random through the streaming M=16 qmm and the chained kernel's joint split.
+"""Shapes drawn at random through the M=16 qmm kernels.
 
 The split of a launch (how many workgroups, which row blocks two of them share, who adds the
 partial tiles) follows from K and N, so the shapes of the stacks exercise a handful of splits;
-these draws exercise the rest: K any multiple of 512 up to 18 432, N any multiple of 16 up to
-20 800, both activation types, a new shape after every launch and earlier ones again without a
-wait in between.  Every result is checked against the oracle's C restatement of the reference
-arithmetic (north-star bar of tests/test_gpu_qmm.py) and must repeat bit for bit; afterwards the
-error word is clear and the partial-tile workspace is back at zero.
+these draws exercise the rest: the streaming kernel on K any multiple of 512 up to 18 432 and N
+any multiple of 16 up to 20 800, both activation types, a new shape after every launch and
+earlier ones again without a wait in between; the chained kernel's joint split on random lists
+of problems; packed weights alone, chained and in a joint split; chains whose links wait for
+each other, with and without the MLP epilogue; gathered experts on skewed routings.  Results
+are checked against the oracle's C restatement of the reference arithmetic (north-star bar of
+tests/test_gpu_qmm.py) or, where a route is stated to give another route's bits, against that
+route; they must repeat bit for bit; afterwards the error word is clear and the partial-tile
+workspace is back at zero.
 """
 import numpy as np
 import pytest
@@ -152,3 +156,58 @@ def test_gathered_experts_on_random_routings(native_lib, monkeypatch, seed):
         assert float((one[0] == y[j]).float().mean()) >= 0.97, (K, N, E, P, j)
         assert float((one[0].float() - y[j].float()).abs().max()) <= 2 ** -7 * float(y[j].float().abs().max())
     VQ.raise_on_device_errors(torch.device(DEV))
+
+
+@pytest.mark.parametrize("seed", [51, 52, 53])
+def test_dependent_chains_of_random_widths(verify_env, native_lib, seed):
+    """y0 = A0 x, y1 = A1 y0, ...: widths at random, every link waiting inside the launch for the one
+    before it, now and then an MLP (gate/up with the silu-mul epilogue, then its down projection).
+    Every link gives the bits of a separate launch on the input the chain actually stored."""
+    from dflash_mlx_amd.gdn_layer import silu_ops
+
+    verify_env.setenv("DFLASH_QMM_KERNEL", "stream")
+    rng = np.random.default_rng(seed)
+    for it in range(4):
+        width = 1024 * int(rng.integers(1, 7))
+        x = make_qmm_case(width, 16, 7000 + 10 * seed + it).to(DEV).x
+        problems, links, prev = [], [], x
+        for i in range(int(rng.integers(2, 7))):
+            nxt = 1024 * int(rng.integers(1, 7))
+            if rng.random() < 0.3:  # an MLP of inner width `inner` in the place of a plain link
+                inner = 1024 * int(rng.integers(1, 9))
+                gate_up = make_qmm_case(width, 2 * inner, 100 * seed + 10 * it + i).to(DEV)
+                down = make_qmm_case(inner, nxt, 100 * seed + 10 * it + i + 5000).to(DEV)
+                for c in (gate_up, down):
+                    c.scales.mul_(0.05); c.biases.mul_(0.05)
+                p0 = VQ.ChainProblem(prev, gate_up.w, gate_up.scales, gate_up.biases, epilogue="silu_mul")
+                p1 = VQ.ChainProblem(p0, down.w, down.scales, down.biases)
+                problems += [p0, p1]
+                links += [("mlp", gate_up), ("plain", down)]
+                prev = p1
+            else:
+                c = make_qmm_case(width, nxt, 100 * seed + 10 * it + i).to(DEV)
+                c.scales.mul_(0.05); c.biases.mul_(0.05)
+                pr = VQ.ChainProblem(prev, c.w, c.scales, c.biases)
+                problems.append(pr)
+                links.append(("plain", c))
+                prev = pr
+            width = nxt
+        chain = VQ.QmmChain(problems)
+        for rep in range(2):
+            for y in chain.outputs:
+                y.fill_(float("nan"))
+            ys = chain()
+            torch.cuda.synchronize()
+            assert chain.error_word() == 0
+            inp = x
+            for i, ((kind, c), y) in enumerate(zip(links, ys)):
+                assert torch.isfinite(y.float()).all(), (it, i)
+                full = VQ.verify_matmul(inp, c.w, c.scales, c.biases, group_size=64, bits=4)
+                if kind == "plain":
+                    assert torch.equal(y, full), (it, rep, i, kind)
+                else:  # (the joined pair splits K like one matrix of its own: same split here and there)
+                    half = c.N // 2
+                    want = silu_ops(full[:, :half]) * full[:, half:]
+                    assert torch.equal(y, want), (it, rep, i, kind)
+                inp = y
+    _workspace_is_clean(torch.device(DEV))
